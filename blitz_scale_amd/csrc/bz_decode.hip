@@ -1,0 +1,359 @@
+// Paged-KV batch decode attention for gfx950: host-side plan (split-K segmentation), the
+// general VALU kernel (any layout / dtype / RoPE mode) and the split-K combine.
+// Replaces src/kernel/attention_decode.cu and the decode half of flashinfer_types.cu of the
+// BlitzScale worker.
+#include <cmath>
+#include <algorithm>
+#include <vector>
+#include <new>
+
+#include "bz_common.hpp"
+#include "bz_decode_plan.hpp"
+
+namespace bz {
+
+// ------------------------------------------------------------------------------------------
+// General kernel.  One workgroup of 256 lanes per (segment, kv head).  A row of D elements is
+// covered by D/8 lanes holding 8 elements each, so the workgroup walks TOK = 256/(D/8) tokens
+// per pass; every token slot keeps its own online-softmax state (m, l, acc) for the G query
+// heads that share the kv head, and the slots are merged once at the end.
+// ------------------------------------------------------------------------------------------
+template <typename KVT, int D> struct RowGeom {
+    static constexpr int kLanes = D / 8;          // lanes per row
+    static constexpr int kTok = 256 / kLanes;     // token slots per workgroup
+    static constexpr int kTokPerWave = 64 / kLanes;
+};
+
+struct DecodeArgs {
+    const void* q;
+    void* out;
+    float* lse;
+    const char* k_data;
+    const char* v_data;
+    const int32_t* indices;
+    const int32_t* indptr;
+    const int32_t* last_page_len;
+    const DecodeSegment* segments;
+    float* part_o;   // [num_partials][Hq][D]
+    float* part_lse; // [num_partials][Hq]
+    const float* k_scale;
+    const float* v_scale;
+    uint64_t stride_page, stride_n, stride_h;
+    uint32_t page_size, num_qo_heads, num_kv_heads;
+    int rope_mode;
+    float sm_scale_log2; // sm_scale * log2(e)
+    RopeFreqs freqs;
+};
+
+template <typename QT, typename KVT, typename OT, int D, int G>
+__global__ __launch_bounds__(256) void decode_general_kernel(DecodeArgs a) {
+    using Geo = RowGeom<KVT, D>;
+    constexpr int LANES = Geo::kLanes;
+    constexpr int TOK = Geo::kTok;
+    constexpr int UNROLL = 4;
+
+    const DecodeSegment seg = a.segments[blockIdx.x];
+    const int kvh = blockIdx.y;
+    const int b = seg.seq;
+    const int tid = threadIdx.x;
+    const int lane_in_row = tid % LANES; // which 8-element slice of the row
+    const int slot = tid / LANES;        // token slot 0..TOK-1
+
+    const int ip0 = a.indptr[b];
+    const int npages = a.indptr[b + 1] - ip0;
+    const int seq_len = (npages - 1) * (int)a.page_size + a.last_page_len[b];
+    const int tok_begin = seg.page_begin * (int)a.page_size;
+    const int tok_end = min(seg.page_end * (int)a.page_size, seq_len);
+
+    // ---- q for the G heads of this kv head, as fp32, pre-rotated if asked ----
+    float q[G][8];
+#pragma unroll
+    for (int g = 0; g < G; ++g) {
+        const size_t qoff = ((size_t)b * a.num_qo_heads + (size_t)kvh * G + g) * D + lane_in_row * 8;
+        Vec8<QT> qv;
+        qv.load(reinterpret_cast<const QT*>(a.q) + qoff);
+        qv.to_float(q[g]);
+    }
+    if (a.rope_mode != BZ_ROPE_NONE) {
+        // partner slice holds the other half of each rotate-half pair
+        const bool upper = lane_in_row >= LANES / 2;
+        const float pos = (float)(seq_len - 1);
+#pragma unroll
+        for (int g = 0; g < G; ++g) {
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                const float other = __shfl_xor(q[g][e], LANES / 2, 64);
+                const int fi = (lane_in_row % (LANES / 2)) * 8 + e;
+                float s, c;
+                sincosf(pos * a.freqs.f[fi], &s, &c);
+                q[g][e] = upper ? (q[g][e] * c + other * s) : (q[g][e] * c - other * s);
+            }
+        }
+    }
+    const float kscale = (a.k_scale ? a.k_scale[kvh] : 1.0f) * a.sm_scale_log2;
+
+    float m[G], l[G], acc[G][8];
+#pragma unroll
+    for (int g = 0; g < G; ++g) {
+        m[g] = -INFINITY;
+        l[g] = 0.f;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) acc[g][e] = 0.f;
+    }
+
+    const size_t esz = sizeof(KVT);
+    const size_t head_off = ((size_t)kvh * a.stride_h + (size_t)lane_in_row * 8) * esz;
+
+    for (int base = tok_begin; base < tok_end; base += TOK * UNROLL) {
+        Vec8<KVT> kv[UNROLL], vv[UNROLL];
+        bool valid[UNROLL];
+        int jj[UNROLL];
+#pragma unroll
+        for (int u = 0; u < UNROLL; ++u) {
+            const int j = base + u * TOK + slot;
+            jj[u] = j;
+            valid[u] = j < tok_end;
+            const int jc = valid[u] ? j : tok_begin; // any in-range token: keeps the load legal
+            const int64_t page = a.indices[ip0 + jc / (int)a.page_size];
+            const size_t off =
+                ((size_t)page * a.stride_page + (size_t)(jc % (int)a.page_size) * a.stride_n) * esz + head_off;
+            kv[u].load(a.k_data + off);
+            vv[u].load(a.v_data + off);
+        }
+#pragma unroll
+        for (int u = 0; u < UNROLL; ++u) {
+            float kf[8], vf[8];
+            kv[u].to_float(kf);
+            vv[u].to_float(vf);
+            if (a.rope_mode == BZ_ROPE_FULL) {
+                const bool upper = lane_in_row >= LANES / 2;
+#pragma unroll
+                for (int e = 0; e < 8; ++e) {
+                    const float other = __shfl_xor(kf[e], LANES / 2, 64);
+                    const int fi = (lane_in_row % (LANES / 2)) * 8 + e;
+                    float s, c;
+                    sincosf((float)jj[u] * a.freqs.f[fi], &s, &c);
+                    kf[e] = upper ? (kf[e] * c + other * s) : (kf[e] * c - other * s);
+                }
+            }
+#pragma unroll
+            for (int g = 0; g < G; ++g) {
+                float s = 0.f;
+#pragma unroll
+                for (int e = 0; e < 8; ++e) s += q[g][e] * kf[e];
+#pragma unroll
+                for (int o = LANES / 2; o > 0; o >>= 1) s += __shfl_xor(s, o, 64);
+                s *= kscale;
+                if (valid[u]) {
+                    const float mn = fmaxf(m[g], s);
+                    const float sc = exp2f(m[g] - mn); // m = -inf on the first token gives 0
+                    const float p = exp2f(s - mn);
+                    l[g] = l[g] * sc + p;
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) acc[g][e] = acc[g][e] * sc + p * vf[e];
+                    m[g] = mn;
+                }
+            }
+        }
+    }
+
+    // ---- merge the token slots: first inside the wave, then across the 4 waves through LDS ----
+#pragma unroll
+    for (int g = 0; g < G; ++g) {
+#pragma unroll
+        for (int o = LANES; o < 64; o <<= 1) {
+            const float mo = __shfl_xor(m[g], o, 64);
+            const float lo = __shfl_xor(l[g], o, 64);
+            const float mn = fmaxf(m[g], mo);
+            const float sa = (m[g] == -INFINITY) ? 0.f : exp2f(m[g] - mn);
+            const float sb = (mo == -INFINITY) ? 0.f : exp2f(mo - mn);
+            l[g] = l[g] * sa + lo * sb;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                const float ao = __shfl_xor(acc[g][e], o, 64);
+                acc[g][e] = acc[g][e] * sa + ao * sb;
+            }
+            m[g] = mn;
+        }
+    }
+    __shared__ float sm_m[4][G];
+    __shared__ float sm_l[4][G];
+    __shared__ float sm_acc[4][G][D];
+    const int wave = tid / 64, lane = tid % 64;
+    if (lane < LANES) {
+#pragma unroll
+        for (int g = 0; g < G; ++g) {
+            if (lane == 0) { sm_m[wave][g] = m[g]; sm_l[wave][g] = l[g]; }
+#pragma unroll
+            for (int e = 0; e < 8; ++e) sm_acc[wave][g][lane * 8 + e] = acc[g][e];
+        }
+    }
+    __syncthreads();
+    const float vscale = a.v_scale ? a.v_scale[kvh] : 1.0f;
+    for (int idx = tid; idx < G * D; idx += 256) {
+        const int g = idx / D, d = idx % D;
+        float mm = -INFINITY;
+#pragma unroll
+        for (int w = 0; w < 4; ++w) mm = fmaxf(mm, sm_m[w][g]);
+        float ll = 0.f, oo = 0.f;
+#pragma unroll
+        for (int w = 0; w < 4; ++w) {
+            const float sc = (sm_m[w][g] == -INFINITY) ? 0.f : exp2f(sm_m[w][g] - mm);
+            ll += sm_l[w][g] * sc;
+            oo += sm_acc[w][g][d] * sc;
+        }
+        const float o = (ll > 0.f) ? oo / ll * vscale : 0.f;
+        const float lse2 = (ll > 0.f) ? mm + log2f(ll) : -INFINITY; // base-2 log-sum-exp of scaled logits
+        const int hq = kvh * G + g;
+        if (seg.partial < 0) {
+            reinterpret_cast<OT*>(a.out)[((size_t)b * a.num_qo_heads + hq) * D + d] = StoreCvt<OT>::from(o);
+            if (a.lse && d == 0) a.lse[(size_t)b * a.num_qo_heads + hq] = lse2 * 0.6931471805599453f;
+        } else {
+            a.part_o[((size_t)seg.partial * a.num_qo_heads + hq) * D + d] = o;
+            if (d == 0) a.part_lse[(size_t)seg.partial * a.num_qo_heads + hq] = lse2;
+        }
+    }
+}
+
+// ------------------------------------------------------------------------------------------
+// Split-K combine: o = sum_i o_i 2^(lse_i - M) / sum_i 2^(lse_i - M) over the partial results of
+// one sequence.  One workgroup of D lanes per (split sequence, q head).
+// ------------------------------------------------------------------------------------------
+template <typename OT>
+__global__ void decode_combine_kernel(const DecodeCombine* combos, const float* part_o, const float* part_lse,
+                                      void* out, float* lse, uint32_t num_qo_heads, uint32_t D) {
+    const DecodeCombine c = combos[blockIdx.x];
+    const uint32_t h = blockIdx.y, d = threadIdx.x;
+    float M = -INFINITY;
+    for (int i = 0; i < c.count; ++i) M = fmaxf(M, part_lse[(size_t)(c.first + i) * num_qo_heads + h]);
+    float wsum = 0.f, o = 0.f;
+    for (int i = 0; i < c.count; ++i) {
+        const float li = part_lse[(size_t)(c.first + i) * num_qo_heads + h];
+        const float w = (li == -INFINITY) ? 0.f : exp2f(li - M);
+        wsum += w;
+        o += w * part_o[((size_t)(c.first + i) * num_qo_heads + h) * D + d];
+    }
+    o = wsum > 0.f ? o / wsum : 0.f;
+    reinterpret_cast<OT*>(out)[((size_t)c.seq * num_qo_heads + h) * D + d] = StoreCvt<OT>::from(o);
+    if (lse && d == 0) lse[(size_t)c.seq * num_qo_heads + h] = (M + log2f(wsum)) * 0.6931471805599453f;
+}
+
+// zero rows of sequences with no pages (seq_len 0): the general kernel never visits them
+template <typename OT>
+__global__ void decode_zero_rows_kernel(const int32_t* empty_seqs, void* out, uint32_t row_elems) {
+    const int b = empty_seqs[blockIdx.x];
+    for (uint32_t i = threadIdx.x; i < row_elems; i += blockDim.x)
+        reinterpret_cast<OT*>(out)[(size_t)b * row_elems + i] = StoreCvt<OT>::from(0.f);
+}
+
+// ------------------------------------------------------------------------------------------
+// dispatch
+// ------------------------------------------------------------------------------------------
+template <typename QT, typename KVT, typename OT, int D>
+static int launch_general_g(const DecodeArgs& a, int G, dim3 grid, hipStream_t s) {
+    switch (G) {
+        case 1: hipLaunchKernelGGL((decode_general_kernel<QT, KVT, OT, D, 1>), grid, dim3(256), 0, s, a); break;
+        case 2: hipLaunchKernelGGL((decode_general_kernel<QT, KVT, OT, D, 2>), grid, dim3(256), 0, s, a); break;
+        case 4: hipLaunchKernelGGL((decode_general_kernel<QT, KVT, OT, D, 4>), grid, dim3(256), 0, s, a); break;
+        case 8: hipLaunchKernelGGL((decode_general_kernel<QT, KVT, OT, D, 8>), grid, dim3(256), 0, s, a); break;
+        default: return BZ_ERR_UNSUPPORTED;
+    }
+    BZ_LAUNCH_CHECK();
+    return 0;
+}
+
+template <typename QT, typename KVT, typename OT>
+static int launch_general_d(const DecodeArgs& a, int D, int G, dim3 grid, hipStream_t s) {
+    if (D == 128) return launch_general_g<QT, KVT, OT, 128>(a, G, grid, s);
+    if (D == 64) return launch_general_g<QT, KVT, OT, 64>(a, G, grid, s);
+    return BZ_ERR_UNSUPPORTED;
+}
+
+template <typename QT, typename OT>
+static int launch_general_kv(const DecodeArgs& a, int kv_dtype, int q_dtype, int D, int G, dim3 grid,
+                             hipStream_t s) {
+    if (kv_dtype == BZ_E4M3) return launch_general_d<QT, e4m3_t, OT>(a, D, G, grid, s);
+    if (kv_dtype == q_dtype) return launch_general_d<QT, QT, OT>(a, D, G, grid, s);
+    return BZ_ERR_UNSUPPORTED;
+}
+
+template <typename OT>
+static void launch_combine(const DecodePlan* p, void* out, float* lse, uint32_t Hq, uint32_t D, hipStream_t s) {
+    hipLaunchKernelGGL((decode_combine_kernel<OT>), dim3(p->num_combos, Hq), dim3(D), 0, s, p->combos_d, p->part_o,
+                       p->part_lse, out, lse, Hq, D);
+}
+template <typename OT>
+static void launch_zero(const DecodePlan* p, void* out, uint32_t row_elems, hipStream_t s) {
+    hipLaunchKernelGGL((decode_zero_rows_kernel<OT>), dim3(p->num_empty), dim3(256), 0, s, p->empty_d, out, row_elems);
+}
+
+int decode_fast_path(const DecodePlan* p, const DecodeArgs& a, int q_dtype, int kv_dtype, int out_dtype, int D,
+                     int G, const bz_paged_kv_t* kv, hipStream_t s); // bz_decode_mfma.hip
+
+} // namespace bz
+
+using namespace bz;
+
+extern "C" int bz_batch_decode(bz_decode_plan_t* plan_, const void* q, int q_dtype, const bz_paged_kv_t* kv,
+                               void* out, int out_dtype, uint32_t num_qo_heads, int rope_mode, float rope_theta,
+                               float sm_scale, const float* k_scale, const float* v_scale, float* lse,
+                               void* stream) {
+    DecodePlan* p = reinterpret_cast<DecodePlan*>(plan_);
+    if (!p || !kv || !q || !out) return BZ_ERR_BAD_ARG;
+    if (!p->planned) return BZ_ERR_NOT_PLANNED;
+    if (kv->batch_size != p->batch_size || kv->page_size != p->page_size || kv->num_kv_heads != p->num_kv_heads ||
+        kv->head_dim != p->head_dim || num_qo_heads != p->num_qo_heads)
+        return BZ_ERR_BAD_ARG;
+    if (q_dtype != BZ_F16 && q_dtype != BZ_BF16) return BZ_ERR_UNSUPPORTED;
+    if (out_dtype != q_dtype && out_dtype != BZ_F32) return BZ_ERR_UNSUPPORTED;
+    if (kv->kv_dtype != q_dtype && kv->kv_dtype != BZ_E4M3) return BZ_ERR_UNSUPPORTED;
+    if (num_qo_heads % kv->num_kv_heads) return BZ_ERR_BAD_ARG;
+    if (rope_mode < BZ_ROPE_NONE || rope_mode > BZ_ROPE_FULL) return BZ_ERR_BAD_ARG;
+    // 8-element vectors need rows that start on a vector boundary
+    if (kv->stride_n % 8 || kv->stride_h % 8 || kv->stride_page % 8) return BZ_ERR_BAD_ARG;
+    const int D = (int)kv->head_dim, G = (int)(num_qo_heads / kv->num_kv_heads);
+    hipStream_t s = (hipStream_t)stream;
+    if (p->batch_size == 0) return 0;
+
+    DecodeArgs a;
+    a.q = q; a.out = out; a.lse = lse;
+    a.k_data = (const char*)kv->k_data; a.v_data = (const char*)kv->v_data;
+    a.indices = kv->indices; a.indptr = kv->indptr; a.last_page_len = kv->last_page_len;
+    a.segments = p->segments_d;
+    a.part_o = p->part_o; a.part_lse = p->part_lse;
+    a.k_scale = k_scale; a.v_scale = v_scale;
+    a.stride_page = kv->stride_page; a.stride_n = kv->stride_n; a.stride_h = kv->stride_h;
+    a.page_size = kv->page_size; a.num_qo_heads = num_qo_heads; a.num_kv_heads = kv->num_kv_heads;
+    a.rope_mode = rope_mode;
+    if (!(sm_scale > 0.f)) sm_scale = 1.0f / sqrtf((float)D);
+    a.sm_scale_log2 = sm_scale * 1.4426950408889634f;
+    a.freqs = make_rope_freqs(D, rope_theta > 0.f ? rope_theta : 1e4f);
+
+    if (p->num_segments > 0) {
+        int rc = decode_fast_path(p, a, q_dtype, kv->kv_dtype, out_dtype, D, G, kv, s);
+        if (rc == BZ_ERR_UNSUPPORTED) {
+            dim3 grid(p->num_segments, kv->num_kv_heads);
+            if (q_dtype == BZ_F16)
+                rc = (out_dtype == BZ_F32) ? launch_general_kv<f16_t, float>(a, kv->kv_dtype, q_dtype, D, G, grid, s)
+                                           : launch_general_kv<f16_t, f16_t>(a, kv->kv_dtype, q_dtype, D, G, grid, s);
+            else
+                rc = (out_dtype == BZ_F32) ? launch_general_kv<bf16_t, float>(a, kv->kv_dtype, q_dtype, D, G, grid, s)
+                                           : launch_general_kv<bf16_t, bf16_t>(a, kv->kv_dtype, q_dtype, D, G, grid, s);
+        }
+        if (rc) return rc;
+    }
+    if (p->num_combos > 0) {
+        if (out_dtype == BZ_F32) launch_combine<float>(p, out, lse, num_qo_heads, D, s);
+        else if (out_dtype == BZ_F16) launch_combine<f16_t>(p, out, lse, num_qo_heads, D, s);
+        else launch_combine<bf16_t>(p, out, lse, num_qo_heads, D, s);
+        BZ_LAUNCH_CHECK();
+    }
+    if (p->num_empty > 0) {
+        const uint32_t row = num_qo_heads * D;
+        if (out_dtype == BZ_F32) launch_zero<float>(p, out, row, s);
+        else if (out_dtype == BZ_F16) launch_zero<f16_t>(p, out, row, s);
+        else launch_zero<bf16_t>(p, out, row, s);
+        BZ_LAUNCH_CHECK();
+    }
+    return 0;
+}

@@ -1,0 +1,41 @@
+// Decode schedule shared by the host planner and the decode kernels.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <vector>
+
+namespace bz {
+
+// One contiguous, page-aligned piece of one sequence's context.
+struct DecodeSegment {
+    int32_t seq;        // sequence index b
+    int32_t page_begin; // first page of the piece, relative to indptr[b]
+    int32_t page_end;   // one past the last page, relative to indptr[b]
+    int32_t partial;    // -1: the piece is the whole sequence, write the final row;
+                        // >=0: slot of the split-K partial result in the float workspace
+};
+
+// One split sequence: its partials are slots [first, first+count).
+struct DecodeCombine {
+    int32_t seq, first, count, pad;
+};
+
+struct DecodePlan {
+    bool planned = false;
+    uint32_t batch_size = 0, num_qo_heads = 0, num_kv_heads = 0, head_dim = 0, page_size = 0;
+    uint32_t num_segments = 0, num_combos = 0, num_empty = 0, num_partials = 0;
+    uint32_t num_workgroups = 0;
+    // device views into the caller's workspaces
+    const DecodeSegment* segments_d = nullptr;
+    const DecodeCombine* combos_d = nullptr;
+    const int32_t* empty_d = nullptr;
+    float* part_o = nullptr;
+    float* part_lse = nullptr;
+    // pinned staging for the schedule upload and the event that guards its reuse
+    void* staging = nullptr;
+    size_t staging_bytes = 0;
+    hipEvent_t upload_done = nullptr;
+    int device = -1;
+};
+
+} // namespace bz

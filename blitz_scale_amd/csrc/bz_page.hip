@@ -1,0 +1,251 @@
+// KV page writes for gfx950: prefill store and decode append, each optionally fused with the
+// Llama rotate-half RoPE of the new K rows and of the matching q rows, and with e4m3
+// quantisation for an fp8 pool.  Replaces src/kernel/page.cu of the BlitzScale worker; pool
+// helpers replace the allocation at src/blitz/cache_manager.h:136-142 and the layer pointer
+// bump at src/model/llama.h:378-381.
+#include <cmath>
+
+#include "bz_common.hpp"
+
+namespace bz {
+
+struct PageWriteArgs {
+    char* k_data;
+    char* v_data;
+    const int32_t* indices;
+    const int32_t* indptr;
+    const int32_t* last_page_len;
+    const void* k_src;
+    const void* v_src;
+    void* q_inout;
+    const int32_t* ragged_indptr; // prefill only
+    const float* k_scale;
+    const float* v_scale;
+    uint64_t stride_page, stride_n, stride_h;
+    uint32_t batch_size, page_size, num_kv_heads, num_qo_heads, num_tokens;
+    int rope;
+    RopeFreqs freqs;
+};
+
+// A row of D elements is handled by D/16 lanes; each lane owns 8 elements of the lower half and
+// the 8 elements of the upper half that form rotate-half pairs with them.
+template <typename ST, typename PT, int D, bool PREFILL>
+__global__ __launch_bounds__(256) void page_write_kernel(PageWriteArgs a) {
+    constexpr int LANES = D / 16;
+    constexpr int ROWS = 256 / LANES;
+    __shared__ float s_cos[D / 2], s_sin[D / 2];
+    __shared__ int s_b;
+
+    int b, pos;
+    size_t src_tok;
+    if (PREFILL) {
+        const int n = blockIdx.x; // global token index
+        if (threadIdx.x == 0) {
+            // largest b with ragged_indptr[b] <= n
+            int lo = 0, hi = (int)a.batch_size;
+            while (hi - lo > 1) {
+                const int mid = (lo + hi) / 2;
+                if (a.ragged_indptr[mid] <= n) lo = mid; else hi = mid;
+            }
+            s_b = lo;
+        }
+        __syncthreads();
+        b = s_b;
+        pos = n - a.ragged_indptr[b];
+        src_tok = (size_t)n;
+        if (n >= a.ragged_indptr[a.batch_size]) return;
+    } else {
+        b = blockIdx.x;
+        const int np = a.indptr[b + 1] - a.indptr[b];
+        if (np <= 0) return;
+        pos = (np - 1) * (int)a.page_size + a.last_page_len[b] - 1;
+        src_tok = (size_t)b;
+    }
+    const int64_t page = a.indices[a.indptr[b] + pos / (int)a.page_size];
+    const int slot = pos % (int)a.page_size;
+
+    if (a.rope) {
+        for (int i = threadIdx.x; i < D / 2; i += 256) {
+            float s, c;
+            sincosf((float)pos * a.freqs.f[i], &s, &c);
+            s_cos[i] = c;
+            s_sin[i] = s;
+        }
+        __syncthreads();
+    }
+
+    const int lane = threadIdx.x % LANES;
+    const int Hq = (a.rope && a.q_inout) ? (int)a.num_qo_heads : 0;
+    const int Hkv = (int)a.num_kv_heads;
+    const int total_rows = Hq + 2 * Hkv;
+    for (int r = threadIdx.x / LANES; r < total_rows; r += ROWS) {
+        if (r < Hq) { // q row: rotate in place
+            ST* row = reinterpret_cast<ST*>(a.q_inout) + (src_tok * a.num_qo_heads + r) * D;
+            Vec8<ST> lo, hi;
+            lo.load(row + lane * 8);
+            hi.load(row + D / 2 + lane * 8);
+            float x[8], y[8];
+            lo.to_float(x);
+            hi.to_float(y);
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                const float c = s_cos[lane * 8 + e], s = s_sin[lane * 8 + e];
+                const float xr = x[e] * c - y[e] * s, yr = y[e] * c + x[e] * s;
+                x[e] = xr;
+                y[e] = yr;
+            }
+            lo.from_float(x);
+            hi.from_float(y);
+            lo.store(row + lane * 8);
+            hi.store(row + D / 2 + lane * 8);
+            continue;
+        }
+        const bool is_k = r < Hq + Hkv;
+        const int h = is_k ? r - Hq : r - Hq - Hkv;
+        const ST* src = reinterpret_cast<const ST*>(is_k ? a.k_src : a.v_src) + (src_tok * Hkv + h) * D;
+        char* pool = is_k ? a.k_data : a.v_data;
+        const size_t off = ((size_t)page * a.stride_page + (size_t)slot * a.stride_n + (size_t)h * a.stride_h);
+        PT* dst = reinterpret_cast<PT*>(pool) + off;
+        Vec8<ST> lo, hi;
+        lo.load(src + lane * 8);
+        hi.load(src + D / 2 + lane * 8);
+        const bool rotate = is_k && a.rope;
+        const float* scale = is_k ? a.k_scale : a.v_scale;
+        if constexpr (sizeof(ST) == sizeof(PT)) {
+            if (!rotate && !scale) { // bit-exact copy
+                Vec8<PT> l2, h2;
+                l2.raw = lo.raw;
+                h2.raw = hi.raw;
+                l2.store(dst + lane * 8);
+                h2.store(dst + D / 2 + lane * 8);
+                continue;
+            }
+        }
+        float x[8], y[8];
+        lo.to_float(x);
+        hi.to_float(y);
+        if (rotate) {
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                const float c = s_cos[lane * 8 + e], s = s_sin[lane * 8 + e];
+                const float xr = x[e] * c - y[e] * s, yr = y[e] * c + x[e] * s;
+                x[e] = xr;
+                y[e] = yr;
+            }
+        }
+        if (scale) {
+            const float sc = scale[h];
+#pragma unroll
+            for (int e = 0; e < 8; ++e) { x[e] = x[e] / sc; y[e] = y[e] / sc; }
+        }
+        Vec8<PT> l2, h2;
+        l2.from_float(x);
+        h2.from_float(y);
+        l2.store(dst + lane * 8);
+        h2.store(dst + D / 2 + lane * 8);
+    }
+}
+
+template <typename ST, typename PT, bool PREFILL>
+static int launch_page_write_d(const PageWriteArgs& a, int D, uint32_t grid, hipStream_t s) {
+    if (grid == 0) return 0;
+    if (D == 128) hipLaunchKernelGGL((page_write_kernel<ST, PT, 128, PREFILL>), dim3(grid), dim3(256), 0, s, a);
+    else if (D == 64) hipLaunchKernelGGL((page_write_kernel<ST, PT, 64, PREFILL>), dim3(grid), dim3(256), 0, s, a);
+    else return BZ_ERR_UNSUPPORTED;
+    BZ_LAUNCH_CHECK();
+    return 0;
+}
+
+template <bool PREFILL>
+static int launch_page_write(const PageWriteArgs& a, int src_dtype, int pool_dtype, int D, uint32_t grid,
+                             hipStream_t s) {
+    if (src_dtype == BZ_F16 && pool_dtype == BZ_F16) return launch_page_write_d<f16_t, f16_t, PREFILL>(a, D, grid, s);
+    if (src_dtype == BZ_BF16 && pool_dtype == BZ_BF16) return launch_page_write_d<bf16_t, bf16_t, PREFILL>(a, D, grid, s);
+    if (src_dtype == BZ_F16 && pool_dtype == BZ_E4M3) return launch_page_write_d<f16_t, e4m3_t, PREFILL>(a, D, grid, s);
+    if (src_dtype == BZ_BF16 && pool_dtype == BZ_E4M3) return launch_page_write_d<bf16_t, e4m3_t, PREFILL>(a, D, grid, s);
+    return BZ_ERR_UNSUPPORTED;
+}
+
+static int fill_args(PageWriteArgs& a, const bz_paged_kv_t* kv, const void* k, const void* v, void* q_inout,
+                     uint32_t num_qo_heads, int rope, float rope_theta, const float* k_scale, const float* v_scale) {
+    if (!kv || !k || !v || !kv->k_data || !kv->v_data) return BZ_ERR_BAD_ARG;
+    if (kv->stride_n % 8 || kv->stride_h % 8 || kv->stride_page % 8) return BZ_ERR_BAD_ARG;
+    a.k_data = (char*)kv->k_data; a.v_data = (char*)kv->v_data;
+    a.indices = kv->indices; a.indptr = kv->indptr; a.last_page_len = kv->last_page_len;
+    a.k_src = k; a.v_src = v; a.q_inout = q_inout; a.ragged_indptr = nullptr;
+    a.k_scale = k_scale; a.v_scale = v_scale;
+    a.stride_page = kv->stride_page; a.stride_n = kv->stride_n; a.stride_h = kv->stride_h;
+    a.batch_size = kv->batch_size; a.page_size = kv->page_size; a.num_kv_heads = kv->num_kv_heads;
+    a.num_qo_heads = num_qo_heads; a.num_tokens = 0;
+    a.rope = rope ? 1 : 0;
+    a.freqs = make_rope_freqs((int)kv->head_dim, rope_theta > 0.f ? rope_theta : 1e4f);
+    return 0;
+}
+
+} // namespace bz
+
+using namespace bz;
+
+extern "C" int bz_store_prefill_kv(const bz_paged_kv_t* kv, const void* k, const void* v, int src_dtype,
+                                   const int32_t* ragged_indptr, uint32_t num_tokens, void* q_inout,
+                                   uint32_t num_qo_heads, int rope, float rope_theta, const float* k_scale,
+                                   const float* v_scale, void* stream) {
+    PageWriteArgs a;
+    int rc = fill_args(a, kv, k, v, q_inout, num_qo_heads, rope, rope_theta, k_scale, v_scale);
+    if (rc) return rc;
+    if (!ragged_indptr) return BZ_ERR_BAD_ARG;
+    a.ragged_indptr = ragged_indptr;
+    a.num_tokens = num_tokens;
+    if (kv->batch_size == 0) return 0;
+    return launch_page_write<true>(a, src_dtype, kv->kv_dtype, (int)kv->head_dim, num_tokens, (hipStream_t)stream);
+}
+
+extern "C" int bz_append_decode_kv(const bz_paged_kv_t* kv, const void* k, const void* v, int src_dtype,
+                                   void* q_inout, uint32_t num_qo_heads, int rope, float rope_theta,
+                                   const float* k_scale, const float* v_scale, void* stream) {
+    PageWriteArgs a;
+    int rc = fill_args(a, kv, k, v, q_inout, num_qo_heads, rope, rope_theta, k_scale, v_scale);
+    if (rc) return rc;
+    return launch_page_write<false>(a, src_dtype, kv->kv_dtype, (int)kv->head_dim, kv->batch_size,
+                                    (hipStream_t)stream);
+}
+
+// ---- pool helpers -----------------------------------------------------------------------------
+extern "C" void bz_paged_kv_set_layout(bz_paged_kv_t* kv, int layout) {
+    const uint64_t H = kv->num_kv_heads, P = kv->page_size, D = kv->head_dim;
+    kv->stride_page = 2 * H * P * D;
+    if (layout == BZ_LAYOUT_HND) { kv->stride_n = D; kv->stride_h = P * D; }
+    else { kv->stride_n = H * D; kv->stride_h = D; }
+}
+
+extern "C" uint64_t bz_kv_pool_bytes(uint32_t num_layers, uint64_t max_pages, uint32_t num_kv_heads,
+                                     uint32_t page_size, uint32_t head_dim, int kv_dtype) {
+    return (uint64_t)2 * num_layers * max_pages * num_kv_heads * page_size * head_dim * dtype_bytes(kv_dtype);
+}
+
+extern "C" int bz_kv_pool_alloc(void** base, uint64_t bytes) {
+    if (!base) return BZ_ERR_BAD_ARG;
+    return (int)hipMalloc(base, (size_t)bytes);
+}
+
+extern "C" int bz_kv_pool_free(void* base) { return (int)hipFree(base); }
+
+extern "C" void bz_kv_layer_view(bz_paged_kv_t* kv, void* pool_base, uint32_t layer, uint64_t max_pages) {
+    const uint64_t es = dtype_bytes(kv->kv_dtype);
+    char* k = (char*)pool_base + (uint64_t)layer * max_pages * kv->stride_page * es;
+    kv->k_data = k;
+    kv->v_data = k + (kv->stride_page / 2) * es;
+}
+
+extern "C" const char* bz_build_info(void) { return "blitz-scale paged-attention path, gfx950, wave64"; }
+
+extern "C" const char* bz_error_string(int code) {
+    switch (code) {
+        case 0: return "success";
+        case BZ_ERR_BAD_ARG: return "bz: invalid argument";
+        case BZ_ERR_UNSUPPORTED: return "bz: unsupported shape or type";
+        case BZ_ERR_WORKSPACE: return "bz: workspace too small";
+        case BZ_ERR_NOT_PLANNED: return "bz: plan() has not been called";
+        default: return hipGetErrorString((hipError_t)code);
+    }
+}

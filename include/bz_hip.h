@@ -1,0 +1,186 @@
+/*
+ * bz_hip.h -- C ABI of the MI355X (gfx950) paged-attention compute path.
+ *
+ * Every entry point replaces one wrapper of the BlitzScale worker's src/kernel
+ * directory (cited per function, paths relative to the reference checkout).
+ * Conventions shared by all of them, following the reference wrappers:
+ *   - all tensors, page tables and workspaces are caller-owned DEVICE memory
+ *     unless a parameter name ends in _h (host memory);
+ *   - launches are asynchronous on `stream` (a hipStream_t passed as void*;
+ *     NULL = the legacy default stream the reference uses everywhere) and never
+ *     synchronise the device;
+ *   - the return value is 0 on success, otherwise a hipError_t value (the C++
+ *     shim turns it into std::runtime_error like the reference does with
+ *     cudaError_t) or one of the BZ_ERR_* codes below for argument errors;
+ *   - nothing here allocates device memory except bz_kv_pool_alloc.
+ */
+#ifndef BZ_HIP_H_
+#define BZ_HIP_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* element types */
+#define BZ_F16 0
+#define BZ_BF16 1
+#define BZ_E4M3 2 /* OCP e4m3fn, KV pool only */
+#define BZ_F32 3  /* attention output only (test instantiation) */
+
+/* RoPE handling inside the attention kernels (Llama rotate-half, f_i = theta^(-2i/D)) */
+#define BZ_ROPE_NONE 0   /* q and cached K are used as they are                       */
+#define BZ_ROPE_Q_ONLY 1 /* q rotated at position seq_len-1; cached K already rotated */
+#define BZ_ROPE_FULL 2   /* q rotated at seq_len-1 and every cached K at its own      */
+                         /* position: the reference's kRoPELlama with a raw-K cache   */
+
+/* argument errors (outside the hipError_t range) */
+#define BZ_ERR_BAD_ARG 10001
+#define BZ_ERR_UNSUPPORTED 10002
+#define BZ_ERR_WORKSPACE 10003
+#define BZ_ERR_NOT_PLANNED 10004
+
+/* In-page element order of the KV pool. */
+#define BZ_LAYOUT_NHD 0 /* [page][K|V][slot][head][dim]: the reference's (page.h:24-32) */
+#define BZ_LAYOUT_HND 1 /* [page][K|V][head][slot][dim]: one (page, head) tile contiguous */
+
+/*
+ * One layer plane of the paged KV pool plus the per-batch CSR page table: the plain-C
+ * image of blitz::kernel::PageTable (src/kernel/page.h:12-64).  Element address relative
+ * to k_data / v_data:  page*stride_page + slot*stride_n + head*stride_h + d   (elements).
+ * seq_len_b = (indptr[b+1]-indptr[b]-1)*page_size + last_page_len[b]   (page.cu:38-40).
+ */
+typedef struct bz_paged_kv {
+    void* k_data;
+    void* v_data;
+    const int32_t* indices;       /* [indptr[batch_size]] page ids */
+    const int32_t* indptr;        /* [batch_size + 1]               */
+    const int32_t* last_page_len; /* [batch_size], 1..page_size     */
+    uint32_t batch_size;
+    uint32_t page_size;
+    uint32_t num_kv_heads;
+    uint32_t head_dim;
+    uint64_t stride_page;
+    uint64_t stride_n;
+    uint64_t stride_h;
+    int32_t kv_dtype;             /* BZ_F16 | BZ_BF16 | BZ_E4M3 */
+    int32_t reserved;
+} bz_paged_kv_t;
+
+/* Fill the stride fields for a layout (stride_page = 2*H*P*D for both; page.h:59-61). */
+void bz_paged_kv_set_layout(bz_paged_kv_t* kv, int layout);
+
+/* Bytes of one layer plane / of the whole pool: 2*L*max_pages*Hkv*P*D elements
+ * (src/blitz/cache_manager.h:136-142).  Address arithmetic is 64-bit throughout. */
+uint64_t bz_kv_pool_bytes(uint32_t num_layers, uint64_t max_pages, uint32_t num_kv_heads, uint32_t page_size,
+                          uint32_t head_dim, int kv_dtype);
+/* hipMalloc of the pool (replaces the cudaMalloc at cache_manager.h:136-142). */
+int bz_kv_pool_alloc(void** base, uint64_t bytes);
+int bz_kv_pool_free(void* base);
+/* k_data / v_data of layer `layer` (the pointer bump of src/model/llama.h:356-359,378-381). */
+void bz_kv_layer_view(bz_paged_kv_t* kv, void* pool_base, uint32_t layer, uint64_t max_pages);
+
+/* ---------------------------------------------------------------------------------------
+ * Decode plan: replaces BlitzBatchDecodeHandler::plan (src/kernel/flashinfer_types.h:44-72,
+ * flashinfer_types.cu:52-80).  Host-side scheduling from the HOST copies of indptr and
+ * last_page_len: cuts every sequence into page-aligned segments (split-K), balances them
+ * over the compute units and copies the schedule into int_buffer (device).  float_buffer
+ * (device) receives the split-K partial results at run time.  Synchronous host work plus
+ * one async H2D copy on `stream`, like the reference's plan().
+ * split_tokens: contexts longer than this are always split (0 = library default 2048,
+ * UINT32_MAX = never split: one piece per sequence).
+ * ------------------------------------------------------------------------------------- */
+typedef struct bz_decode_plan bz_decode_plan_t;
+
+bz_decode_plan_t* bz_decode_plan_create(void); /* create_flashinfer_decode_handler, flashinfer_types.cu:18-22 */
+void bz_decode_plan_destroy(bz_decode_plan_t* plan);
+int bz_decode_plan(bz_decode_plan_t* plan, void* float_buffer, size_t float_buffer_bytes, void* int_buffer,
+                   size_t int_buffer_bytes, const int32_t* indptr_h, const int32_t* last_page_len_h,
+                   uint32_t batch_size, uint32_t num_qo_heads, uint32_t num_kv_heads, uint32_t head_dim,
+                   uint32_t page_size, uint32_t split_tokens, void* stream);
+/* introspection for tests and the bench: number of segments / of sequences that were split */
+int bz_decode_plan_info(const bz_decode_plan_t* plan, uint32_t* num_segments, uint32_t* num_split_seqs,
+                        uint32_t* num_workgroups);
+
+/*
+ * batch_decode_attention (src/kernel/attention.h:24-31, attention_decode.cu:13-40).
+ * q, out: [batch, num_qo_heads, head_dim] of q_dtype (out_dtype may be BZ_F32 for tests).
+ * sm_scale <= 0 selects 1/sqrt(head_dim) (the default the reference never overrides).
+ * k_scale / v_scale: device fp32 [num_kv_heads] dequantisation factors for an e4m3 pool
+ * (NULL = 1).  lse: optional device fp32 [batch, num_qo_heads] (reference passes nullptr).
+ */
+int bz_batch_decode(bz_decode_plan_t* plan, const void* q, int q_dtype, const bz_paged_kv_t* kv, void* out,
+                    int out_dtype, uint32_t num_qo_heads, int rope_mode, float rope_theta, float sm_scale,
+                    const float* k_scale, const float* v_scale, float* lse, void* stream);
+
+/* ---------------------------------------------------------------------------------------
+ * Prefill plan: replaces BatchPrefillRaggedHandler::plan (flashinfer_types.h:12-41,
+ * flashinfer_types.cu:24-49).  Builds the (request, q-tile) work list, longest first.
+ * ------------------------------------------------------------------------------------- */
+typedef struct bz_prefill_plan bz_prefill_plan_t;
+
+bz_prefill_plan_t* bz_prefill_plan_create(void); /* create_flashinfer_prefill_handler, flashinfer_types.cu:12-16 */
+void bz_prefill_plan_destroy(bz_prefill_plan_t* plan);
+int bz_prefill_plan(bz_prefill_plan_t* plan, void* float_buffer, size_t float_buffer_bytes, void* int_buffer,
+                    size_t int_buffer_bytes, const int32_t* qo_indptr_h, const int32_t* kv_indptr_h,
+                    uint32_t batch_size, uint32_t num_qo_heads, uint32_t num_kv_heads, uint32_t head_dim,
+                    uint32_t page_size, void* stream);
+
+/*
+ * batch_prefill_attention (src/kernel/attention.h:9-22, attention_prefill.cu:11-46): ragged
+ * self-attention, q [N,Hq,D], k,v [N,Hkv,D], out [N,Hq,D], qo_indptr == kv_indptr (the only
+ * way the reference calls it, src/layer/attn.h:175-187).  causal != 0 masks j > i.
+ * rope_mode BZ_ROPE_NONE: q,k used as they are (rotate them first with bz_rope_store_prefill_kv);
+ * BZ_ROPE_FULL: q and k rows are rotated IN PLACE by their offset inside the request before the
+ * contraction (the caller's k buffer then holds rotated K for the page store that follows).
+ */
+int bz_batch_prefill_ragged(bz_prefill_plan_t* plan, void* q, const int32_t* qo_indptr, void* k, void* v,
+                            const int32_t* kv_indptr, void* out, int dtype, uint32_t batch_size,
+                            uint32_t num_qo_heads, uint32_t num_kv_heads, uint32_t head_dim, int causal,
+                            int rope_mode, float rope_theta, float sm_scale, void* stream);
+
+/* ---------------------------------------------------------------------------------------
+ * KV page writes
+ * ------------------------------------------------------------------------------------- */
+/* store_prefill_kv_cache (src/kernel/page.h:66-67, page.cu:21-94): token t of request b goes to
+ * page indices[indptr[b]+t/P], slot t%P.  k, v: [N, Hkv, D] of src_dtype.
+ * rope != 0 rotates K at position t on the way in; q_inout (optional, [N, Hq, D], num_qo_heads)
+ * is rotated in place by the same angles: the fused RoPE of the prefill path.
+ * k_scale / v_scale: device fp32 [Hkv]; for an e4m3 pool the value stored is quant(x / scale). */
+int bz_store_prefill_kv(const bz_paged_kv_t* kv, const void* k, const void* v, int src_dtype,
+                        const int32_t* ragged_indptr, uint32_t num_tokens, void* q_inout, uint32_t num_qo_heads,
+                        int rope, float rope_theta, const float* k_scale, const float* v_scale, void* stream);
+
+/* append_decode_kv_cache (src/kernel/page.h:69-70, page.cu:96-115): one new row per sequence at
+ * position seq_len-1 (page indices[indptr[b+1]-1], slot last_page_len[b]-1).  k, v: [B, Hkv, D].
+ * rope / q_inout as above with position seq_len-1: the fused RoPE + append of the decode path. */
+int bz_append_decode_kv(const bz_paged_kv_t* kv, const void* k, const void* v, int src_dtype, void* q_inout,
+                        uint32_t num_qo_heads, int rope, float rope_theta, const float* k_scale,
+                        const float* v_scale, void* stream);
+
+/* ---------------------------------------------------------------------------------------
+ * element-wise kernels of src/layer's call sites
+ * ------------------------------------------------------------------------------------- */
+/* rms_norm (src/kernel/rms_norm.h:11-19, norm.cu:7-22); input may alias output (llama.h:389-391) */
+int bz_rms_norm(const void* input, const void* weight, void* output, int dtype, uint32_t num_tokens,
+                uint32_t hidden_size, float eps, void* stream);
+/* add_rms_norm (rms_norm.h:26-34, norm.cu:24-39): residual += input; input = rms_norm(residual)*w */
+int bz_add_rms_norm(void* input, void* residual, const void* weight, int dtype, uint32_t num_tokens,
+                    uint32_t hidden_size, float eps, void* stream);
+/* silu_and_mul (src/kernel/activation.h:7-16, activation.cu:9-26): input [N, 2I] gate first, output [N, I] */
+int bz_silu_and_mul(const void* input, void* output, int dtype, uint32_t num_tokens, uint32_t inter_size,
+                    void* stream);
+/* add_residual (src/kernel/add.h:8-14, add.cu:13-61): residual += input, one rounding per element */
+int bz_add_residual(const void* input, void* residual, int dtype, uint32_t num_tokens, uint32_t dim,
+                    void* stream);
+
+/* library / device identification: "gfx950" build string, and hipGetErrorString passthrough */
+const char* bz_build_info(void);
+const char* bz_error_string(int code);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* BZ_HIP_H_ */

@@ -1,0 +1,49 @@
+"""CPU tests of the drop-in boundary: the shared library loads without a GPU and exports every
+symbol include/bz_hip.h declares; the ctypes table covers exactly that set."""
+import os
+import re
+
+from blitz_scale_amd import _lib
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def declared_symbols():
+    names = set()
+    for fn in os.listdir(os.path.join(ROOT, "include")):
+        if fn.endswith(".h"):
+            text = open(os.path.join(ROOT, "include", fn)).read()
+            text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+            names |= set(re.findall(r"\b(bz_[a-z0-9_]+)\s*\(", text))
+    return names
+
+
+def test_library_exports_every_declared_symbol():
+    lib = _lib.load()
+    decl = declared_symbols()
+    assert len(decl) >= 20
+    for name in sorted(decl):
+        assert hasattr(lib, name), f"{name} declared in include/ but not exported"
+    assert decl == set(_lib.SIGNATURES), (decl ^ set(_lib.SIGNATURES))
+
+
+def test_identification_and_error_strings_need_no_gpu():
+    lib = _lib.load()
+    assert b"gfx950" in lib.bz_build_info()
+    assert lib.bz_error_string(0) == b"success"
+    assert b"workspace" in lib.bz_error_string(_lib.BZ_ERR_WORKSPACE)
+
+
+def test_layout_strides_and_pool_size():
+    lib = _lib.load()
+    kv = _lib.BzPagedKV()
+    kv.num_kv_heads, kv.page_size, kv.head_dim, kv.kv_dtype = 8, 16, 128, _lib.BZ_BF16
+    lib.bz_paged_kv_set_layout(kv, _lib.BZ_LAYOUT_NHD)  # src/kernel/page.h:59-61
+    assert (kv.stride_page, kv.stride_n, kv.stride_h) == (2 * 8 * 16 * 128, 8 * 128, 128)
+    lib.bz_paged_kv_set_layout(kv, _lib.BZ_LAYOUT_HND)
+    assert (kv.stride_page, kv.stride_n, kv.stride_h) == (2 * 8 * 16 * 128, 128, 16 * 128)
+    # src/blitz/cache_manager.h:136-142: sizeof(T) * max_pages * (H*P*D) * 2 * layers
+    assert lib.bz_kv_pool_bytes(32, 30000, 8, 64, 128, _lib.BZ_F16) == 2 * 30000 * 8 * 64 * 128 * 2 * 32
+    lib.bz_kv_layer_view(kv, 1 << 40, 3, 1000)  # layer stride = max_pages * stride_page (llama.h:378-381)
+    assert kv.k_data == (1 << 40) + 3 * 1000 * kv.stride_page * 2
+    assert kv.v_data == kv.k_data + kv.stride_page  # v = k + H*P*D elements (page.h:42-43)

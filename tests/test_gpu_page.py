@@ -1,0 +1,123 @@
+"""GPU parity: KV page writes (prefill store, decode append, fused RoPE, e4m3 quantisation).
+Placement and raw copies are bit-exact; rotated / quantised rows are compared value-wise because the
+device uses fused multiply-adds in the rotation (one storage step on rare elements)."""
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from blitz_scale_amd import kernel as K
+from blitz_scale_amd import workloads as wl
+from blitz_scale_amd._lib import BZ_BF16, BZ_E4M3, BZ_F16, BZ_LAYOUT_HND, BZ_LAYOUT_NHD
+
+from _gpu import DeviceDecode, to_dev, to_host_bits
+from _util import DecodeProblem
+
+pytestmark = pytest.mark.gpu
+SENT = 0x7BFF
+
+
+def _setup(seed, lens, Hq, Hkv, D, P, dtype, layout, kv_dtype=None, reserve_extra=1):
+    p = DecodeProblem(seed, [l + reserve_extra for l in lens], Hq, Hkv, D, P, dtype, kv_dtype=kv_dtype, layout=layout)
+    fill = SENT if p.kv_dtype != BZ_E4M3 else 0x55
+    p.pool = np.full_like(p.pool, fill)
+    return p, fill
+
+
+@pytest.mark.parametrize("layout", [BZ_LAYOUT_NHD, BZ_LAYOUT_HND])
+@pytest.mark.parametrize("dtype,D,P", [(BZ_F16, 128, 16), (BZ_BF16, 128, 64), (BZ_F16, 64, 8)])
+def test_store_prefill_bit_exact(layout, dtype, D, P):
+    rng = np.random.default_rng(50)
+    lens, Hkv = [1, 15, 16, 17, 100, 333], 4
+    p, fill = _setup(51, lens, 8, Hkv, D, P, dtype, layout)
+    ri = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+    k, v = wl.randn_bits(rng, (ri[-1], Hkv, D), dtype), wl.randn_bits(rng, (ri[-1], Hkv, D), dtype)
+    want = p.pool.copy()
+    oracle.store_prefill_kv(p.oracle_kv(want), k, v, dtype, ri)
+    dev = DeviceDecode(p)
+    K.store_prefill_kv_cache(dev.pt, to_dev(k, dtype), to_dev(v, dtype), to_dev(ri.view(np.float32), 3).view(torch.int32))
+    torch.cuda.synchronize()
+    got = to_host_bits(dev.pool)
+    assert np.array_equal(got, want)
+    assert (got != fill).sum() >= 2 * ri[-1] * Hkv * D - 64  # only the stored rows changed
+
+
+@pytest.mark.parametrize("layout", [BZ_LAYOUT_NHD, BZ_LAYOUT_HND])
+@pytest.mark.parametrize("dtype", [BZ_F16, BZ_BF16])
+def test_append_decode_bit_exact(layout, dtype):
+    rng = np.random.default_rng(52)
+    ctx, Hkv, D, P = [1, 16, 17, 32, 33, 500, 0], 8, 128, 16
+    p = DecodeProblem(53, ctx, 32, Hkv, D, P, dtype, layout=layout)
+    p.pool = np.full_like(p.pool, SENT)
+    k, v = wl.randn_bits(rng, (len(ctx), Hkv, D), dtype), wl.randn_bits(rng, (len(ctx), Hkv, D), dtype)
+    want = p.pool.copy()
+    oracle.append_decode_kv(p.oracle_kv(want), k, v, dtype)
+    dev = DeviceDecode(p)
+    K.append_decode_kv_cache(dev.pt, to_dev(k, dtype), to_dev(v, dtype))
+    torch.cuda.synchronize()
+    assert np.array_equal(to_host_bits(dev.pool), want)
+    # position rule: page indices[indptr[b+1]-1], slot last_page_len[b]-1
+    b = 4
+    page, slot = int(p.indices[p.indptr[b + 1] - 1]), int(p.last_page_len[b]) - 1
+    off = page * p.stride_page + slot * p.stride_n + 3 * p.stride_h
+    assert np.array_equal(want[off:off + D], k[b, 3])
+
+
+@pytest.mark.parametrize("theta", [1e4, 5e5])
+def test_fused_rope_append(theta):
+    """Decode path: q rotated in place and the new K rotated into the cache at position seq_len-1."""
+    rng = np.random.default_rng(54)
+    ctx, Hq, Hkv, D, P, dtype = [1, 40, 2048, 8191], 32, 8, 128, 16, BZ_BF16
+    p = DecodeProblem(55, ctx, Hq, Hkv, D, P, dtype)
+    k, v = wl.randn_bits(rng, (4, Hkv, D), dtype), wl.randn_bits(rng, (4, Hkv, D), dtype)
+    want = p.pool.copy()
+    kv = p.oracle_kv(want)
+    oracle.append_decode_kv(kv, k, v, dtype, rope=True, rope_theta=theta)
+    want_q = oracle.rope_decode_q(p.q, dtype, kv, Hq, theta)
+    dev = DeviceDecode(p)
+    K.append_decode_kv_cache(dev.pt, to_dev(k, dtype), to_dev(v, dtype), q=dev.q, num_qo_heads=Hq, rope=True,
+                             rope_theta=theta)
+    torch.cuda.synchronize()
+    got, got_q = to_host_bits(dev.pool), to_host_bits(dev.q)
+    for g, w in ((got, want), (got_q, want_q)):
+        gf, wf = wl.to_f32(g, dtype), wl.to_f32(w, dtype)
+        assert np.abs(gf - wf).max() <= 2.0 ** -6  # at most one bf16 step at |x| < 4
+        assert (g != w).mean() < 2e-3
+    # and the decode over the appended cache agrees with the checker
+    dev.plan()
+    out = dev.decode(3)
+    ref = oracle.batch_decode(want_q, dtype, kv, Hq)
+    assert np.abs(out - ref).max() < 2e-3
+
+
+def test_fused_rope_store_prefill():
+    rng = np.random.default_rng(56)
+    lens, Hq, Hkv, D, P, dtype, theta = [3, 64, 130], 8, 4, 128, 16, BZ_F16, 1e4
+    p, fill = _setup(57, lens, Hq, Hkv, D, P, dtype, BZ_LAYOUT_HND)
+    ri = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+    q = wl.randn_bits(rng, (ri[-1], Hq, D), dtype)
+    k, v = wl.randn_bits(rng, (ri[-1], Hkv, D), dtype), wl.randn_bits(rng, (ri[-1], Hkv, D), dtype)
+    want = p.pool.copy()
+    oracle.store_prefill_kv(p.oracle_kv(want), k, v, dtype, ri, rope=True, rope_theta=theta)
+    want_q = oracle.rope_ragged(q, dtype, ri, Hq, D, theta)
+    dev = DeviceDecode(p)
+    qd = to_dev(q, dtype)
+    K.store_prefill_kv_cache(dev.pt, to_dev(k, dtype), to_dev(v, dtype), to_dev(ri.view(np.float32), 3).view(torch.int32),
+                             q=qd, num_qo_heads=Hq, rope=True, rope_theta=theta)
+    torch.cuda.synchronize()
+    for g, w in ((to_host_bits(dev.pool), want), (to_host_bits(qd), want_q)):
+        assert np.abs(wl.to_f32(g, dtype) - wl.to_f32(w, dtype)).max() <= 2.0 ** -8
+        assert (g != w).mean() < 2e-3
+
+
+def test_append_quantises_to_e4m3():
+    rng = np.random.default_rng(58)
+    ctx, Hkv, D, P = [5, 16, 100], 8, 128, 16
+    p = DecodeProblem(59, ctx, 64, Hkv, D, P, BZ_BF16, kv_dtype=BZ_E4M3)
+    k, v = wl.randn_bits(rng, (3, Hkv, D), BZ_BF16), wl.randn_bits(rng, (3, Hkv, D), BZ_BF16)
+    want = p.pool.copy()
+    oracle.append_decode_kv(p.oracle_kv(want), k, v, BZ_BF16, k_scale=p.k_scale, v_scale=p.v_scale)
+    dev = DeviceDecode(p)
+    K.append_decode_kv_cache(dev.pt, to_dev(k, BZ_BF16), to_dev(v, BZ_BF16), k_scale=dev.k_scale, v_scale=dev.v_scale)
+    torch.cuda.synchronize()
+    assert np.array_equal(to_host_bits(dev.pool), want)  # x / scale and RNE-saturating e4m3: bit exact
