@@ -287,8 +287,9 @@ static void launch_zero(const DecodePlan* p, void* out, uint32_t row_elems, hipS
     hipLaunchKernelGGL((decode_zero_rows_kernel<OT>), dim3(p->num_empty), dim3(256), 0, s, p->empty_d, out, row_elems);
 }
 
-int decode_fast_path(const DecodePlan* p, const DecodeArgs& a, int q_dtype, int kv_dtype, int out_dtype, int D,
-                     int G, const bz_paged_kv_t* kv, hipStream_t s); // bz_decode_mfma.hip
+int decode_fast_path(const DecodePlan* p, const void* q, void* out, float* lse, int q_dtype, int out_dtype,
+                     int rope_mode, float sm_scale_log2, const RopeFreqs& freqs, const bz_paged_kv_t* kv,
+                     uint32_t num_qo_heads, hipStream_t s); // bz_decode_mfma.hip
 
 } // namespace bz
 
@@ -330,7 +331,22 @@ extern "C" int bz_batch_decode(bz_decode_plan_t* plan_, const void* q, int q_dty
     a.freqs = make_rope_freqs(D, rope_theta > 0.f ? rope_theta : 1e4f);
 
     if (p->num_segments > 0) {
-        int rc = decode_fast_path(p, a, q_dtype, kv->kv_dtype, out_dtype, D, G, kv, s);
+        int rc = BZ_ERR_UNSUPPORTED;
+        const bool used_fast = !p->force_general && !k_scale && !v_scale;
+        if (used_fast)
+            rc = decode_fast_path(p, q, out, lse, q_dtype, out_dtype, rope_mode, a.sm_scale_log2, a.freqs, kv,
+                                  num_qo_heads, s);
+        if (rc == 0) {
+            // the MFMA path brings its own combine; only empty sequences are left to do
+            if (p->num_empty > 0) {
+                const uint32_t row = num_qo_heads * D;
+                if (out_dtype == BZ_F32) launch_zero<float>(p, out, row, s);
+                else if (out_dtype == BZ_F16) launch_zero<f16_t>(p, out, row, s);
+                else launch_zero<bf16_t>(p, out, row, s);
+                BZ_LAUNCH_CHECK();
+            }
+            return 0;
+        }
         if (rc == BZ_ERR_UNSUPPORTED) {
             dim3 grid(p->num_segments, kv->num_kv_heads);
             if (q_dtype == BZ_F16)

@@ -2,6 +2,7 @@
 // (src/kernel/flashinfer_types.cu:52-80 of the BlitzScale worker).  Pure integer work on the
 // host copies of the page table plus one asynchronous upload of the schedule.
 #include <algorithm>
+#include <cstdlib>
 #include <cstring>
 #include <new>
 #include <vector>
@@ -100,15 +101,73 @@ extern "C" int bz_decode_plan(bz_decode_plan_t* plan_, void* float_buffer, size_
         return (x.page_end - x.page_begin) > (y.page_end - y.page_begin);
     });
 
+    // ---- MFMA path schedule: equal shares of the flattened (sequence, kv head, tile) space ------
+    // Every wave slot of the chip (8 single-wave workgroups per CU) gets the same number of 32-token
+    // tiles; a share that crosses a (sequence, kv head) boundary becomes several pieces, and a
+    // (sequence, kv head) that is cut, or longer than split_tokens, is combined from partials.
+    std::vector<MfmaPiece> mp;
+    std::vector<int32_t> mptr;
+    std::vector<MfmaCombine> mc;
+    uint32_t mfma_partials = 0;
+    const uint32_t group = num_qo_heads / num_kv_heads;
+    const bool mfma_shape = head_dim == 128 && page_size % 16 == 0 && group <= 16;
+    if (mfma_shape) {
+        uint64_t total_tiles = 0;
+        for (uint32_t b = 0; b < batch_size; ++b) {
+            const int32_t np = indptr_h[b + 1] - indptr_h[b];
+            if (np <= 0) continue;
+            const int64_t len = (int64_t)(np - 1) * page_size + last_page_len_h[b];
+            total_tiles += (uint64_t)((len + 31) / 32) * num_kv_heads;
+        }
+        const uint64_t max_slots = (uint64_t)cus * 8;
+        const uint64_t share = std::max<uint64_t>(1, (total_tiles + max_slots - 1) / max_slots);
+        const uint32_t cap_tiles = never_split ? 0x7fffffffu : std::max<uint32_t>(1, split_tokens / 32);
+        uint64_t room = share; // tiles the current slot can still take
+        mptr.push_back(0);
+        for (uint32_t b = 0; b < batch_size; ++b) {
+            const int32_t np = indptr_h[b + 1] - indptr_h[b];
+            if (np <= 0) continue;
+            const int64_t len = (int64_t)(np - 1) * page_size + last_page_len_h[b];
+            const int32_t tiles = (int32_t)((len + 31) / 32);
+            for (uint32_t h = 0; h < num_kv_heads; ++h) {
+                const size_t first_piece = mp.size();
+                int32_t t = 0;
+                while (t < tiles) {
+                    if (room == 0) { mptr.push_back((int32_t)mp.size()); room = share; }
+                    const int32_t take = (int32_t)std::min<uint64_t>({(uint64_t)(tiles - t), never_split ? (uint64_t)(tiles - t) : room, cap_tiles});
+                    mp.push_back({(int32_t)b, (int32_t)h, t, t + take, -1, {0, 0, 0}});
+                    t += take;
+                    room = (never_split && room < (uint64_t)take) ? 0 : room - std::min<uint64_t>(room, take);
+                }
+                const size_t cnt = mp.size() - first_piece;
+                if (cnt > 1) {
+                    mc.push_back({(int32_t)b, (int32_t)h, (int32_t)mfma_partials, (int32_t)cnt});
+                    for (size_t i = 0; i < cnt; ++i) mp[first_piece + i].partial = (int32_t)(mfma_partials + i);
+                    mfma_partials += (uint32_t)cnt;
+                }
+            }
+        }
+        mptr.push_back((int32_t)mp.size());
+    }
+
     // ---- workspaces -------------------------------------------------------------------------
     const size_t seg_bytes = align_up(segs.size() * sizeof(DecodeSegment), 256);
     const size_t combo_bytes = align_up(combos.size() * sizeof(DecodeCombine), 256);
     const size_t empty_bytes = align_up(empty.size() * sizeof(int32_t), 256);
-    const size_t total = seg_bytes + combo_bytes + empty_bytes;
-    if (total > int_buffer_bytes) return BZ_ERR_WORKSPACE;
+    const size_t base_total = seg_bytes + combo_bytes + empty_bytes;
+    if (base_total > int_buffer_bytes) return BZ_ERR_WORKSPACE;
     const size_t part_o_bytes = align_up((size_t)partials * num_qo_heads * head_dim * sizeof(float), 256);
     const size_t part_lse_bytes = align_up((size_t)partials * num_qo_heads * sizeof(float), 256);
     if (part_o_bytes + part_lse_bytes > float_buffer_bytes) return BZ_ERR_WORKSPACE;
+    // the MFMA schedule is optional: without room for it the general kernel runs
+    const size_t mp_bytes = align_up(mp.size() * sizeof(MfmaPiece), 256);
+    const size_t mptr_bytes = align_up(mptr.size() * sizeof(int32_t), 256);
+    const size_t mc_bytes = align_up(mc.size() * sizeof(MfmaCombine), 256);
+    const size_t mpart_o_bytes = align_up((size_t)mfma_partials * 16 * 128 * sizeof(float), 256);
+    const size_t mpart_lse_bytes = align_up((size_t)mfma_partials * 16 * sizeof(float), 256);
+    const bool mfma_ok = mfma_shape && !mp.empty() && base_total + mp_bytes + mptr_bytes + mc_bytes <= int_buffer_bytes &&
+                         mpart_o_bytes + mpart_lse_bytes <= float_buffer_bytes;
+    const size_t total = mfma_ok ? base_total + mp_bytes + mptr_bytes + mc_bytes : base_total;
 
     hipStream_t s = (hipStream_t)stream;
     if (!p->upload_done) BZ_CHECK_HIP(hipEventCreateWithFlags(&p->upload_done, hipEventDisableTiming));
@@ -126,6 +185,11 @@ extern "C" int bz_decode_plan(bz_decode_plan_t* plan_, void* float_buffer, size_
     if (!segs.empty()) memcpy(st, segs.data(), segs.size() * sizeof(DecodeSegment));
     if (!combos.empty()) memcpy(st + seg_bytes, combos.data(), combos.size() * sizeof(DecodeCombine));
     if (!empty.empty()) memcpy(st + seg_bytes + combo_bytes, empty.data(), empty.size() * sizeof(int32_t));
+    if (mfma_ok) {
+        memcpy(st + base_total, mp.data(), mp.size() * sizeof(MfmaPiece));
+        memcpy(st + base_total + mp_bytes, mptr.data(), mptr.size() * sizeof(int32_t));
+        if (!mc.empty()) memcpy(st + base_total + mp_bytes + mptr_bytes, mc.data(), mc.size() * sizeof(MfmaCombine));
+    }
     if (total) BZ_CHECK_HIP(hipMemcpyAsync(int_buffer, st, total, hipMemcpyHostToDevice, s));
     BZ_CHECK_HIP(hipEventRecord(p->upload_done, s));
 
@@ -139,6 +203,26 @@ extern "C" int bz_decode_plan(bz_decode_plan_t* plan_, void* float_buffer, size_
     p->num_segments = (uint32_t)segs.size(); p->num_combos = (uint32_t)combos.size();
     p->num_empty = (uint32_t)empty.size(); p->num_partials = partials;
     p->num_workgroups = (uint32_t)segs.size() * num_kv_heads;
+    p->mfma_ok = mfma_ok;
+    if (mfma_ok) {
+        p->mfma_pieces_d = (const MfmaPiece*)((char*)int_buffer + base_total);
+        p->mfma_piece_ptr_d = (const int32_t*)((char*)int_buffer + base_total + mp_bytes);
+        p->mfma_combos_d = (const MfmaCombine*)((char*)int_buffer + base_total + mp_bytes + mptr_bytes);
+        p->mfma_part_o = (float*)float_buffer; // the two paths never run in the same call: same workspace
+        p->mfma_part_lse = (float*)((char*)float_buffer + mpart_o_bytes);
+        p->mfma_slots = (uint32_t)mptr.size() - 1;
+        p->mfma_pieces = (uint32_t)mp.size();
+        p->mfma_combos = (uint32_t)mc.size();
+        p->mfma_partials = mfma_partials;
+        int32_t last = -1;
+        p->mfma_split_seqs = 0;
+        for (const MfmaCombine& c : mc)
+            if (c.seq != last) { ++p->mfma_split_seqs; last = c.seq; }
+    }
+    // BZ_DECODE_PATH=general keeps the MFMA kernel out (used to test the general kernel on shapes
+    // both kernels cover)
+    const char* path = getenv("BZ_DECODE_PATH");
+    p->force_general = path && !strcmp(path, "general");
     p->planned = true;
     return 0;
 }
@@ -147,8 +231,9 @@ extern "C" int bz_decode_plan_info(const bz_decode_plan_t* plan_, uint32_t* num_
                                    uint32_t* num_workgroups) {
     const DecodePlan* p = reinterpret_cast<const DecodePlan*>(plan_);
     if (!p || !p->planned) return BZ_ERR_NOT_PLANNED;
-    if (num_segments) *num_segments = p->num_segments;
-    if (num_split_seqs) *num_split_seqs = p->num_combos;
-    if (num_workgroups) *num_workgroups = p->num_workgroups;
+    const bool mfma = p->mfma_ok && !p->force_general;
+    if (num_segments) *num_segments = mfma ? p->mfma_pieces : p->num_segments;
+    if (num_split_seqs) *num_split_seqs = mfma ? p->mfma_split_seqs : p->num_combos;
+    if (num_workgroups) *num_workgroups = mfma ? p->mfma_slots : p->num_workgroups;
     return 0;
 }

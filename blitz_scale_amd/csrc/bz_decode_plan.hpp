@@ -20,6 +20,19 @@ struct DecodeCombine {
     int32_t seq, first, count, pad;
 };
 
+// MFMA path: a contiguous run of 32-token tiles of one (sequence, kv head).
+struct MfmaPiece {
+    int32_t seq, kvh;
+    int32_t tile_begin, tile_end; // in 32-token tiles from the start of the sequence
+    int32_t partial;              // -1: whole (sequence, kv head) -> final rows; else partial slot
+    int32_t pad[3];
+};
+
+// One split (sequence, kv head): partial slots [first, first+count).
+struct MfmaCombine {
+    int32_t seq, kvh, first, count;
+};
+
 struct DecodePlan {
     bool planned = false;
     uint32_t batch_size = 0, num_qo_heads = 0, num_kv_heads = 0, head_dim = 0, page_size = 0;
@@ -31,6 +44,15 @@ struct DecodePlan {
     const int32_t* empty_d = nullptr;
     float* part_o = nullptr;
     float* part_lse = nullptr;
+    // MFMA path schedule (valid when mfma_ok)
+    bool mfma_ok = false;
+    bool force_general = false; // tests: run the general kernel even where the MFMA path applies
+    uint32_t mfma_slots = 0, mfma_combos = 0, mfma_partials = 0, mfma_pieces = 0, mfma_split_seqs = 0;
+    const MfmaPiece* mfma_pieces_d = nullptr;
+    const int32_t* mfma_piece_ptr_d = nullptr;
+    const MfmaCombine* mfma_combos_d = nullptr;
+    float* mfma_part_o = nullptr;
+    float* mfma_part_lse = nullptr;
     // pinned staging for the schedule upload and the event that guards its reuse
     void* staging = nullptr;
     size_t staging_bytes = 0;

@@ -5,6 +5,8 @@ The fp32-output instantiation is held to 2e-5 to show the arithmetic itself agre
 is stored in bf16 the bound is widened to half a bf16 step for |o| >= 0.5 (the storage grid is then
 coarser than 2e-3).
 """
+import os
+
 import numpy as np
 import pytest
 import torch
@@ -21,10 +23,21 @@ pytestmark = pytest.mark.gpu
 
 
 def check(p, split_tokens=0, rope_mode=BZ_ROPE_NONE, theta=1e4, f32_tol=2e-5, parallel=False):
-    dev = DeviceDecode(p)
-    info = dev.plan(split_tokens)
+    """Both kernels are held to the same bar: the MFMA kernel where it applies (library default) and
+    the general kernel (BZ_DECODE_PATH=general at plan time)."""
     ref, ref_lse = oracle.batch_decode(p.q, p.dtype, p.oracle_kv(), p.Hq, rope_mode=rope_mode, rope_theta=theta,
                                        k_scale=p.k_scale, v_scale=p.v_scale, want_lse=True, parallel=parallel)
+    os.environ["BZ_DECODE_PATH"] = "general"
+    try:
+        _check_one(p, split_tokens, rope_mode, theta, f32_tol, ref, ref_lse)
+    finally:
+        del os.environ["BZ_DECODE_PATH"]
+    return _check_one(p, split_tokens, rope_mode, theta, f32_tol, ref, ref_lse)
+
+
+def _check_one(p, split_tokens, rope_mode, theta, f32_tol, ref, ref_lse):
+    dev = DeviceDecode(p)
+    info = dev.plan(split_tokens)
     got32, lse = dev.decode(BZ_F32, rope_mode, theta, want_lse=True)
     err32 = np.abs(got32 - ref).max()
     assert err32 <= f32_tol, f"fp32-out max abs err {err32}"
