@@ -7,7 +7,8 @@ import ctypes as C
 import os
 
 HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(HERE, "lib", "libbz_hip.so")
+# BZ_HIP_LIB points at another build of the same library (e.g. an experimental kernel variant)
+LIB_PATH = os.environ.get("BZ_HIP_LIB") or os.path.join(HERE, "lib", "libbz_hip.so")
 
 BZ_F16, BZ_BF16, BZ_E4M3, BZ_F32 = 0, 1, 2, 3
 BZ_ROPE_NONE, BZ_ROPE_Q_ONLY, BZ_ROPE_FULL = 0, 1, 2

@@ -36,7 +36,8 @@ struct MfmaDecodeArgs {
     const int32_t* indptr;
     const int32_t* last_page_len;
     const MfmaPiece* pieces;
-    const int32_t* piece_ptr;
+    const MfmaTile* tiles;
+    const int32_t* tile_ptr;
     float* part_o;   // [num_partials][16][128]
     float* part_lse; // [num_partials][16]
     uint64_t stride_page, stride_n, stride_h; // elements
@@ -78,19 +79,37 @@ template <> struct Mma<false> {
 
 __device__ __forceinline__ uint32_t& u4(uint4& v, int i) { return reinterpret_cast<uint32_t*>(&v)[i]; }
 
-// The read-only inputs are separate __restrict__ parameters so that wave-uniform reads of the page
-// table and of the schedule go through the scalar unit.
+// The read-only inputs are separate __restrict__ parameters so that wave-uniform reads go through
+// the scalar unit.
+//
+// Under load a dependent memory round trip costs several microseconds, so the kernel has none in its
+// steady state: the planner lists every tile of a wave slot as a 16-byte record, and the wave fetches
+// the records, the page ids they point at and the metadata of their pieces for 32 tiles at a time
+// (one lane per tile) well before they are needed; inside the tile loop everything wave-uniform comes
+// out of those registers with v_readlane.  The K/V loads of tile g+1 and the q rows of the next piece
+// are issued before the arithmetic of tile g.
+// wave-level ordering of LDS traffic: LDS instructions of one wave execute in order, so making the
+// compiler keep the order is all that is needed (a workgroup barrier would also drain the global loads
+// that are in flight for the next tile)
+__device__ __forceinline__ void wave_lds_sync() {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
+
+constexpr int kInfoInts = 12; // per-tile description kept in LDS (see fetch_info)
+
 template <bool BF16, typename OT, bool ROPE_Q>
 __global__ __launch_bounds__(64, 2) void decode_mfma_kernel(MfmaDecodeArgs a, const char* __restrict__ q_ptr,
                                                             const char* __restrict__ k_data,
                                                             const char* __restrict__ v_data,
                                                             const int32_t* __restrict__ indices,
-                                                            const int32_t* __restrict__ indptr,
-                                                            const int32_t* __restrict__ last_page_len,
                                                             const MfmaPiece* __restrict__ pieces,
-                                                            const int32_t* __restrict__ piece_ptr) {
+                                                            const MfmaTile* __restrict__ tiles,
+                                                            const int32_t* __restrict__ tile_ptr) {
     using M = Mma<BF16>;
     __shared__ __attribute__((aligned(16))) unsigned char v_lds[kTileTok * kVRowBytes];
+    __shared__ __attribute__((aligned(16))) int info_lds[2][32][kInfoInts];
 
     const int lane = threadIdx.x;
     const int n = lane & 15; // query head (scores) / d column (output) / token row (K operand)
@@ -99,27 +118,121 @@ __global__ __launch_bounds__(64, 2) void decode_mfma_kernel(MfmaDecodeArgs a, co
     const size_t row_bytes = (size_t)a.stride_n * 2;
     const int G = (int)a.group;
 
-    const int p_begin = piece_ptr[blockIdx.x], p_end = piece_ptr[blockIdx.x + 1];
-    for (int pi = p_begin; pi < p_end; ++pi) {
-        const MfmaPiece pc = pieces[pi];
-        const int b = pc.seq, kvh = pc.kvh;
-        const int ip0 = indptr[b];
-        const int npages = indptr[b + 1] - ip0;
-        const int seq_len = (npages - 1) * P + last_page_len[b];
-        const int tok_end = min(pc.tile_end * kTileTok, seq_len);
-        const size_t head_bytes = (size_t)kvh * a.stride_h * 2;
+    const int g_begin = tile_ptr[blockIdx.x], g_end = tile_ptr[blockIdx.x + 1];
+    if (g_begin >= g_end) return;
+#if defined(BZ_EXP) && BZ_EXP >= 3
+    long long* ts_buf = reinterpret_cast<long long*>(reinterpret_cast<char*>(a.part_o) + (64u << 20));
+    if (lane == 0) ts_buf[blockIdx.x * 4 + 0] = wall_clock64();
+    int exp_pieces = 0;
+#endif
 
-        // ---- Q as MFMA B operand: lane (head n, group j) holds q[head][32*ks + 8*j .. +7], ks = 0..3.
-        // With in-kernel RoPE the rotated q is split into a storage-precision head and tail (q = hi + lo)
-        // and both are contracted, so the rotation costs no precision.
-        uint4 qhi[4], qlo[4];
+    // ---- descriptions of 32 tiles at a time: lane l < 32 fetches the record of tile base+l, the two
+    // page ids it points at and the piece it belongs to, and leaves 12 ints in LDS:
+    //   [pid0, pid1, t, seq | kvh, flags (1: first tile of its piece, 2: last), partial, tok_end | seq_len]
+    struct Desc { int v[9]; };
+    auto fetch_info = [&](int base) -> Desc {
+        Desc d;
+        const int g = base + (lane & 31);
+        const bool live = g < g_end;
+        const MfmaTile rec = live ? tiles[g] : MfmaTile{0, 0, 0, 0};
+        const int4 m0 = live ? *reinterpret_cast<const int4*>(&pieces[rec.piece]) : make_int4(0, 0, 0, 0);
+        const int4 m1 = live ? *(reinterpret_cast<const int4*>(&pieces[rec.piece]) + 1) : make_int4(0, 0, 0, 0);
+        const int4 m2 = live ? *(reinterpret_cast<const int4*>(&pieces[rec.piece]) + 2) : make_int4(0, 0, 0, 0);
+        d.v[0] = live ? indices[rec.idx0] : 0;
+        d.v[1] = live ? indices[rec.idx1] : 0;
+        d.v[2] = rec.t;
+        d.v[3] = m0.x;                                             // seq
+        d.v[4] = m0.y;                                             // kvh
+        d.v[5] = (rec.t == m0.z ? 1 : 0) | (rec.t + 1 == m0.w ? 2 : 0);
+        d.v[6] = m1.x;                                             // partial slot or -1
+        d.v[7] = min(m0.w * kTileTok, m2.z);                       // tok_end of the piece
+        d.v[8] = m2.z;                                             // seq_len
+        return d;
+    };
+    auto stash_info = [&](const Desc& d, int buf) {
+        if (lane < 32) {
+            int* dst = &info_lds[buf][lane][0];
+            *reinterpret_cast<int4*>(dst) = make_int4(d.v[0], d.v[1], d.v[2], d.v[3]);
+            *reinterpret_cast<int4*>(dst + 4) = make_int4(d.v[4], d.v[5], d.v[6], d.v[7]);
+            dst[8] = d.v[8];
+        }
+    };
+    struct TileUni { int pid0, pid1, t, seq, kvh, flags, partial, tok_end, seq_len; }; // wave-uniform
+    auto read_info = [&](int buf, int i) -> TileUni {
+        const int* src = &info_lds[buf][i][0];
+        const int4 x = *reinterpret_cast<const int4*>(src);
+        const int4 y = *reinterpret_cast<const int4*>(src + 4);
+        const int z = src[8];
+        TileUni u;
+        u.pid0 = __builtin_amdgcn_readfirstlane(x.x); u.pid1 = __builtin_amdgcn_readfirstlane(x.y);
+        u.t = __builtin_amdgcn_readfirstlane(x.z); u.seq = __builtin_amdgcn_readfirstlane(x.w);
+        u.kvh = __builtin_amdgcn_readfirstlane(y.x); u.flags = __builtin_amdgcn_readfirstlane(y.y);
+        u.partial = __builtin_amdgcn_readfirstlane(y.z); u.tok_end = __builtin_amdgcn_readfirstlane(y.w);
+        u.seq_len = __builtin_amdgcn_readfirstlane(z);
+        return u;
+    };
+
+    uint4 kreg[2][4], vreg[8], qnext[4];
+    auto issue_loads = [&](const TileUni& u) {
+        size_t base[2];
+        const int pid[2] = {u.pid0, u.pid1};
 #pragma unroll
-        for (int ks = 0; ks < 4; ++ks) { qhi[ks] = make_uint4(0, 0, 0, 0); qlo[ks] = make_uint4(0, 0, 0, 0); }
+        for (int s = 0; s < 2; ++s) {
+            const int slot0 = (u.t * kTileTok + 16 * s) % P; // a subtile past the last page reads the last page, masked later
+            base[s] = ((size_t)pid[s] * a.stride_page + (size_t)slot0 * a.stride_n + (size_t)u.kvh * a.stride_h) * 2;
+        }
+#pragma unroll
+        for (int ks = 0; ks < 4; ++ks) {
+            kreg[0][ks] = *reinterpret_cast<const uint4*>(k_data + base[0] + (size_t)n * row_bytes + ks * 64 + j * 16);
+            kreg[1][ks] = *reinterpret_cast<const uint4*>(k_data + base[1] + (size_t)n * row_bytes + ks * 64 + j * 16);
+        }
+#pragma unroll
+        for (int w = 0; w < 8; ++w) { // rows 4w..4w+3 of the tile, 16 lanes x 16 B per row
+            const int row = 4 * w + j;
+            vreg[w] = *reinterpret_cast<const uint4*>(v_data + base[row >> 4] + (size_t)(row & 15) * row_bytes + n * 16);
+        }
+    };
+    // q rows of a piece as MFMA B operand: lane (head n, group j) holds q[head][32*ks + 8*j .. +7]
+    auto issue_q = [&](const TileUni& u) {
+#pragma unroll
+        for (int ks = 0; ks < 4; ++ks) qnext[ks] = make_uint4(0, 0, 0, 0);
         if (n < G) {
-            const char* qrow = q_ptr + ((size_t)b * a.num_qo_heads + (size_t)kvh * G + n) * 256;
+            const char* qrow = q_ptr + ((size_t)u.seq * a.num_qo_heads + (size_t)u.kvh * G + n) * 256;
 #pragma unroll
-            for (int ks = 0; ks < 4; ++ks) qhi[ks] = *reinterpret_cast<const uint4*>(qrow + ks * 64 + j * 16);
-            if (ROPE_Q) {
+            for (int ks = 0; ks < 4; ++ks) qnext[ks] = *reinterpret_cast<const uint4*>(qrow + ks * 64 + j * 16);
+        }
+    };
+
+    {
+        const Desc d0 = fetch_info(g_begin);
+        stash_info(d0, 0);
+        wave_lds_sync();
+    }
+    int chunk_base = g_begin, buf = 0;
+    Desc dnext;
+    TileUni un = read_info(0, 0); // description of the tile whose loads are issued next
+    issue_q(un);
+    issue_loads(un);
+
+
+    uint4 qhi[4], qlo[4];
+    float m_run = -INFINITY, l_run = 0.f;
+    f32x4_t acc[8];
+
+    for (int g = g_begin; g < g_end; ++g) {
+        const TileUni uc = un; // the tile computed in this iteration (its loads are in flight or done)
+        const int i = g - chunk_base;
+        // descriptions of the next 32 tiles: fetched at i == 8, parked in the other LDS buffer at i == 24
+        if (i == 8 && chunk_base + 32 < g_end) dnext = fetch_info(chunk_base + 32);
+        if (i == 24 && chunk_base + 32 < g_end) { stash_info(dnext, buf ^ 1); wave_lds_sync(); }
+        const int t = uc.t, tok_end = uc.tok_end, seq_len = uc.seq_len;
+
+        if (uc.flags & 1) { // ================= first tile of a piece =================
+#pragma unroll
+            for (int ks = 0; ks < 4; ++ks) { qhi[ks] = qnext[ks]; qlo[ks] = make_uint4(0, 0, 0, 0); }
+            if (ROPE_Q && n < G) {
+                // the rotated q is split into a storage-precision head and tail (q = hi + lo) and both are
+                // contracted, so rotating inside the kernel costs no precision
                 const float pos = (float)(seq_len - 1);
 #pragma unroll
                 for (int ks = 0; ks < 2; ++ks) { // dims d = 32ks+8j+e pair with d+64, held at ks+2
@@ -143,191 +256,212 @@ __global__ __launch_bounds__(64, 2) void decode_mfma_kernel(MfmaDecodeArgs a, co
                     }
                 }
             }
+            m_run = -INFINITY;
+            l_run = 0.f;
+#pragma unroll
+            for (int d = 0; d < 8; ++d) acc[d] = f32x4_t{0.f, 0.f, 0.f, 0.f};
         }
 
-        float m_run = -INFINITY, l_run = 0.f;
-        f32x4_t acc[8];
+        // ================= one tile =================
+        const int tile_tok0 = t * kTileTok;
+        const bool ragged = tile_tok0 + kTileTok > tok_end; // wave-uniform
+        wave_lds_sync(); // transposed reads of the previous tile come before V is overwritten
+#if defined(BZ_EXP) && BZ_EXP == 4
+        { uint32_t x = 0;
 #pragma unroll
-        for (int d = 0; d < 8; ++d) acc[d] = f32x4_t{0.f, 0.f, 0.f, 0.f};
-
-        // Page ids of the two 16-token subtiles of a tile.  A tile may reach past the last page of the
-        // sequence: the lookup stays in bounds (last page, slot 0) and the tokens are masked later.
-        // The ids are fetched one tile ahead of the loads that need them.
-        int pid[2];
-        auto load_pids = [&](int tile) {
+          for (int w = 0; w < 8; ++w) x ^= vreg[w].x ^ vreg[w].y ^ vreg[w].z ^ vreg[w].w;
+          acc[1][0] += __uint_as_float(x & 0x3fffffu); }
+#else
 #pragma unroll
-            for (int u = 0; u < 2; ++u) {
-                int pg = (tile * kTileTok + 16 * u) / P;
-                pg = pg < npages ? pg : npages - 1;
-                pid[u] = indices[ip0 + pg];
-            }
-        };
-        auto subtile_base = [&](int tile, int u) -> size_t {
-            const int tok = tile * kTileTok + 16 * u;
-            const int slot0 = (tok / P < npages) ? tok % P : 0;
-            return ((size_t)pid[u] * a.stride_page + (size_t)slot0 * a.stride_n) * 2 + head_bytes;
-        };
-
-        uint4 kreg[2][4], vreg[8];
-        auto issue_loads = [&](int tile) {
-            const size_t b0 = subtile_base(tile, 0), b1 = subtile_base(tile, 1);
+        for (int w = 0; w < 8; ++w) {
+            uint4 v = vreg[w];
+            if (ragged && tile_tok0 + 4 * w + j >= tok_end) v = make_uint4(0, 0, 0, 0); // 0 * garbage must be 0
+            *reinterpret_cast<uint4*>(v_lds + (4 * w + j) * kVRowBytes + n * 16) = v;
+        }
+#endif
+        uint4 kcur[2][4];
 #pragma unroll
-            for (int ks = 0; ks < 4; ++ks) {
-                kreg[0][ks] = *reinterpret_cast<const uint4*>(k_data + b0 + (size_t)n * row_bytes + ks * 64 + j * 16);
-                kreg[1][ks] = *reinterpret_cast<const uint4*>(k_data + b1 + (size_t)n * row_bytes + ks * 64 + j * 16);
-            }
+        for (int u = 0; u < 2; ++u)
 #pragma unroll
-            for (int w = 0; w < 8; ++w) { // rows 4w..4w+3 of the tile, 16 lanes x 16 B per row
-                const int row = 4 * w + j;
-                const size_t bb = (row < 16) ? b0 : b1;
-                vreg[w] = *reinterpret_cast<const uint4*>(v_data + bb + (size_t)(row & 15) * row_bytes + n * 16);
-            }
-        };
-
-        load_pids(pc.tile_begin);
-        issue_loads(pc.tile_begin);
-        load_pids(pc.tile_begin + 1);
-        for (int t = pc.tile_begin; t < pc.tile_end; ++t) {
-            const int tile_tok0 = t * kTileTok;
-            const bool ragged = tile_tok0 + kTileTok > tok_end; // wave-uniform
-            __syncthreads(); // transposed reads of the previous tile are done before V is overwritten
-#pragma unroll
-            for (int w = 0; w < 8; ++w) {
-                uint4 v = vreg[w];
-                if (ragged && tile_tok0 + 4 * w + j >= tok_end) v = make_uint4(0, 0, 0, 0); // 0 * garbage must be 0
-                *reinterpret_cast<uint4*>(v_lds + (4 * w + j) * kVRowBytes + n * 16) = v;
-            }
-            uint4 kcur[2][4];
+            for (int ks = 0; ks < 4; ++ks) kcur[u][ks] = kreg[u][ks];
+        if (g + 1 < g_end) {
+            if (i + 1 == 32) { chunk_base += 32; buf ^= 1; }
+            un = read_info(buf, (g + 1) - chunk_base);
+#if !(defined(BZ_EXP) && BZ_EXP == 4)
+            if (un.flags & 1) issue_q(un); // next tile opens a new piece
+#endif
+            issue_loads(un);
+        }
+#if defined(BZ_EXP) && (BZ_EXP == 1 || BZ_EXP == 2 || BZ_EXP == 4)
+        { // experiment: loads only
+            uint32_t x = 0;
 #pragma unroll
             for (int u = 0; u < 2; ++u)
 #pragma unroll
-                for (int ks = 0; ks < 4; ++ks) kcur[u][ks] = kreg[u][ks];
-            if (t + 1 < pc.tile_end) {
-                issue_loads(t + 1);
-                load_pids(t + 2);
-            }
-
-            // ---- scores: S^T[token][head], lane (head n, group j) gets tokens 16u + 4j + r
-            f32x4_t s[2];
+                for (int ks = 0; ks < 4; ++ks) x ^= kcur[u][ks].x ^ kcur[u][ks].y ^ kcur[u][ks].z ^ kcur[u][ks].w;
+            acc[0][0] += __uint_as_float(x & 0x3fffffu);
+            l_run = 1.f; m_run = 0.f;
+        }
+#else
+        // ---- scores: S^T[token][head], lane (head n, group j) gets tokens 16u + 4j + r
+        f32x4_t s[2];
 #pragma unroll
-            for (int u = 0; u < 2; ++u) {
-                s[u] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+        for (int u = 0; u < 2; ++u) {
+            s[u] = f32x4_t{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-                for (int ks = 0; ks < 4; ++ks) s[u] = M::run(kcur[u][ks], qhi[ks], s[u]);
-                if (ROPE_Q) {
+            for (int ks = 0; ks < 4; ++ks) s[u] = M::run(kcur[u][ks], qhi[ks], s[u]);
+            if (ROPE_Q) {
 #pragma unroll
-                    for (int ks = 0; ks < 4; ++ks) s[u] = M::run(kcur[u][ks], qlo[ks], s[u]);
-                }
-            }
-            float tmax = -INFINITY;
-#pragma unroll
-            for (int u = 0; u < 2; ++u)
-#pragma unroll
-                for (int r = 0; r < 4; ++r) {
-                    float v = s[u][r] * a.sm_scale_log2;
-                    if (ragged && tile_tok0 + 16 * u + 4 * j + r >= tok_end) v = -INFINITY;
-                    s[u][r] = v;
-                    tmax = fmaxf(tmax, v);
-                }
-            tmax = fmaxf(tmax, __shfl_xor(tmax, 16, 64));
-            tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
-            const float m_new = fmaxf(m_run, tmax);      // finite: every tile holds at least one live token
-            const float alpha = exp2f(m_run - m_new);    // 0 on the first tile (m_run = -inf)
-            // The probabilities enter the second contraction as a storage-precision head plus tail
-            // (p = hi + lo, two MFMAs per block): the matrix cores cost nothing here and the result
-            // keeps fp32-level accuracy instead of the 8 to 11 bits of a single rounded operand.
-            float psum = 0.f;
-            uint4 pa, pb;
-#pragma unroll
-            for (int u = 0; u < 2; ++u) {
-                const float p0 = exp2f(s[u][0] - m_new), p1 = exp2f(s[u][1] - m_new);
-                const float p2 = exp2f(s[u][2] - m_new), p3 = exp2f(s[u][3] - m_new);
-                psum += (p0 + p1) + (p2 + p3);
-                const uint32_t h01 = M::pack2(p0, p1), h23 = M::pack2(p2, p3);
-                u4(pa, 2 * u) = h01;
-                u4(pa, 2 * u + 1) = h23;
-                u4(pb, 2 * u) = M::pack2(p0 - M::unpack_lo(h01), p1 - M::unpack_hi(h01));
-                u4(pb, 2 * u + 1) = M::pack2(p2 - M::unpack_lo(h23), p3 - M::unpack_hi(h23));
-            }
-            psum += __shfl_xor(psum, 16, 64);
-            psum += __shfl_xor(psum, 32, 64);
-            l_run = l_run * alpha + psum;
-            m_run = m_new;
-
-            // ---- rescale the output rows (head 4j+i lives in lane 4j+i of the score layout)
-            if (__any(alpha != 1.0f)) {
-#pragma unroll
-                for (int i = 0; i < 4; ++i) {
-                    const float al = __shfl(alpha, 4 * j + i, 64);
-#pragma unroll
-                    for (int d = 0; d < 8; ++d) acc[d][i] *= al;
-                }
-            }
-            __syncthreads(); // V tile visible to every lane
-            // ---- O[head][d] += P[head][tok] V[tok][d], eight 16-wide d blocks
-#pragma unroll
-            for (int d = 0; d < 8; ++d) {
-                uint4 vb;
-#pragma unroll
-                for (int u = 0; u < 2; ++u) {
-                    const unsigned char* src =
-                        v_lds + (16 * u + 4 * j + (n >> 2)) * kVRowBytes + d * 32 + (n & 3) * 8;
-                    const s16x4_t tr = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-                        (s16x4_t __attribute__((address_space(3)))*)(src));
-                    const uint2 w = __builtin_bit_cast(uint2, tr);
-                    u4(vb, 2 * u) = w.x;
-                    u4(vb, 2 * u + 1) = w.y;
-                }
-                acc[d] = M::run(pa, vb, acc[d]);
-                acc[d] = M::run(pb, vb, acc[d]);
+                for (int ks = 0; ks < 4; ++ks) s[u] = M::run(kcur[u][ks], qlo[ks], s[u]);
             }
         }
+        float tmax = -INFINITY;
+#pragma unroll
+        for (int u = 0; u < 2; ++u)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                float v = s[u][r] * a.sm_scale_log2;
+                if (ragged && tile_tok0 + 16 * u + 4 * j + r >= tok_end) v = -INFINITY;
+                s[u][r] = v;
+                tmax = fmaxf(tmax, v);
+            }
+        tmax = fmaxf(tmax, __shfl_xor(tmax, 16, 64));
+        tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
+        const float m_new = fmaxf(m_run, tmax);   // finite: every tile holds at least one live token
+        const float alpha = exp2f(m_run - m_new); // 0 on the first tile (m_run = -inf)
+        // The probabilities enter the second contraction as a storage-precision head plus tail
+        // (p = hi + lo, two MFMAs per block): the matrix cores cost nothing here and the result
+        // keeps fp32-level accuracy instead of the 8 to 11 bits of a single rounded operand.
+        float psum = 0.f;
+        uint4 pa, pb;
+#pragma unroll
+        for (int u = 0; u < 2; ++u) {
+            const float p0 = exp2f(s[u][0] - m_new), p1 = exp2f(s[u][1] - m_new);
+            const float p2 = exp2f(s[u][2] - m_new), p3 = exp2f(s[u][3] - m_new);
+            psum += (p0 + p1) + (p2 + p3);
+            const uint32_t h01 = M::pack2(p0, p1), h23 = M::pack2(p2, p3);
+            u4(pa, 2 * u) = h01;
+            u4(pa, 2 * u + 1) = h23;
+            u4(pb, 2 * u) = M::pack2(p0 - M::unpack_lo(h01), p1 - M::unpack_hi(h01));
+            u4(pb, 2 * u + 1) = M::pack2(p2 - M::unpack_lo(h23), p3 - M::unpack_hi(h23));
+        }
+        psum += __shfl_xor(psum, 16, 64);
+        psum += __shfl_xor(psum, 32, 64);
+        l_run = l_run * alpha + psum;
+        m_run = m_new;
 
-        // ---- epilogue: normalise and write the final rows, or the split-K partial
-        const float inv_l = l_run > 0.f ? 1.0f / l_run : 0.f;
-        const float lse2 = l_run > 0.f ? m_run + log2f(l_run) : -INFINITY;
+        // ---- rescale the output rows (head 4j+i lives in lane 4j+i of the score layout)
+        if (__any(alpha != 1.0f)) {
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const int head = 4 * j + i;
-            const float il = __shfl(inv_l, head, 64);
-            if (head < G) {
-                const int hq = kvh * G + head;
-                if (pc.partial < 0) {
-                    OT* orow = reinterpret_cast<OT*>(a.out) + ((size_t)b * a.num_qo_heads + hq) * 128;
+            for (int i = 0; i < 4; ++i) {
+                const float al = __shfl(alpha, 4 * j + i, 64);
 #pragma unroll
-                    for (int d = 0; d < 8; ++d) orow[d * 16 + n] = StoreCvt<OT>::from(acc[d][i] * il);
+                for (int d = 0; d < 8; ++d) acc[d][i] *= al;
+            }
+        }
+        wave_lds_sync(); // V tile written before the transposed reads
+        // ---- O[head][d] += P[head][tok] V[tok][d], eight 16-wide d blocks
+#pragma unroll
+        for (int d = 0; d < 8; ++d) {
+            uint4 vb;
+#pragma unroll
+            for (int u = 0; u < 2; ++u) {
+                const unsigned char* src = v_lds + (16 * u + 4 * j + (n >> 2)) * kVRowBytes + d * 32 + (n & 3) * 8;
+                const s16x4_t tr = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+                    (s16x4_t __attribute__((address_space(3)))*)(src));
+                const uint2 w = __builtin_bit_cast(uint2, tr);
+                u4(vb, 2 * u) = w.x;
+                u4(vb, 2 * u + 1) = w.y;
+            }
+            acc[d] = M::run(pa, vb, acc[d]);
+            acc[d] = M::run(pb, vb, acc[d]);
+        }
+#endif
+
+#if defined(BZ_EXP) && BZ_EXP == 4
+        if ((uc.flags & 2) && g + 1 == g_end && acc[0][0] + acc[1][0] == 1.2345f) a.part_lse[0] = acc[0][0];
+        if (false) {
+#else
+        if (uc.flags & 2) { // ================= last tile of a piece: final rows, or the split-K partial
+#endif
+#if defined(BZ_EXP) && BZ_EXP >= 3
+            ++exp_pieces;
+#endif
+            const int b = uc.seq, kvh = uc.kvh, partial = uc.partial;
+            const float inv_l = l_run > 0.f ? 1.0f / l_run : 0.f;
+            const float lse2 = l_run > 0.f ? m_run + log2f(l_run) : -INFINITY;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int head = 4 * j + i;
+                const float il = __shfl(inv_l, head, 64);
+                if (head < G) {
+                    if (partial < 0) {
+                        OT* orow = reinterpret_cast<OT*>(a.out) + ((size_t)b * a.num_qo_heads + kvh * G + head) * 128;
+#pragma unroll
+                        for (int d = 0; d < 8; ++d) orow[d * 16 + n] = StoreCvt<OT>::from(acc[d][i] * il);
+                    } else {
+                        float* prow = a.part_o + ((size_t)partial * 16 + head) * 128;
+#pragma unroll
+                        for (int d = 0; d < 8; ++d) prow[d * 16 + n] = acc[d][i] * il;
+                    }
+                }
+            }
+            if (j == 0 && n < G) {
+                if (partial < 0) {
+                    if (a.lse) a.lse[(size_t)b * a.num_qo_heads + kvh * G + n] = lse2 * 0.6931471805599453f;
                 } else {
-                    float* prow = a.part_o + ((size_t)pc.partial * 16 + head) * 128;
-#pragma unroll
-                    for (int d = 0; d < 8; ++d) prow[d * 16 + n] = acc[d][i] * il;
+                    a.part_lse[(size_t)partial * 16 + n] = lse2;
                 }
-            }
-        }
-        if (j == 0 && n < G) {
-            if (pc.partial < 0) {
-                if (a.lse) a.lse[(size_t)b * a.num_qo_heads + kvh * G + n] = lse2 * 0.6931471805599453f;
-            } else {
-                a.part_lse[(size_t)pc.partial * 16 + n] = lse2;
             }
         }
     }
+#if defined(BZ_EXP) && BZ_EXP >= 3
+    if (lane == 0) {
+        ts_buf[blockIdx.x * 4 + 1] = wall_clock64();
+        unsigned hwid, xcc;
+        asm volatile("s_getreg_b32 %0, hwreg(HW_REG_HW_ID)" : "=s"(hwid));
+        asm volatile("s_getreg_b32 %0, hwreg(HW_REG_XCC_ID)" : "=s"(xcc));
+        ts_buf[blockIdx.x * 4 + 2] = hwid;
+        ts_buf[blockIdx.x * 4 + 3] = (long long)(xcc & 0xf) | ((long long)exp_pieces << 8) | ((long long)(g_end - g_begin) << 20);
+    }
+#endif
 }
 
 // Combine the partials of one split (sequence, kv head): o = sum_i o_i 2^(lse_i - M) / sum_i 2^(lse_i - M).
+// One workgroup of 128 lanes per (split, q head of the group).  The partials are fetched eight at a
+// time with all loads issued before any is used, and merged with a running maximum, so a split with up
+// to eight partials costs two dependent memory round trips (schedule entry, then data).
 template <typename OT>
-__global__ __launch_bounds__(128) void decode_mfma_combine_kernel(const MfmaCombine* combos, const float* part_o,
-                                                                  const float* part_lse, void* out, float* lse,
-                                                                  uint32_t num_qo_heads, uint32_t G) {
+__global__ __launch_bounds__(128) void decode_mfma_combine_kernel(const MfmaCombine* __restrict__ combos,
+                                                                  const float* __restrict__ part_o,
+                                                                  const float* __restrict__ part_lse, void* out,
+                                                                  float* lse, uint32_t num_qo_heads, uint32_t G) {
     const MfmaCombine c = combos[blockIdx.x];
     const uint32_t g = blockIdx.y, d = threadIdx.x;
-    float M = -INFINITY;
-    for (int i = 0; i < c.count; ++i) M = fmaxf(M, part_lse[(size_t)(c.first + i) * 16 + g]);
-    float wsum = 0.f, o = 0.f;
-    for (int i = 0; i < c.count; ++i) {
-        const float li = part_lse[(size_t)(c.first + i) * 16 + g];
-        const float w = (li == -INFINITY) ? 0.f : exp2f(li - M);
-        wsum += w;
-        o += w * part_o[((size_t)(c.first + i) * 16 + g) * 128 + d];
+    float M = -INFINITY, wsum = 0.f, o = 0.f;
+    for (int i0 = 0; i0 < c.count; i0 += 8) {
+        float li[8], oi[8];
+#pragma unroll
+        for (int k = 0; k < 8; ++k) {
+            const bool live = i0 + k < c.count;
+            const size_t slot = (size_t)(c.first + (live ? i0 + k : 0));
+            li[k] = live ? part_lse[slot * 16 + g] : -INFINITY;
+            oi[k] = live ? part_o[(slot * 16 + g) * 128 + d] : 0.f;
+        }
+        float m2 = M;
+#pragma unroll
+        for (int k = 0; k < 8; ++k) m2 = fmaxf(m2, li[k]);
+        if (m2 == -INFINITY) continue;
+        const float sc = exp2f(M - m2); // 0 while nothing has been merged yet
+        wsum *= sc;
+        o *= sc;
+#pragma unroll
+        for (int k = 0; k < 8; ++k) {
+            const float w = exp2f(li[k] - m2); // -inf -> 0
+            wsum += w;
+            o += w * oi[k];
+        }
+        M = m2;
     }
     o = wsum > 0.f ? o / wsum : 0.f;
     const size_t hq = (size_t)c.seq * num_qo_heads + (size_t)c.kvh * G + g;
@@ -337,16 +471,16 @@ __global__ __launch_bounds__(128) void decode_mfma_combine_kernel(const MfmaComb
 
 struct DecodeArgs; // general-kernel argument block (bz_decode.hip); only its scalar fields are forwarded here
 
+template <bool BF16, typename OT, bool ROPE_Q>
+static void launch_mfma_k(const DecodePlan* p, const MfmaDecodeArgs& a, hipStream_t s) {
+    hipLaunchKernelGGL((decode_mfma_kernel<BF16, OT, ROPE_Q>), dim3(p->mfma_slots), dim3(64), 0, s, a,
+                       (const char*)a.q, a.k_data, a.v_data, a.indices, a.pieces, a.tiles, a.tile_ptr);
+}
+
 template <bool BF16, typename OT>
 static int launch_mfma(const DecodePlan* p, const MfmaDecodeArgs& a, hipStream_t s) {
-    if (a.rope_q)
-        hipLaunchKernelGGL((decode_mfma_kernel<BF16, OT, true>), dim3(p->mfma_slots), dim3(64), 0, s, a,
-                           (const char*)a.q, a.k_data, a.v_data, a.indices, a.indptr, a.last_page_len, a.pieces,
-                           a.piece_ptr);
-    else
-        hipLaunchKernelGGL((decode_mfma_kernel<BF16, OT, false>), dim3(p->mfma_slots), dim3(64), 0, s, a,
-                           (const char*)a.q, a.k_data, a.v_data, a.indices, a.indptr, a.last_page_len, a.pieces,
-                           a.piece_ptr);
+    if (a.rope_q) launch_mfma_k<BF16, OT, true>(p, a, s);
+    else launch_mfma_k<BF16, OT, false>(p, a, s);
     BZ_LAUNCH_CHECK();
     if (p->mfma_combos > 0) {
         hipLaunchKernelGGL((decode_mfma_combine_kernel<OT>), dim3(p->mfma_combos, a.group), dim3(128), 0, s,
@@ -367,7 +501,7 @@ int decode_fast_path(const DecodePlan* p, const void* q, void* out, float* lse, 
     a.q = q; a.out = out; a.lse = lse;
     a.k_data = (const char*)kv->k_data; a.v_data = (const char*)kv->v_data;
     a.indices = kv->indices; a.indptr = kv->indptr; a.last_page_len = kv->last_page_len;
-    a.pieces = p->mfma_pieces_d; a.piece_ptr = p->mfma_piece_ptr_d;
+    a.pieces = p->mfma_pieces_d; a.tiles = p->mfma_tiles_d; a.tile_ptr = p->mfma_tile_ptr_d;
     a.part_o = p->mfma_part_o; a.part_lse = p->mfma_part_lse;
     a.stride_page = kv->stride_page; a.stride_n = kv->stride_n; a.stride_h = kv->stride_h;
     a.page_size = kv->page_size; a.num_qo_heads = num_qo_heads; a.group = num_qo_heads / kv->num_kv_heads;

@@ -101,12 +101,15 @@ extern "C" int bz_decode_plan(bz_decode_plan_t* plan_, void* float_buffer, size_
         return (x.page_end - x.page_begin) > (y.page_end - y.page_begin);
     });
 
-    // ---- MFMA path schedule: equal shares of the flattened (sequence, kv head, tile) space ------
-    // Every wave slot of the chip (8 single-wave workgroups per CU) gets the same number of 32-token
-    // tiles; a share that crosses a (sequence, kv head) boundary becomes several pieces, and a
-    // (sequence, kv head) that is cut, or longer than split_tokens, is combined from partials.
+    // ---- MFMA path schedule ---------------------------------------------------------------------
+    // The flattened (sequence, kv head, 32-token tile) space is divided into equal shares, one per
+    // wave slot of the chip (8 single-wave workgroups per CU).  A share that crosses a (sequence, kv
+    // head) boundary becomes several pieces; a (sequence, kv head) that ends up in more than one
+    // piece, or is longer than split_tokens, is folded from partial results.  Every tile of a share
+    // gets a 16-byte record so that the kernel never has to chase the piece list tile by tile.
     std::vector<MfmaPiece> mp;
-    std::vector<int32_t> mptr;
+    std::vector<MfmaTile> mt;
+    std::vector<int32_t> mptr; // tiles of slot s: [mptr[s], mptr[s+1])
     std::vector<MfmaCombine> mc;
     uint32_t mfma_partials = 0;
     const uint32_t group = num_qo_heads / num_kv_heads;
@@ -122,7 +125,25 @@ extern "C" int bz_decode_plan(bz_decode_plan_t* plan_, void* float_buffer, size_
         const uint64_t max_slots = (uint64_t)cus * 8;
         const uint64_t share = std::max<uint64_t>(1, (total_tiles + max_slots - 1) / max_slots);
         const uint32_t cap_tiles = never_split ? 0x7fffffffu : std::max<uint32_t>(1, split_tokens / 32);
-        uint64_t room = share; // tiles the current slot can still take
+        // Workgroups are dealt round-robin to the 8 XCDs, and on MI355X the odd XCDs stream HBM about
+        // a tenth slower than the even ones under full load (measured per wave with wall_clock64), so
+        // the slots that land on them get a smaller share.  BZ_DECODE_XCD_SKEW overrides the percentage.
+        double skew = 0.09;
+        if (const char* e = getenv("BZ_DECODE_XCD_SKEW")) skew = atof(e) / 100.0;
+        if (share < 8) skew = 0.0; // too few tiles per slot to express the difference
+        const uint64_t nslots = std::min<uint64_t>(max_slots, (total_tiles + share - 1) / share);
+        auto slot_weight = [&](uint64_t s) { return (s & 1) ? 1.0 - skew / 2 : 1.0 + skew / 2; };
+        double wsum = 0.0;
+        for (uint64_t s2 = 0; s2 < nslots; ++s2) wsum += slot_weight(s2);
+        uint64_t slot = 0;
+        double wacc = slot_weight(0);
+        auto slot_share = [&](void) { // tiles of the current slot: difference of rounded running boundaries
+            const uint64_t hi = (slot + 1 >= nslots) ? total_tiles : (uint64_t)((double)total_tiles * wacc / wsum + 0.5);
+            const uint64_t lo = (uint64_t)((double)total_tiles * (wacc - slot_weight(slot)) / wsum + 0.5);
+            return std::max<uint64_t>(1, hi > lo ? hi - lo : 1);
+        };
+        uint64_t room = slot_share(); // tiles the current slot can still take
+        mt.reserve(total_tiles);
         mptr.push_back(0);
         for (uint32_t b = 0; b < batch_size; ++b) {
             const int32_t np = indptr_h[b + 1] - indptr_h[b];
@@ -133,21 +154,40 @@ extern "C" int bz_decode_plan(bz_decode_plan_t* plan_, void* float_buffer, size_
                 const size_t first_piece = mp.size();
                 int32_t t = 0;
                 while (t < tiles) {
-                    if (room == 0) { mptr.push_back((int32_t)mp.size()); room = share; }
-                    const int32_t take = (int32_t)std::min<uint64_t>({(uint64_t)(tiles - t), never_split ? (uint64_t)(tiles - t) : room, cap_tiles});
-                    mp.push_back({(int32_t)b, (int32_t)h, t, t + take, -1, {0, 0, 0}});
+                    if (room == 0) {
+                        mptr.push_back((int32_t)mt.size());
+                        ++slot;
+                        wacc += slot_weight(slot);
+                        room = slot_share();
+                    }
+                    const uint64_t left = (uint64_t)(tiles - t);
+                    const int32_t take = never_split ? (int32_t)left
+                                                     : (int32_t)std::min<uint64_t>({left, room, (uint64_t)cap_tiles});
+                    room -= std::min<uint64_t>(room, (uint64_t)take);
+                    for (int32_t tt = t; tt < t + take; ++tt) {
+                        const int32_t pg0 = std::min<int32_t>((int32_t)(((int64_t)tt * 32) / page_size), np - 1);
+                        const int32_t pg1 = std::min<int32_t>((int32_t)(((int64_t)tt * 32 + 16) / page_size), np - 1);
+                        mt.push_back({indptr_h[b] + pg0, indptr_h[b] + pg1, tt, (int32_t)mp.size()});
+                    }
+                    mp.push_back({(int32_t)b, (int32_t)h, t, t + take, -1, -1, 0, 0, indptr_h[b], np, (int32_t)len,
+                                  {0, 0, 0, 0, 0}});
                     t += take;
-                    room = (never_split && room < (uint64_t)take) ? 0 : room - std::min<uint64_t>(room, take);
                 }
                 const size_t cnt = mp.size() - first_piece;
                 if (cnt > 1) {
                     mc.push_back({(int32_t)b, (int32_t)h, (int32_t)mfma_partials, (int32_t)cnt});
-                    for (size_t i = 0; i < cnt; ++i) mp[first_piece + i].partial = (int32_t)(mfma_partials + i);
+                    for (size_t i = 0; i < cnt; ++i) {
+                        MfmaPiece& pc = mp[first_piece + i];
+                        pc.partial = (int32_t)(mfma_partials + i);
+                        pc.combo = (int32_t)mc.size() - 1;
+                        pc.count = (int32_t)cnt;
+                        pc.first = (int32_t)mfma_partials;
+                    }
                     mfma_partials += (uint32_t)cnt;
                 }
             }
         }
-        mptr.push_back((int32_t)mp.size());
+        mptr.push_back((int32_t)mt.size());
     }
 
     // ---- workspaces -------------------------------------------------------------------------
@@ -163,11 +203,12 @@ extern "C" int bz_decode_plan(bz_decode_plan_t* plan_, void* float_buffer, size_
     const size_t mp_bytes = align_up(mp.size() * sizeof(MfmaPiece), 256);
     const size_t mptr_bytes = align_up(mptr.size() * sizeof(int32_t), 256);
     const size_t mc_bytes = align_up(mc.size() * sizeof(MfmaCombine), 256);
+    const size_t cnt_bytes = align_up(mt.size() * sizeof(MfmaTile), 256); // tile records
     const size_t mpart_o_bytes = align_up((size_t)mfma_partials * 16 * 128 * sizeof(float), 256);
     const size_t mpart_lse_bytes = align_up((size_t)mfma_partials * 16 * sizeof(float), 256);
-    const bool mfma_ok = mfma_shape && !mp.empty() && base_total + mp_bytes + mptr_bytes + mc_bytes <= int_buffer_bytes &&
+    const bool mfma_ok = mfma_shape && !mp.empty() && base_total + mp_bytes + mptr_bytes + mc_bytes + cnt_bytes <= int_buffer_bytes &&
                          mpart_o_bytes + mpart_lse_bytes <= float_buffer_bytes;
-    const size_t total = mfma_ok ? base_total + mp_bytes + mptr_bytes + mc_bytes : base_total;
+    const size_t total = mfma_ok ? base_total + mp_bytes + mptr_bytes + mc_bytes + cnt_bytes : base_total;
 
     hipStream_t s = (hipStream_t)stream;
     if (!p->upload_done) BZ_CHECK_HIP(hipEventCreateWithFlags(&p->upload_done, hipEventDisableTiming));
@@ -189,6 +230,7 @@ extern "C" int bz_decode_plan(bz_decode_plan_t* plan_, void* float_buffer, size_
         memcpy(st + base_total, mp.data(), mp.size() * sizeof(MfmaPiece));
         memcpy(st + base_total + mp_bytes, mptr.data(), mptr.size() * sizeof(int32_t));
         if (!mc.empty()) memcpy(st + base_total + mp_bytes + mptr_bytes, mc.data(), mc.size() * sizeof(MfmaCombine));
+        memcpy(st + base_total + mp_bytes + mptr_bytes + mc_bytes, mt.data(), mt.size() * sizeof(MfmaTile));
     }
     if (total) BZ_CHECK_HIP(hipMemcpyAsync(int_buffer, st, total, hipMemcpyHostToDevice, s));
     BZ_CHECK_HIP(hipEventRecord(p->upload_done, s));
@@ -208,6 +250,8 @@ extern "C" int bz_decode_plan(bz_decode_plan_t* plan_, void* float_buffer, size_
         p->mfma_pieces_d = (const MfmaPiece*)((char*)int_buffer + base_total);
         p->mfma_piece_ptr_d = (const int32_t*)((char*)int_buffer + base_total + mp_bytes);
         p->mfma_combos_d = (const MfmaCombine*)((char*)int_buffer + base_total + mp_bytes + mptr_bytes);
+        p->mfma_tiles_d = (const MfmaTile*)((char*)int_buffer + base_total + mp_bytes + mptr_bytes + mc_bytes);
+        p->mfma_tile_ptr_d = p->mfma_piece_ptr_d;
         p->mfma_part_o = (float*)float_buffer; // the two paths never run in the same call: same workspace
         p->mfma_part_lse = (float*)((char*)float_buffer + mpart_o_bytes);
         p->mfma_slots = (uint32_t)mptr.size() - 1;
@@ -223,6 +267,7 @@ extern "C" int bz_decode_plan(bz_decode_plan_t* plan_, void* float_buffer, size_
     // both kernels cover)
     const char* path = getenv("BZ_DECODE_PATH");
     p->force_general = path && !strcmp(path, "general");
+
     p->planned = true;
     return 0;
 }

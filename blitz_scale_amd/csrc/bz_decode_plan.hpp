@@ -25,7 +25,16 @@ struct MfmaPiece {
     int32_t seq, kvh;
     int32_t tile_begin, tile_end; // in 32-token tiles from the start of the sequence
     int32_t partial;              // -1: whole (sequence, kv head) -> final rows; else partial slot
-    int32_t pad[3];
+    int32_t combo, count, first;  // split (sequence, kv head): its index, number of partials, first slot
+    int32_t ip0, npages, seq_len; // indptr[seq], pages and tokens of the sequence (from the host table)
+    int32_t pad[5];
+};
+
+// One 32-token tile of a wave slot's share, in processing order.
+struct MfmaTile {
+    int32_t idx0, idx1; // positions in indices[] of the pages of the two 16-token subtiles (kept in range)
+    int32_t t;          // tile number inside its sequence
+    int32_t piece;      // index into the piece array
 };
 
 // One split (sequence, kv head): partial slots [first, first+count).
@@ -51,6 +60,8 @@ struct DecodePlan {
     const MfmaPiece* mfma_pieces_d = nullptr;
     const int32_t* mfma_piece_ptr_d = nullptr;
     const MfmaCombine* mfma_combos_d = nullptr;
+    const MfmaTile* mfma_tiles_d = nullptr;
+    const int32_t* mfma_tile_ptr_d = nullptr; // tiles of slot s: [tile_ptr[s], tile_ptr[s+1])
     float* mfma_part_o = nullptr;
     float* mfma_part_lse = nullptr;
     // pinned staging for the schedule upload and the event that guards its reuse
