@@ -1,24 +1,453 @@
-// Ragged causal prefill attention for gfx950.
+// Ragged (causal) prefill self-attention on the gfx950 matrix cores: replaces
+// src/kernel/attention_prefill.cu and the prefill half of flashinfer_types.cu of the BlitzScale
+// worker.  head_dim 128, f16 or bf16, any number of q heads per kv head.
+//
+// One workgroup of 4 waves takes 128 consecutive q rows of one (request, q head); wave w owns rows
+// 32w..32w+31.  K/V tiles of 64 tokens are staged through double-buffered LDS and shared by the four
+// waves.  Both contractions are issued "transposed" on v_mfma_f32_32x32x16:
+//     S^T[kv][q] = K[kv][:] . Q[q][:]      (A = K tile from LDS,      B = Q rows from registers)
+//     O^T[d][q]  = V^T[d][kv] . P^T[kv][q] (A = V tile, transposed LDS read, B = P from registers)
+// so that in both results a lane's column index is its own q row: the softmax statistics, the
+// rescaling of O and the P operand of the second contraction are all lane-local (one shuffle per
+// tile joins the two half-waves).
+#include <algorithm>
+#include <cmath>
+#include <cstring>
 #include <new>
+#include <vector>
+
 #include "bz_common.hpp"
 
 namespace bz {
+
+typedef __attribute__((ext_vector_type(8))) __bf16 pf_bf16x8;
+typedef __attribute__((ext_vector_type(8))) _Float16 pf_f16x8;
+typedef __attribute__((ext_vector_type(2))) __bf16 pf_bf16x2;
+typedef __attribute__((ext_vector_type(2))) _Float16 pf_f16x2;
+typedef __attribute__((ext_vector_type(2))) float pf_f32x2;
+typedef __attribute__((ext_vector_type(16))) float pf_f32x16;
+typedef __attribute__((ext_vector_type(4))) short pf_s16x4;
+
+constexpr int kBM = 128;       // q rows per workgroup
+constexpr int kBN = 64;        // kv tokens per tile
+constexpr int kKRow = 272;     // LDS row stride of the K tile (256 B + 16: 16 rows cover all banks)
+constexpr int kVRow = 320;     // LDS row stride of the V tile (256 B + 64: 4 rows x 64 B cover all banks)
+constexpr int kKTile = kBN * kKRow;
+constexpr int kVTile = kBN * kVRow;
+
+struct PrefillItem {
+    int32_t tok0; // global index of the request's first token
+    int32_t len;  // tokens in the request
+    int32_t q0;   // first q row of this tile, relative to the request
+    int32_t pad;
+};
+
 struct PrefillPlan {
     bool planned = false;
-    uint32_t batch_size = 0, num_qo_heads = 0, num_kv_heads = 0, head_dim = 0;
+    uint32_t batch_size = 0, num_qo_heads = 0, num_kv_heads = 0, head_dim = 0, num_items = 0;
+    uint32_t total_tokens = 0;
+    const PrefillItem* items_d = nullptr;
+    void* staging = nullptr;
+    size_t staging_bytes = 0;
+    hipEvent_t upload_done = nullptr;
 };
+
+struct PrefillArgs {
+    void* out;
+    const PrefillItem* items;
+    uint32_t num_qo_heads, num_kv_heads;
+    int causal;
+    float sm_scale_log2;
+};
+
+template <bool BF16> struct PfMma;
+template <> struct PfMma<false> {
+    __device__ static __forceinline__ pf_f32x16 run(uint4 a, uint4 b, pf_f32x16 c) {
+        return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(pf_f16x8, a), __builtin_bit_cast(pf_f16x8, b), c,
+                                                      0, 0, 0);
+    }
+    __device__ static __forceinline__ uint32_t pack2(float lo, float hi) {
+        const pf_f16x2 h = __builtin_convertvector(pf_f32x2{lo, hi}, pf_f16x2);
+        return __builtin_bit_cast(uint32_t, h);
+    }
+    __device__ static __forceinline__ float lo(uint32_t w) { return (float)__builtin_bit_cast(pf_f16x2, w)[0]; }
+    __device__ static __forceinline__ float hi(uint32_t w) { return (float)__builtin_bit_cast(pf_f16x2, w)[1]; }
+};
+template <> struct PfMma<true> {
+    __device__ static __forceinline__ pf_f32x16 run(uint4 a, uint4 b, pf_f32x16 c) {
+        return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(pf_bf16x8, a), __builtin_bit_cast(pf_bf16x8, b),
+                                                       c, 0, 0, 0);
+    }
+    __device__ static __forceinline__ uint32_t pack2(float lo, float hi) {
+        return (uint32_t)f32_to_bf16_bits(lo) | ((uint32_t)f32_to_bf16_bits(hi) << 16);
+    }
+    __device__ static __forceinline__ float lo(uint32_t w) { return __uint_as_float(w << 16); }
+    __device__ static __forceinline__ float hi(uint32_t w) { return __uint_as_float(w & 0xffff0000u); }
+};
+
+__device__ __forceinline__ uint32_t& pf_u4(uint4& v, int i) { return reinterpret_cast<uint32_t*>(&v)[i]; }
+
+// SPLIT_P: the probabilities enter the second contraction as head + tail of the storage type (two
+// MFMAs), used for bf16 whose 8-bit significand alone would eat the error budget.
+template <bool BF16, bool SPLIT_P>
+__global__ __launch_bounds__(256, 2) void prefill_kernel(PrefillArgs a, const char* __restrict__ q_ptr,
+                                                         const char* __restrict__ k_ptr,
+                                                         const char* __restrict__ v_ptr) {
+    using M = PfMma<BF16>;
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+    unsigned char* k_lds = smem;              // [2][kKTile]
+    unsigned char* v_lds = smem + 2 * kKTile; // [2][kVTile]
+
+    const PrefillItem it = a.items[blockIdx.x];
+    const int head = blockIdx.y;
+    const int Hq = (int)a.num_qo_heads, Hkv = (int)a.num_kv_heads;
+    const int kvh = head / (Hq / Hkv);
+    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+    const int qn = lane & 31; // q row of this lane inside the wave's 32 rows
+    const int h = lane >> 5;  // half-wave: which 8 of the 16 contraction indices of an MFMA step
+    const int L = it.len;
+    const int q_pos = it.q0 + 32 * wave + qn; // position inside the request (may be >= L: masked at the end)
+    const int wave_q_lo = it.q0 + 32 * wave, wave_q_hi = wave_q_lo + 31;
+
+    // ---- Q rows as B operands: lane (q, h) holds q[q][16*ks + 8*h .. +7], ks = 0..7
+    uint4 qreg[8];
+    {
+        const size_t qtok = (size_t)it.tok0 + (size_t)min(q_pos, L - 1);
+        const char* qrow = q_ptr + (qtok * Hq + head) * 256;
+#pragma unroll
+        for (int ks = 0; ks < 8; ++ks) qreg[ks] = *reinterpret_cast<const uint4*>(qrow + ks * 32 + h * 16);
+    }
+
+    const int kv_limit = a.causal ? min(L, it.q0 + kBM) : L; // tokens any row of this workgroup can see
+    const int n_tiles = (kv_limit + kBN - 1) / kBN;
+
+    // ---- global -> register -> LDS staging of one K/V tile: thread i moves 16 B of rows i/16 + 16*r,
+    // r = 0..3.  Rows past the end of the request re-read its last row (valid memory; masked later).
+    uint4 kg0, kg1, kg2, kg3, vg0, vg1, vg2, vg3;
+    const int st_row = tid >> 4, st_col = (tid & 15) * 16;
+#define BZ_PF_LOAD_ROW(t_, r_, kreg_, vreg_)                                                              \
+    {                                                                                                     \
+        const size_t tok = (size_t)it.tok0 + (size_t)min((t_) * kBN + st_row + 16 * (r_), L - 1);          \
+        const size_t off = (tok * Hkv + kvh) * 256 + (size_t)st_col;                                       \
+        kreg_ = *reinterpret_cast<const uint4*>(k_ptr + off);                                              \
+        vreg_ = *reinterpret_cast<const uint4*>(v_ptr + off);                                              \
+    }
+#define BZ_PF_LOAD_TILE(t_)                                                                               \
+    BZ_PF_LOAD_ROW(t_, 0, kg0, vg0) BZ_PF_LOAD_ROW(t_, 1, kg1, vg1) BZ_PF_LOAD_ROW(t_, 2, kg2, vg2)        \
+    BZ_PF_LOAD_ROW(t_, 3, kg3, vg3)
+#define BZ_PF_STASH_ROW(buf_, r_, kreg_, vreg_)                                                           \
+    *reinterpret_cast<uint4*>(k_lds + (buf_) * kKTile + (st_row + 16 * (r_)) * kKRow + st_col) = kreg_;     \
+    *reinterpret_cast<uint4*>(v_lds + (buf_) * kVTile + (st_row + 16 * (r_)) * kVRow + st_col) = vreg_;
+#define BZ_PF_STASH_TILE(buf_)                                                                            \
+    BZ_PF_STASH_ROW(buf_, 0, kg0, vg0) BZ_PF_STASH_ROW(buf_, 1, kg1, vg1) BZ_PF_STASH_ROW(buf_, 2, kg2, vg2) \
+    BZ_PF_STASH_ROW(buf_, 3, kg3, vg3)
+
+    float m_run = -INFINITY, l_run = 0.f;
+    pf_f32x16 acc[4]; // O^T: block db covers d = 32*db .. +31; element 4b+r is d = 32*db + 8b + 4h + r
+#pragma unroll
+    for (int db = 0; db < 4; ++db)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) acc[db][i] = 0.f;
+
+    BZ_PF_LOAD_TILE(0)
+    BZ_PF_STASH_TILE(0)
+    __syncthreads();
+
+    for (int t = 0; t < n_tiles; ++t) {
+        const int buf = t & 1;
+        const int kv0 = t * kBN;
+        if (t + 1 < n_tiles) { BZ_PF_LOAD_TILE(t + 1) }
+
+        const bool skip = a.causal && kv0 > wave_q_hi; // nothing in this tile is visible to the wave's rows
+        if (!skip) {
+            // ---- S^T = K Q^T: two 32-token blocks, eight 16-wide steps over d
+            pf_f32x16 s[2];
+#pragma unroll
+            for (int kb = 0; kb < 2; ++kb) {
+#pragma unroll
+                for (int i = 0; i < 16; ++i) s[kb][i] = 0.f;
+                const unsigned char* krow = k_lds + buf * kKTile + (32 * kb + qn) * kKRow + h * 16;
+#pragma unroll
+                for (int ks = 0; ks < 8; ++ks) {
+                    const uint4 ka = *reinterpret_cast<const uint4*>(krow + ks * 32);
+                    s[kb] = M::run(ka, qreg[ks], s[kb]);
+                }
+            }
+            // ---- scale, mask, online softmax.  Element 4b+r of block kb is token kv0 + 32kb + 8b + 4h + r.
+            const bool need_mask = (a.causal && kv0 + kBN - 1 > wave_q_lo) || (kv0 + kBN > L);
+            float tmax = -INFINITY;
+#pragma unroll
+            for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+                for (int i = 0; i < 16; ++i) {
+                    float v = s[kb][i] * a.sm_scale_log2;
+                    if (need_mask) {
+                        const int kv = kv0 + 32 * kb + 8 * (i >> 2) + 4 * h + (i & 3);
+                        if (kv >= L || (a.causal && kv > q_pos)) v = -INFINITY;
+                    }
+                    s[kb][i] = v;
+                    tmax = fmaxf(tmax, v);
+                }
+            tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
+            const float m_new = fmaxf(m_run, tmax); // finite from the first tile on: token 0 is visible to every row
+            const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
+            float psum = 0.f;
+            uint4 pa[4], pb[4]; // P^T operands of the four 16-token steps (head, and tail when SPLIT_P)
+#pragma unroll
+            for (int st = 0; st < 4; ++st) {
+                const int kb = st >> 1, b0 = 2 * (st & 1);
+#pragma unroll
+                for (int w = 0; w < 4; ++w) { // elements e = 2w, 2w+1 of the operand: block b0 + e/4, r = e%4
+                    const int i0 = 4 * (b0 + (w >> 1)) + 2 * (w & 1);
+                    const float p0 = __builtin_amdgcn_exp2f(s[kb][i0] - m_new);
+                    const float p1 = __builtin_amdgcn_exp2f(s[kb][i0 + 1] - m_new);
+                    psum += p0 + p1;
+                    const uint32_t hw = M::pack2(p0, p1);
+                    pf_u4(pa[st], w) = hw;
+                    if (SPLIT_P) pf_u4(pb[st], w) = M::pack2(p0 - M::lo(hw), p1 - M::hi(hw));
+                }
+            }
+            psum += __shfl_xor(psum, 32, 64);
+            l_run = l_run * alpha + psum;
+            m_run = m_new;
+#pragma unroll
+            for (int db = 0; db < 4; ++db)
+#pragma unroll
+                for (int i = 0; i < 16; ++i) acc[db][i] *= alpha;
+
+            // ---- O^T += V^T P^T.  A operand through the transposing LDS read: a 16-lane group fetches
+            // 4 token rows x 16 d columns and every lane ends up with the 4 tokens of its own d column.
+            const int grp_d = ((lane >> 4) & 1) * 16; // d columns 0..15 or 16..31 of the block
+            const int srow = (lane & 15) >> 2, scol = (lane & 3) * 4;
+#pragma unroll
+            for (int st = 0; st < 4; ++st) {
+                const unsigned char* vbase = v_lds + buf * kVTile + (16 * st + 4 * h + srow) * kVRow + (grp_d + scol) * 2;
+#pragma unroll
+                for (int db = 0; db < 4; ++db) {
+                    uint4 va;
+                    const pf_s16x4 t0 = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+                        (pf_s16x4 __attribute__((address_space(3)))*)(vbase + db * 64));
+                    const pf_s16x4 t1 = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+                        (pf_s16x4 __attribute__((address_space(3)))*)(vbase + 8 * kVRow + db * 64));
+                    const uint2 w0 = __builtin_bit_cast(uint2, t0), w1 = __builtin_bit_cast(uint2, t1);
+                    va = make_uint4(w0.x, w0.y, w1.x, w1.y);
+                    acc[db] = M::run(va, pa[st], acc[db]);
+                    if (SPLIT_P) acc[db] = M::run(va, pb[st], acc[db]);
+                }
+            }
+        }
+        if (t + 1 < n_tiles) { BZ_PF_STASH_TILE(buf ^ 1) }
+        __syncthreads();
+    }
+
+#undef BZ_PF_LOAD_ROW
+#undef BZ_PF_LOAD_TILE
+#undef BZ_PF_STASH_ROW
+#undef BZ_PF_STASH_TILE
+    // ---- epilogue: normalise, transpose the wave's 32 x 128 block through LDS, store whole rows
+    const float inv_l = l_run > 0.f ? 1.0f / l_run : 0.f;
+    unsigned char* o_lds = smem + wave * (32 * kKRow); // the K buffers are free now (barrier above)
+#pragma unroll
+    for (int db = 0; db < 4; ++db)
+#pragma unroll
+        for (int b = 0; b < 4; ++b) {
+            const uint32_t w0 = M::pack2(acc[db][4 * b] * inv_l, acc[db][4 * b + 1] * inv_l);
+            const uint32_t w1 = M::pack2(acc[db][4 * b + 2] * inv_l, acc[db][4 * b + 3] * inv_l);
+            *reinterpret_cast<uint2*>(o_lds + qn * kKRow + (32 * db + 8 * b + 4 * h) * 2) = make_uint2(w0, w1);
+        }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+#pragma unroll
+    for (int ps = 0; ps < 8; ++ps) {
+        const int row = 4 * ps + (lane >> 4);
+        const int pos = wave_q_lo + row;
+        if (pos < L) {
+            const uint4 v = *reinterpret_cast<const uint4*>(o_lds + row * kKRow + (lane & 15) * 16);
+            char* orow = (char*)a.out + (((size_t)it.tok0 + pos) * Hq + head) * 256;
+            *reinterpret_cast<uint4*>(orow + (lane & 15) * 16) = v;
+        }
+    }
+}
+
+// ---- in-place RoPE of ragged q and k rows (used when the caller asks the attention call itself to rotate)
+struct RopeRaggedArgs {
+    void* q;
+    void* k;
+    const int32_t* indptr;
+    uint32_t batch_size, num_qo_heads, num_kv_heads;
+    RopeFreqs freqs;
+};
+
+template <typename T>
+__global__ __launch_bounds__(256) void rope_ragged_kernel(RopeRaggedArgs a) {
+    __shared__ float s_cos[64], s_sin[64];
+    __shared__ int s_b;
+    const int ntok = a.indptr[a.batch_size];
+    const int tok = blockIdx.x;
+    if (tok >= ntok) return;
+    if (threadIdx.x == 0) {
+        int lo = 0, hi = (int)a.batch_size;
+        while (hi - lo > 1) {
+            const int mid = (lo + hi) / 2;
+            if (a.indptr[mid] <= tok) lo = mid; else hi = mid;
+        }
+        s_b = lo;
+    }
+    __syncthreads();
+    const int pos = tok - a.indptr[s_b];
+    if (threadIdx.x < 64) {
+        float s, c;
+        sincosf((float)pos * a.freqs.f[threadIdx.x], &s, &c);
+        s_cos[threadIdx.x] = c;
+        s_sin[threadIdx.x] = s;
+    }
+    __syncthreads();
+    const int lane8 = threadIdx.x & 7; // 8 lanes per row: 8 low-half and the 8 matching high-half elements each
+    const int rows = (int)(a.num_qo_heads + a.num_kv_heads);
+    for (int r = threadIdx.x >> 3; r < rows; r += 32) {
+        T* row = (r < (int)a.num_qo_heads)
+                     ? reinterpret_cast<T*>(a.q) + ((size_t)tok * a.num_qo_heads + r) * 128
+                     : reinterpret_cast<T*>(a.k) + ((size_t)tok * a.num_kv_heads + (r - a.num_qo_heads)) * 128;
+        Vec8<T> lo, hi;
+        lo.load(row + lane8 * 8);
+        hi.load(row + 64 + lane8 * 8);
+        float x[8], y[8];
+        lo.to_float(x);
+        hi.to_float(y);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            const float c = s_cos[lane8 * 8 + e], s = s_sin[lane8 * 8 + e];
+            const float xr = x[e] * c - y[e] * s, yr = y[e] * c + x[e] * s;
+            x[e] = xr;
+            y[e] = yr;
+        }
+        lo.from_float(x);
+        hi.from_float(y);
+        lo.store(row + lane8 * 8);
+        hi.store(row + 64 + lane8 * 8);
+    }
+}
+
+static inline size_t pf_align_up(size_t x, size_t a) { return (x + a - 1) / a * a; }
+
 } // namespace bz
+
 using namespace bz;
 
 extern "C" bz_prefill_plan_t* bz_prefill_plan_create(void) {
     return reinterpret_cast<bz_prefill_plan_t*>(new (std::nothrow) PrefillPlan());
 }
-extern "C" void bz_prefill_plan_destroy(bz_prefill_plan_t* p) { delete reinterpret_cast<PrefillPlan*>(p); }
-extern "C" int bz_prefill_plan(bz_prefill_plan_t*, void*, size_t, void*, size_t, const int32_t*, const int32_t*,
-                               uint32_t, uint32_t, uint32_t, uint32_t, uint32_t, void*) {
-    return BZ_ERR_UNSUPPORTED;
+
+extern "C" void bz_prefill_plan_destroy(bz_prefill_plan_t* plan_) {
+    PrefillPlan* p = reinterpret_cast<PrefillPlan*>(plan_);
+    if (!p) return;
+    if (p->upload_done) {
+        (void)hipEventSynchronize(p->upload_done);
+        (void)hipEventDestroy(p->upload_done);
+    }
+    if (p->staging) (void)hipHostFree(p->staging);
+    delete p;
 }
-extern "C" int bz_batch_prefill_ragged(bz_prefill_plan_t*, void*, const int32_t*, void*, void*, const int32_t*, void*,
-                                       int, uint32_t, uint32_t, uint32_t, uint32_t, int, int, float, float, void*) {
-    return BZ_ERR_UNSUPPORTED;
+
+extern "C" int bz_prefill_plan(bz_prefill_plan_t* plan_, void* float_buffer, size_t float_buffer_bytes,
+                               void* int_buffer, size_t int_buffer_bytes, const int32_t* qo_indptr_h,
+                               const int32_t* kv_indptr_h, uint32_t batch_size, uint32_t num_qo_heads,
+                               uint32_t num_kv_heads, uint32_t head_dim, uint32_t page_size, void* stream) {
+    (void)float_buffer; (void)float_buffer_bytes; (void)page_size;
+    PrefillPlan* p = reinterpret_cast<PrefillPlan*>(plan_);
+    if (!p || !qo_indptr_h || !kv_indptr_h || !int_buffer) return BZ_ERR_BAD_ARG;
+    if (num_kv_heads == 0 || num_qo_heads % num_kv_heads) return BZ_ERR_BAD_ARG;
+    p->planned = false;
+    if (head_dim != 128) return BZ_ERR_UNSUPPORTED;
+    // self-attention only: the reference passes the same array twice (src/layer/attn.h:175-187)
+    for (uint32_t b = 0; b <= batch_size; ++b)
+        if (qo_indptr_h[b] != kv_indptr_h[b]) return BZ_ERR_UNSUPPORTED;
+    std::vector<PrefillItem> items;
+    for (uint32_t b = 0; b < batch_size; ++b) {
+        const int32_t len = qo_indptr_h[b + 1] - qo_indptr_h[b];
+        if (len < 0) return BZ_ERR_BAD_ARG;
+        for (int32_t q0 = 0; q0 < len; q0 += kBM) items.push_back({qo_indptr_h[b], len, q0, 0});
+    }
+    // longest first: a tile's work grows with the number of tokens its rows can see
+    std::stable_sort(items.begin(), items.end(), [](const PrefillItem& x, const PrefillItem& y) {
+        return std::min(x.len, x.q0 + kBM) > std::min(y.len, y.q0 + kBM);
+    });
+    const size_t bytes = pf_align_up(items.size() * sizeof(PrefillItem), 256);
+    if (bytes > int_buffer_bytes) return BZ_ERR_WORKSPACE;
+    hipStream_t s = (hipStream_t)stream;
+    if (!p->upload_done) BZ_CHECK_HIP(hipEventCreateWithFlags(&p->upload_done, hipEventDisableTiming));
+    else BZ_CHECK_HIP(hipEventSynchronize(p->upload_done));
+    if (bytes > p->staging_bytes) {
+        if (p->staging) BZ_CHECK_HIP(hipHostFree(p->staging));
+        p->staging = nullptr;
+        p->staging_bytes = 0;
+        const size_t want = std::max<size_t>(pf_align_up(bytes * 2, 4096), 1 << 16);
+        BZ_CHECK_HIP(hipHostMalloc(&p->staging, want, hipHostMallocDefault));
+        p->staging_bytes = want;
+    }
+    if (bytes) {
+        memset(p->staging, 0, bytes);
+        memcpy(p->staging, items.data(), items.size() * sizeof(PrefillItem));
+        BZ_CHECK_HIP(hipMemcpyAsync(int_buffer, p->staging, bytes, hipMemcpyHostToDevice, s));
+    }
+    BZ_CHECK_HIP(hipEventRecord(p->upload_done, s));
+    p->items_d = (const PrefillItem*)int_buffer;
+    p->num_items = (uint32_t)items.size();
+    p->batch_size = batch_size; p->num_qo_heads = num_qo_heads; p->num_kv_heads = num_kv_heads;
+    p->head_dim = head_dim;
+    p->total_tokens = (uint32_t)qo_indptr_h[batch_size];
+    p->planned = true;
+    return 0;
+}
+
+template <bool BF16, bool SPLIT_P>
+static int launch_prefill(const PrefillPlan* p, const PrefillArgs& a, const void* q, const void* k, const void* v,
+                          hipStream_t s) {
+    const size_t smem = 2 * (size_t)(kKTile + kVTile);
+    auto kern = prefill_kernel<BF16, SPLIT_P>;
+    static bool attr_done = false; // raising the dynamic LDS limit is idempotent; a repeated call is harmless
+    if (!attr_done) {
+        BZ_CHECK_HIP(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
+        attr_done = true;
+    }
+    hipLaunchKernelGGL(kern, dim3(p->num_items, a.num_qo_heads), dim3(256), smem, s, a, (const char*)q, (const char*)k,
+                       (const char*)v);
+    BZ_LAUNCH_CHECK();
+    return 0;
+}
+
+extern "C" int bz_batch_prefill_ragged(bz_prefill_plan_t* plan_, void* q, const int32_t* qo_indptr, void* k, void* v,
+                                       const int32_t* kv_indptr, void* out, int dtype, uint32_t batch_size,
+                                       uint32_t num_qo_heads, uint32_t num_kv_heads, uint32_t head_dim, int causal,
+                                       int rope_mode, float rope_theta, float sm_scale, void* stream) {
+    PrefillPlan* p = reinterpret_cast<PrefillPlan*>(plan_);
+    if (!p || !q || !k || !v || !out || !qo_indptr || !kv_indptr) return BZ_ERR_BAD_ARG;
+    if (!p->planned) return BZ_ERR_NOT_PLANNED;
+    if (batch_size != p->batch_size || num_qo_heads != p->num_qo_heads || num_kv_heads != p->num_kv_heads ||
+        head_dim != p->head_dim)
+        return BZ_ERR_BAD_ARG;
+    if (dtype != BZ_F16 && dtype != BZ_BF16) return BZ_ERR_UNSUPPORTED;
+    if (rope_mode != BZ_ROPE_NONE && rope_mode != BZ_ROPE_FULL) return BZ_ERR_BAD_ARG;
+    if (((uintptr_t)q | (uintptr_t)k | (uintptr_t)v | (uintptr_t)out) % 16) return BZ_ERR_BAD_ARG;
+    hipStream_t s = (hipStream_t)stream;
+    if (p->num_items == 0) return 0;
+    if (rope_mode == BZ_ROPE_FULL) {
+        RopeRaggedArgs ra;
+        ra.q = q; ra.k = k; ra.indptr = qo_indptr;
+        ra.batch_size = batch_size; ra.num_qo_heads = num_qo_heads; ra.num_kv_heads = num_kv_heads;
+        ra.freqs = make_rope_freqs(128, rope_theta > 0.f ? rope_theta : 1e4f);
+        if (dtype == BZ_F16) hipLaunchKernelGGL((rope_ragged_kernel<f16_t>), dim3(p->total_tokens), dim3(256), 0, s, ra);
+        else hipLaunchKernelGGL((rope_ragged_kernel<bf16_t>), dim3(p->total_tokens), dim3(256), 0, s, ra);
+        BZ_LAUNCH_CHECK();
+    }
+    PrefillArgs a;
+    a.out = out;
+    a.items = p->items_d;
+    a.num_qo_heads = num_qo_heads; a.num_kv_heads = num_kv_heads;
+    a.causal = causal ? 1 : 0;
+    if (!(sm_scale > 0.f)) sm_scale = 1.0f / sqrtf((float)head_dim);
+    a.sm_scale_log2 = sm_scale * 1.4426950408889634f;
+    if (dtype == BZ_F16) return launch_prefill<false, false>(p, a, q, k, v, s);
+    return launch_prefill<true, true>(p, a, q, k, v, s);
 }

@@ -1,0 +1,114 @@
+"""GPU parity: ragged (causal) prefill attention through the C ABI against the CPU checker.
+Tolerance: max-abs <= 2e-3 for f16 (widened to half a storage step for bf16 results >= 0.5)."""
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from blitz_scale_amd import kernel as K
+from blitz_scale_amd import workloads as wl
+from blitz_scale_amd._lib import BZ_BF16, BZ_F16, BZ_LAYOUT_HND, BZ_ROPE_FULL, BZ_ROPE_NONE
+
+from _gpu import DeviceDecode, to_dev, to_host_bits
+from _util import DecodeProblem, ulp_tol
+
+pytestmark = pytest.mark.gpu
+
+
+class Prefill:
+    def __init__(self, seed, lens, Hq, Hkv, D, dtype):
+        rng = np.random.default_rng(seed)
+        self.lens, self.Hq, self.Hkv, self.D, self.dtype = lens, Hq, Hkv, D, dtype
+        self.indptr = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+        N = int(self.indptr[-1])
+        self.q = wl.randn_bits(rng, (N, Hq, D), dtype)
+        self.k = wl.randn_bits(rng, (N, Hkv, D), dtype)
+        self.v = wl.randn_bits(rng, (N, Hkv, D), dtype)
+        self.float_ws = torch.empty(1 << 20, dtype=torch.uint8, device="cuda")
+        self.int_ws = torch.empty(8 << 20, dtype=torch.uint8, device="cuda")
+        self.handler = K.BatchPrefillRaggedHandler()
+
+    def run(self, causal=True, rope_mode=BZ_ROPE_NONE, theta=1e4):
+        B = len(self.lens)
+        self.handler.plan(self.float_ws, self.float_ws.numel(), self.int_ws, self.int_ws.numel(), self.indptr,
+                          self.indptr, B, self.Hq, self.Hkv, self.D, 16)
+        qd, kd, vd = to_dev(self.q, self.dtype), to_dev(self.k, self.dtype), to_dev(self.v, self.dtype)
+        ip = torch.from_numpy(self.indptr).cuda()
+        out = torch.full_like(qd, float("nan"))
+        K.batch_prefill_attention(self.handler, qd, ip, kd, vd, ip, out, B, self.Hq, self.Hkv, self.D, causal=causal,
+                                  rope_mode=rope_mode, rope_theta=theta)
+        torch.cuda.synchronize()
+        self.q_after, self.k_after = to_host_bits(qd), to_host_bits(kd)
+        return wl.to_f32(to_host_bits(out), self.dtype)
+
+
+@pytest.mark.parametrize("dtype", [BZ_F16, BZ_BF16])
+@pytest.mark.parametrize("causal", [True, False])
+@pytest.mark.parametrize("Hq,Hkv", [(4, 4), (8, 2)])
+def test_small_ragged_full_check(dtype, causal, Hq, Hkv):
+    pf = Prefill(200 + Hq, [1, 7, 64, 65, 127, 128, 129, 300, 2], Hq, Hkv, 128, dtype)
+    got = pf.run(causal=causal)
+    ref = oracle.batch_prefill_ragged(pf.q, pf.k, pf.v, dtype, pf.indptr, Hq, Hkv, 128, causal=causal, parallel=True)
+    assert not np.isnan(got).any()
+    assert (np.abs(got - ref) <= ulp_tol(ref, dtype)).all(), np.abs(got - ref).max()
+    if dtype == BZ_F16:
+        assert np.abs(got - ref).max() <= 2e-3
+
+
+def test_rope_inside_the_call_rotates_q_and_k_in_place():
+    theta, dtype = 1e4, BZ_F16
+    pf = Prefill(210, [5, 200, 131], 8, 4, 128, dtype)
+    got = pf.run(causal=True, rope_mode=BZ_ROPE_FULL, theta=theta)
+    q_rot = oracle.rope_ragged(pf.q, dtype, pf.indptr, 8, 128, theta)
+    k_rot = oracle.rope_ragged(pf.k, dtype, pf.indptr, 4, 128, theta)
+    for g, w in ((pf.q_after, q_rot), (pf.k_after, k_rot)):
+        assert np.abs(wl.to_f32(g, dtype) - wl.to_f32(w, dtype)).max() <= 2.0 ** -8
+        assert (g != w).mean() < 2e-3
+    # attention over exactly the bits the device left behind
+    ref = oracle.batch_prefill_ragged(pf.q_after, pf.k_after, pf.v, dtype, pf.indptr, 8, 4, 128, causal=True, parallel=True)
+    assert np.abs(got - ref).max() <= 2e-3
+
+
+def test_prefill_then_store_then_decode_is_consistent():
+    """Row i of the prefill output equals a decode over the first i+1 cached tokens (GPU against GPU and
+    against the checker): ties the three kernels of the path together."""
+    dtype, Hq, Hkv, D, P = BZ_F16, 8, 2, 128, 16
+    pf = Prefill(220, [77, 300], Hq, Hkv, D, dtype)
+    got = pf.run(causal=True)
+    for r, L in enumerate(pf.lens):
+        p = DecodeProblem(221 + r, [L], Hq, Hkv, D, P, dtype)
+        dev = DeviceDecode(p)
+        s, e = pf.indptr[r], pf.indptr[r + 1]
+        ri = torch.tensor([0, L], dtype=torch.int32, device="cuda")
+        K.store_prefill_kv_cache(dev.pt, to_dev(pf.k[s:e], dtype), to_dev(pf.v[s:e], dtype), ri)
+        dev.plan()
+        dec = dev.decode(3, q=to_dev(pf.q[e - 1:e], dtype))
+        assert np.abs(dec[0] - got[e - 1]).max() <= 2e-3
+
+
+@pytest.mark.parametrize("batch", [4, 16])
+def test_c4_shape_sampled_rows(batch):
+    """Llama-2-13B-shaped prefill (40/40 heads, D 128, f16, lengths U[128,4096], causal); batch 16 is the
+    full BASELINE config 4.  The checker evaluates a seeded sample of rows (all heads) plus the first and
+    last row of every request."""
+    cfg = wl.CONFIGS["C4"]
+    rng = np.random.default_rng(wl.DEFAULT_SEED)
+    lens = [int(x) for x in rng.integers(128, 4097, size=batch)]
+    pf = Prefill(wl.DEFAULT_SEED, lens, cfg["Hq"], cfg["Hkv"], cfg["D"], cfg["dtype"])
+    got = pf.run(causal=True)
+    N = int(pf.indptr[-1])
+    rows = np.unique(np.concatenate([rng.integers(0, N, size=48), pf.indptr[:-1], pf.indptr[1:] - 1])).astype(np.int32)
+    ref = oracle.batch_prefill_ragged(pf.q, pf.k, pf.v, cfg["dtype"], pf.indptr, cfg["Hq"], cfg["Hkv"], cfg["D"],
+                                      causal=True, rows=rows, parallel=True)
+    assert not np.isnan(got).any()
+    assert np.abs(got[rows] - ref).max() <= 2e-3
+
+
+def test_prefill_error_codes():
+    pf = Prefill(230, [5], 4, 4, 128, BZ_F16)
+    qd = to_dev(pf.q, BZ_F16)
+    ip = torch.from_numpy(pf.indptr).cuda()
+    with pytest.raises(K.BzError, match="BatchPrefillWithRaggedKVCache error"):
+        K.batch_prefill_attention(pf.handler, qd, ip, qd, qd, ip, qd, 1, 4, 4, 128)  # not planned
+    with pytest.raises(K.BzError, match="Handler plan"):
+        pf.handler.plan(pf.float_ws, 1, pf.int_ws, 1, pf.indptr, pf.indptr, 1, 4, 4, 64, 16)  # head_dim 64
