@@ -13,7 +13,7 @@ LIB_PATH = os.environ.get("BZ_HIP_LIB") or os.path.join(HERE, "lib", "libbz_hip.
 BZ_F16, BZ_BF16, BZ_E4M3, BZ_F32 = 0, 1, 2, 3
 BZ_ROPE_NONE, BZ_ROPE_Q_ONLY, BZ_ROPE_FULL = 0, 1, 2
 BZ_LAYOUT_NHD, BZ_LAYOUT_HND = 0, 1
-BZ_ERR_BAD_ARG, BZ_ERR_UNSUPPORTED, BZ_ERR_WORKSPACE, BZ_ERR_NOT_PLANNED = 10001, 10002, 10003, 10004
+BZ_ERR_BAD_ARG, BZ_ERR_UNSUPPORTED, BZ_ERR_WORKSPACE, BZ_ERR_NOT_PLANNED, BZ_ERR_NO_PAGES = 10001, 10002, 10003, 10004, 10005
 
 
 class BzPagedKV(C.Structure):
@@ -62,6 +62,17 @@ SIGNATURES = {
     "bz_add_rms_norm": (_i32, [_vp, _vp, _vp, _i32, _u32, _u32, _f32, _vp]),
     "bz_silu_and_mul": (_i32, [_vp, _vp, _i32, _u32, _u32, _vp]),
     "bz_add_residual": (_i32, [_vp, _vp, _i32, _u32, _u32, _vp]),
+    "bz_cm_create": (_i32, [C.POINTER(_vp), _u32, _u32, _u32, _u32, _u32, _i32, _i32, _i32]),
+    "bz_cm_destroy": (None, [_vp]),
+    "bz_cm_batch_prefill": (_i32, [_vp, _vp, _u32, C.POINTER(_i32)]),
+    "bz_cm_batch_grow": (_i32, [_vp, _i32]),
+    "bz_cm_batch_filter": (_i32, [_vp, _i32, _vp, _u32]),
+    "bz_cm_batch_extend": (_i32, [_vp, _i32, _i32]),
+    "bz_cm_batch_release": (_i32, [_vp, _i32]),
+    "bz_cm_batch_table": (_i32, [_vp, _i32, C.POINTER(_vp), C.POINTER(_u32), C.POINTER(_vp), C.POINTER(_vp),
+                                 C.POINTER(_u32)]),
+    "bz_cm_stats": (_i32, [_vp, C.POINTER(_u64), C.POINTER(_u64), C.POINTER(_u64)]),
+    "bz_cm_pool": (_i32, [_vp, C.POINTER(_vp), C.POINTER(_u64)]),
     "bz_build_info": (C.c_char_p, []),
     "bz_error_string": (C.c_char_p, [_i32]),
 }

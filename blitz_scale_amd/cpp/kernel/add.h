@@ -1,0 +1,15 @@
+// Drop-in for src/kernel/add.h.
+#pragma once
+
+#include "bz_types.h"
+
+namespace blitz::kernel {
+
+/// residual += input with one rounding per element (src/kernel/add.h:8-14, add.cu:29-32).
+template<typename DType>
+void add_residual(DType* input, DType* residual, uint32_t num_tokens, uint32_t dim) {
+    bz_throw(bz_add_residual(input, residual, bz_dtype<DType>::value, num_tokens, dim, attention_options().stream),
+             "AddKernel");
+}
+
+} // namespace blitz::kernel

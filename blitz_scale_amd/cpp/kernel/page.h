@@ -1,0 +1,113 @@
+// Drop-in for src/kernel/page.h of the BlitzScale worker: the per-batch page table and the two
+// KV-page writers, over the C ABI of libbz_hip.so.
+#pragma once
+
+#include <cstddef>
+#include <cstdint>
+#include <vector>
+
+#include "bz_types.h"
+
+namespace blitz::kernel {
+
+/// Per-batch CSR page table plus the base pointers of one layer plane of the pool
+/// (same members as the reference struct, src/kernel/page.h:12-64, plus the in-page layout).
+/// Element address: page*stride_page + slot*stride_n + head*stride_h + d from k_data / v_data.
+template<typename DType, typename IdType>
+struct PageTable {
+    // host copy, maintained by the cache manager
+    std::vector<IdType> indices;
+    std::vector<IdType> indptr;
+    std::vector<IdType> last_page_len;
+    uint32_t batch_size;
+
+    const uint32_t page_size;
+    const uint32_t num_heads;
+    const uint32_t head_size;
+
+    const size_t stride_page; // 2 * num_heads * page_size * head_size: K half then V half
+    const size_t stride_n;    // between consecutive slots of one head
+    const size_t stride_h;    // between heads
+    const int layout;         // BZ_LAYOUT_HND (default) or BZ_LAYOUT_NHD (the reference's order)
+
+    // pinned host blob [indices | indptr | last_page_len]
+    IdType* indices_h = nullptr;
+    IdType* indptr_h = nullptr;
+    IdType* last_page_len_h = nullptr;
+
+    // one layer plane: v_data = k_data + num_heads * page_size * head_size
+    DType* k_data;
+    DType* v_data;
+    // device copy of the table, set by the caller right before a step (src/blitz/stub.h:1310-1313)
+    IdType* indices_d = nullptr;
+    IdType* indptr_d = nullptr;
+    IdType* last_page_len_d = nullptr;
+
+    PageTable(uint32_t batch_size_, uint32_t page_size_, uint32_t num_heads_, uint32_t head_size_, DType* base_ptr,
+              int layout_ = BZ_LAYOUT_HND) :
+        batch_size(batch_size_),
+        page_size(page_size_),
+        num_heads(num_heads_),
+        head_size(head_size_),
+        stride_page((size_t)2 * num_heads_ * page_size_ * head_size_),
+        stride_n(layout_ == BZ_LAYOUT_HND ? (size_t)head_size_ : (size_t)num_heads_ * head_size_),
+        stride_h(layout_ == BZ_LAYOUT_HND ? (size_t)page_size_ * head_size_ : (size_t)head_size_),
+        layout(layout_),
+        k_data(base_ptr),
+        v_data(base_ptr + (size_t)num_heads_ * page_size_ * head_size_) {}
+
+    /// plain-C image handed to the library
+    bz_paged_kv_t c_view() const {
+        bz_paged_kv_t kv;
+        kv.k_data = k_data; kv.v_data = v_data;
+        kv.indices = reinterpret_cast<const int32_t*>(indices_d);
+        kv.indptr = reinterpret_cast<const int32_t*>(indptr_d);
+        kv.last_page_len = reinterpret_cast<const int32_t*>(last_page_len_d);
+        kv.batch_size = batch_size; kv.page_size = page_size; kv.num_kv_heads = num_heads; kv.head_dim = head_size;
+        kv.stride_page = stride_page; kv.stride_n = stride_n; kv.stride_h = stride_h;
+        kv.kv_dtype = bz_dtype<DType>::value; kv.reserved = 0;
+        return kv;
+    }
+};
+
+/// src/kernel/page.h:66-67.  Token t of request b goes to page indices[indptr[b] + t/P], slot t%P.
+/// q (optional) is rotated in place with the same angles when K is rotated on the way in.
+template<typename DType, typename IdType, typename SrcType = DType>
+void store_prefill_kv_cache(PageTable<DType, IdType>& page_table, SrcType* k_data, SrcType* v_data,
+                            IdType* ragged_indptr, uint32_t num_tokens, SrcType* q_inout = nullptr,
+                            uint32_t num_qo_heads = 0, const float* k_scale = nullptr,
+                            const float* v_scale = nullptr) {
+    static_assert(sizeof(IdType) == 4, "page tables are int32");
+    const AttentionOptions& o = attention_options();
+    const bz_paged_kv_t kv = page_table.c_view();
+    bz_throw(bz_store_prefill_kv(&kv, k_data, v_data, bz_dtype<SrcType>::value,
+                                 reinterpret_cast<const int32_t*>(ragged_indptr), num_tokens, q_inout, num_qo_heads,
+                                 o.rotate_k_on_write ? 1 : 0, o.rope_theta, k_scale, v_scale, o.stream),
+             "AppendPagedKVCache");
+}
+
+/// src/kernel/page.h:69-70.  One new row per sequence at position seq_len-1.
+template<typename DType, typename IdType, typename SrcType = DType>
+void append_decode_kv_cache(PageTable<DType, IdType>& page_table, SrcType* k_data, SrcType* v_data,
+                            SrcType* q_inout = nullptr, uint32_t num_qo_heads = 0, const float* k_scale = nullptr,
+                            const float* v_scale = nullptr) {
+    static_assert(sizeof(IdType) == 4, "page tables are int32");
+    const AttentionOptions& o = attention_options();
+    const bz_paged_kv_t kv = page_table.c_view();
+    bz_throw(bz_append_decode_kv(&kv, k_data, v_data, bz_dtype<SrcType>::value, q_inout, num_qo_heads,
+                                 o.rotate_k_on_write ? 1 : 0, o.rope_theta, k_scale, v_scale, o.stream),
+             "AppendPagedKVCacheDecode");
+}
+
+/// declared and never defined in the reference (src/kernel/page.h:72-73); here it is the token count
+template<typename DType, typename IdType>
+uint32_t cal_total_num_rows(const PageTable<DType, IdType>& page_table) {
+    uint32_t rows = 0;
+    for (uint32_t b = 0; b < page_table.batch_size; ++b) {
+        const IdType n = page_table.indptr[b + 1] - page_table.indptr[b];
+        if (n > 0) rows += (uint32_t)(n - 1) * page_table.page_size + (uint32_t)page_table.last_page_len[b];
+    }
+    return rows;
+}
+
+} // namespace blitz::kernel

@@ -133,6 +133,16 @@ __global__ __launch_bounds__(256) void page_write_kernel(PageWriteArgs a) {
                 y[e] = yr;
             }
         }
+        if (PREFILL && rotate && Hq > 0) {
+            // fused RoPE of the prefill path: the caller's k rows are rotated in place as well, so the
+            // attention call that follows contracts rotated q with rotated k
+            Vec8<ST> lr, hr;
+            lr.from_float(x);
+            hr.from_float(y);
+            ST* srcw = const_cast<ST*>(src);
+            lr.store(srcw + lane * 8);
+            hr.store(srcw + D / 2 + lane * 8);
+        }
         if (scale) {
             const float sc = scale[h];
 #pragma unroll
@@ -186,7 +196,7 @@ static int fill_args(PageWriteArgs& a, const bz_paged_kv_t* kv, const void* k, c
 
 using namespace bz;
 
-extern "C" int bz_store_prefill_kv(const bz_paged_kv_t* kv, const void* k, const void* v, int src_dtype,
+extern "C" int bz_store_prefill_kv(const bz_paged_kv_t* kv, void* k, const void* v, int src_dtype,
                                    const int32_t* ragged_indptr, uint32_t num_tokens, void* q_inout,
                                    uint32_t num_qo_heads, int rope, float rope_theta, const float* k_scale,
                                    const float* v_scale, void* stream) {
@@ -246,6 +256,7 @@ extern "C" const char* bz_error_string(int code) {
         case BZ_ERR_UNSUPPORTED: return "bz: unsupported shape or type";
         case BZ_ERR_WORKSPACE: return "bz: workspace too small";
         case BZ_ERR_NOT_PLANNED: return "bz: plan() has not been called";
+        case BZ_ERR_NO_PAGES: return "bz: out of KV pages";
         default: return hipGetErrorString((hipError_t)code);
     }
 }

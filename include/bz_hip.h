@@ -41,6 +41,7 @@ extern "C" {
 #define BZ_ERR_UNSUPPORTED 10002
 #define BZ_ERR_WORKSPACE 10003
 #define BZ_ERR_NOT_PLANNED 10004
+#define BZ_ERR_NO_PAGES 10005 /* page allocator exhausted, or a page table outgrew its pinned chunk */
 
 /* In-page element order of the KV pool. */
 #define BZ_LAYOUT_NHD 0 /* [page][K|V][slot][head][dim]: the reference's (page.h:24-32) */
@@ -146,10 +147,11 @@ int bz_batch_prefill_ragged(bz_prefill_plan_t* plan, void* q, const int32_t* qo_
  * ------------------------------------------------------------------------------------- */
 /* store_prefill_kv_cache (src/kernel/page.h:66-67, page.cu:21-94): token t of request b goes to
  * page indices[indptr[b]+t/P], slot t%P.  k, v: [N, Hkv, D] of src_dtype.
- * rope != 0 rotates K at position t on the way in; q_inout (optional, [N, Hq, D], num_qo_heads)
- * is rotated in place by the same angles: the fused RoPE of the prefill path.
+ * rope != 0 rotates K at position t on the way in.  With q_inout (optional, [N, Hq, D],
+ * num_qo_heads) given as well, q AND the caller's k rows are rotated in place by the same angles:
+ * the fused RoPE of the prefill path, after which bz_batch_prefill_ragged runs with BZ_ROPE_NONE.
  * k_scale / v_scale: device fp32 [Hkv]; for an e4m3 pool the value stored is quant(x / scale). */
-int bz_store_prefill_kv(const bz_paged_kv_t* kv, const void* k, const void* v, int src_dtype,
+int bz_store_prefill_kv(const bz_paged_kv_t* kv, void* k, const void* v, int src_dtype,
                         const int32_t* ragged_indptr, uint32_t num_tokens, void* q_inout, uint32_t num_qo_heads,
                         int rope, float rope_theta, const float* k_scale, const float* v_scale, void* stream);
 
@@ -175,6 +177,34 @@ int bz_silu_and_mul(const void* input, void* output, int dtype, uint32_t num_tok
 /* add_residual (src/kernel/add.h:8-14, add.cu:13-61): residual += input, one rounding per element */
 int bz_add_residual(const void* input, void* residual, int dtype, uint32_t num_tokens, uint32_t dim,
                     void* stream);
+
+/* ---------------------------------------------------------------------------------------
+ * Host page-table logic: pool owner, first-fit page allocator and per-batch page tables in pinned
+ * memory.  Replaces the integer semantics of src/blitz/cache_manager.h:123-324 and of the page-table
+ * parts of src/blitz/batch.h (prefill constructor :206-276, update :280-295, filter :297-418,
+ * extend :482-576).  Pure host work; with_device = 0 skips the pool and the pinned allocation so
+ * that the logic can run without a GPU.  A batch's table is the blob [indices | indptr |
+ * last_page_len] that Stub::forward uploads in one copy (src/blitz/stub.h:1288-1313).
+ * ------------------------------------------------------------------------------------- */
+typedef struct bz_cache_manager bz_cache_manager_t;
+
+int bz_cm_create(bz_cache_manager_t** out, uint32_t num_kv_heads, uint32_t num_layers, uint32_t head_dim,
+                 uint32_t page_size, uint32_t max_pages, int kv_dtype, int layout, int with_device);
+void bz_cm_destroy(bz_cache_manager_t* cm);
+/* new batch from prompt lengths: each prompt reserves len+1 slots (batch.h:246-250), lowest free page ids */
+int bz_cm_batch_prefill(bz_cache_manager_t* cm, const int32_t* prompt_lens, uint32_t batch, int* batch_id);
+/* every sequence grows by one slot, a full last page gets a new page (cache_manager.h:255-324) */
+int bz_cm_batch_grow(bz_cache_manager_t* cm, int batch_id);
+/* keep the listed sequences (ascending positions), free the pages of the others (batch.h:297-418) */
+int bz_cm_batch_filter(bz_cache_manager_t* cm, int batch_id, const uint32_t* keep, uint32_t n_keep);
+/* append src's sequences to dst; src ceases to exist (batch.h:482-576) */
+int bz_cm_batch_extend(bz_cache_manager_t* cm, int dst_batch_id, int src_batch_id);
+int bz_cm_batch_release(bz_cache_manager_t* cm, int batch_id);
+/* host pointers into the batch's blob; valid until the batch changes */
+int bz_cm_batch_table(bz_cache_manager_t* cm, int batch_id, const int32_t** indices_h, uint32_t* nnz_pages,
+                      const int32_t** indptr_h, const int32_t** last_page_len_h, uint32_t* batch);
+int bz_cm_stats(bz_cache_manager_t* cm, uint64_t* free_pages, uint64_t* allocated_pages, uint64_t* total_pages);
+int bz_cm_pool(bz_cache_manager_t* cm, void** base, uint64_t* bytes);
 
 /* library / device identification: "gfx950" build string, and hipGetErrorString passthrough */
 const char* bz_build_info(void);

@@ -234,5 +234,21 @@ def prefill_reservation(lens, page_size):
     return indptr, lpl
 
 
+def first_fit(free_mask, n):
+    """Lowest n free page ids; marks them used.  None (mask untouched) when fewer are free."""
+    out = np.empty(max(n, 1), np.int32)
+    got = lib().bzo_first_fit(_p(free_mask), len(free_mask), n, _p(out))
+    return None if got < n else out[:n].copy()
+
+
+def table_grow(indices, indptr, last_page_len, page_size, free_mask):
+    """One step of growth; returns the new (indices, indptr, last_page_len) or None when out of pages."""
+    B = len(last_page_len)
+    ind = np.concatenate([_c(indices, np.int32), np.zeros(B + 1, np.int32)])
+    ip, lpl = _c(indptr, np.int32).copy(), _c(last_page_len, np.int32).copy()
+    n = lib().bzo_table_grow(_p(ind), _p(ip), _p(lpl), B, page_size, _p(free_mask), len(free_mask))
+    return None if n < 0 else (ind[:n].copy(), ip, lpl)
+
+
 def num_threads(parallel=True):
     return lib(parallel).bzo_num_threads()

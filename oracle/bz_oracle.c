@@ -525,3 +525,30 @@ int bzo_num_threads(void) { return omp_get_max_threads(); }
 #else
 int bzo_num_threads(void) { return 1; }
 #endif
+
+/* one decode step of page-table growth (cache_manager.h:255-324): a sequence whose last page is full
+ * gets the next lowest free page and restarts at slot 1, every other sequence gains one slot.
+ * indices must have room for B more entries.  Returns the new number of pages, or -1 (nothing
+ * changed) when the pool cannot supply the pages -- the reference throws at that point with the
+ * slot counts already bumped (cache_manager.h:264-281); all-or-nothing is the contract checked here. */
+int bzo_table_grow(int32_t* indices, int32_t* indptr, int32_t* last_page_len, int B, int P, uint8_t* free_mask,
+                   int max_pages) {
+    int nfull = 0;
+    for (int i = 0; i < B; ++i) nfull += (last_page_len[i] == P);
+    int32_t* fresh = (int32_t*)malloc(sizeof(int32_t) * (size_t)(nfull > 0 ? nfull : 1));
+    if (bzo_first_fit(free_mask, max_pages, nfull, fresh) < nfull) { free(fresh); return -1; }
+    int nnz = indptr[B];
+    int32_t* out = (int32_t*)malloc(sizeof(int32_t) * (size_t)(nnz + nfull + 1));
+    int w = 0, f = 0, start = 0;
+    for (int i = 0; i < B; ++i) {
+        int end = indptr[i + 1];
+        for (int j = start; j < end; ++j) out[w++] = indices[j];
+        start = end;
+        if (last_page_len[i] == P) { out[w++] = fresh[f++]; last_page_len[i] = 1; }
+        else last_page_len[i] += 1;
+        indptr[i + 1] = w;
+    }
+    memcpy(indices, out, sizeof(int32_t) * (size_t)w);
+    free(out); free(fresh);
+    return w;
+}

@@ -1,0 +1,262 @@
+// GPU test of the C++ drop-in headers: one prefill step and one decode step of a small transformer
+// layer through blitz::layer::Attention / GatedLinearUnit, blitz::CacheManager and the blitz::kernel
+// entry points, instantiated as <__half, int32_t> like the reference (src/server/disaggregate.cc:372),
+// checked against the same sequence built from the CPU checker's functions and a plain CPU GEMM.
+// Build: see tests/test_cpp_dropin.py.  Exit code 0 = pass.
+#include <cmath>
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <vector>
+
+#include <hip/hip_runtime.h>
+
+#include "blitz/cache_manager.h"
+#include "kernel/activation.h"
+#include "kernel/add.h"
+#include "kernel/attention.h"
+#include "kernel/rms_norm.h"
+#include "layer/attn.h"
+#include "layer/glu.h"
+
+// ---- the checker (oracle/bz_oracle.c), linked as a shared library --------------------------------
+extern "C" {
+typedef struct {
+    const void *k_base, *v_base;
+    const int32_t *indices, *indptr, *last_page_len;
+    int32_t batch_size, page_size, num_kv_heads, head_dim;
+    int64_t stride_page, stride_n, stride_h;
+    int32_t kv_dtype;
+} bzo_paged_kv;
+float bzo_f16_to_f32(uint16_t);
+uint16_t bzo_f32_to_f16(float);
+void bzo_rms_norm(const void*, const void*, int, int, int, float, float*);
+void bzo_add_rms_norm(const void*, void*, const void*, int, int, int, float, float*);
+void bzo_silu_and_mul(const void*, int, int, int, float*);
+void bzo_add_residual(const void*, void*, int, size_t);
+void bzo_rope_ragged_inplace(void*, int, const int32_t*, int, int, int, float);
+void bzo_rope_decode_q_inplace(void*, int, const bzo_paged_kv*, int, float);
+void bzo_store_prefill_kv(const bzo_paged_kv*, const void*, const void*, int, const int32_t*, int, float, const float*,
+                          const float*);
+void bzo_append_decode_kv(const bzo_paged_kv*, const void*, const void*, int, int, float, const float*, const float*);
+void bzo_batch_prefill_ragged(const void*, const void*, const void*, int, const int32_t*, int, int, int, int, int, int,
+                              float, float, const int32_t*, int, float*);
+void bzo_batch_decode(const void*, int, const bzo_paged_kv*, int, int, float, float, const float*, const float*, float*,
+                      float*);
+}
+
+#define HIP_OK(x)                                                                      \
+    do {                                                                               \
+        hipError_t e_ = (x);                                                           \
+        if (e_ != hipSuccess) {                                                        \
+            printf("HIP error %s at %s:%d\n", hipGetErrorString(e_), __FILE__, __LINE__); \
+            exit(2);                                                                   \
+        }                                                                              \
+    } while (0)
+
+using half_t = __half;
+typedef std::vector<uint16_t> bits_t;
+
+// naive row-major GEMM, fp32 accumulate in index order, one rounding to f16: test infrastructure only
+__global__ void naive_gemm(int m, int n, int k, const uint16_t* A, const uint16_t* B, uint16_t* Cm) {
+    const int col = blockIdx.x * blockDim.x + threadIdx.x, row = blockIdx.y;
+    if (col >= n) return;
+    float acc = 0.f;
+    for (int i = 0; i < k; ++i)
+        acc += __half2float(__ushort_as_half(A[(size_t)row * k + i])) * __half2float(__ushort_as_half(B[(size_t)i * n + col]));
+    Cm[(size_t)row * n + col] = __half_as_ushort(__float2half_rn(acc));
+}
+struct NaiveGemm : blitz::util::GemmWrapper {
+    void gemm(int m, int n, int k, const void* A, const void* B, void* C) override {
+        hipLaunchKernelGGL(naive_gemm, dim3((n + 127) / 128, m), dim3(128), 0, 0, m, n, k, (const uint16_t*)A,
+                           (const uint16_t*)B, (uint16_t*)C);
+    }
+};
+static void cpu_gemm(int m, int n, int k, const uint16_t* A, const uint16_t* B, uint16_t* C) {
+    for (int r = 0; r < m; ++r)
+        for (int c = 0; c < n; ++c) {
+            float acc = 0.f;
+            for (int i = 0; i < k; ++i) acc = fmaf(bzo_f16_to_f32(A[(size_t)r * k + i]), bzo_f16_to_f32(B[(size_t)i * n + c]), acc);
+            C[(size_t)r * n + c] = bzo_f32_to_f16(acc);
+        }
+}
+
+static uint64_t rng_state = 0x5EED;
+static float frand() { // uniform(-1, 1), splitmix64
+    uint64_t z = (rng_state += 0x9E3779B97F4A7C15ull);
+    z = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ull;
+    z = (z ^ (z >> 27)) * 0x94D049BB133111EBull;
+    z ^= z >> 31;
+    return (float)((double)(z >> 11) / 9007199254740992.0 * 2.0 - 1.0);
+}
+static bits_t rand_bits(size_t n, float scale, float mean = 0.f) {
+    bits_t v(n);
+    for (auto& x : v) x = bzo_f32_to_f16(mean + scale * frand());
+    return v;
+}
+static void round_to(const std::vector<float>& f, uint16_t* dst) {
+    for (size_t i = 0; i < f.size(); ++i) dst[i] = bzo_f32_to_f16(f[i]);
+}
+static double max_abs_diff(const uint16_t* a, const uint16_t* b, size_t n) {
+    double m = 0;
+    for (size_t i = 0; i < n; ++i) m = fmax(m, fabs((double)bzo_f16_to_f32(a[i]) - (double)bzo_f16_to_f32(b[i])));
+    return m;
+}
+
+int main() {
+    const uint32_t hidden = 256, Hq = 4, Hkv = 2, D = 128, inter = 512, P = 16, max_pages = 64, layers = 2;
+    const float theta = 1e4f;
+    blitz::kernel::attention_options().rope_theta = theta;
+
+    // ---- weights: attention segment then GLU segment, as one device buffer walked by seg_iter
+    const size_t attn_w = hidden + 2 * (size_t)Hq * D * hidden + 2 * (size_t)Hkv * D * hidden;
+    const size_t glu_w = hidden + 3 * (size_t)hidden * inter;
+    bits_t w_h = rand_bits(attn_w + glu_w, 0.06f);
+    for (size_t i = 0; i < hidden; ++i) w_h[i] = bzo_f32_to_f16(1.0f + 0.02f * frand());          // input norm
+    for (size_t i = 0; i < hidden; ++i) w_h[attn_w + i] = bzo_f32_to_f16(1.0f + 0.02f * frand()); // post-attn norm
+    half_t* w_d;
+    HIP_OK(hipMalloc(&w_d, w_h.size() * 2));
+    HIP_OK(hipMemcpy(w_d, w_h.data(), w_h.size() * 2, hipMemcpyHostToDevice));
+
+    // ---- engine objects
+    blitz::CacheManager<half_t, int32_t> cm(Hkv, layers, D, P, max_pages, BZ_LAYOUT_HND, true, 64 << 10);
+    void *float_ws, *int_ws;
+    HIP_OK(hipMalloc(&float_ws, 8 << 20));
+    HIP_OK(hipMalloc(&int_ws, 1 << 20));
+    blitz::kernel::BatchPrefillRaggedHandler<half_t, int32_t> prefill_h(blitz::kernel::create_flashinfer_prefill_handler());
+    blitz::kernel::BlitzBatchDecodeHandler<half_t, int32_t> decode_h(blitz::kernel::create_flashinfer_decode_handler());
+    if (prefill_h.empty() || decode_h.empty()) return 3;
+    const uint32_t maxN = 64;
+    const size_t ws_elems = maxN * (hidden + 3 * (size_t)std::max<uint32_t>(hidden, inter) + (size_t)(2 * Hq + 2 * Hkv) * D);
+    half_t* ws_d;
+    HIP_OK(hipMalloc(&ws_d, ws_elems * 2));
+    NaiveGemm gemm;
+    half_t* seg = w_d;
+    blitz::layer::Attention<half_t, int32_t> attn(&gemm, &prefill_h, &decode_h, D, hidden, Hq, Hkv, ws_d, &seg);
+    blitz::layer::GatedLinearUnit<half_t> glu(&gemm, hidden, inter, ws_d, &seg);
+    if (seg != w_d + attn_w + glu_w || attn.size_in_bytes() != attn_w * 2 || glu.size_in_bytes() != glu_w * 2) {
+        printf("weight segment walk is off\n");
+        return 4;
+    }
+
+    // ---- a prefill batch of two prompts; layer 1's plane is used to exercise the layer stride
+    std::vector<int32_t> lens = {20, 37};
+    blitz::HostBatch<half_t, int32_t> batch(&cm, lens);
+    auto& pt = batch.page_table;
+    cm.set_layer(pt, 1);
+    const uint32_t N = 57, B = 2;
+    int32_t* table_d;
+    HIP_OK(hipMalloc(&table_d, 1 << 20));
+    auto upload_table = [&]() { // one copy of the pinned blob, pointers are offsets into it (src/blitz/stub.h:1288-1313)
+        const size_t n = pt.indices.size() + pt.indptr.size() + pt.last_page_len.size();
+        HIP_OK(hipMemcpyAsync(table_d, pt.indices_h, n * 4, hipMemcpyHostToDevice, 0));
+        pt.indices_d = table_d;
+        pt.indptr_d = table_d + pt.indices.size();
+        pt.last_page_len_d = pt.indptr_d + pt.indptr.size();
+    };
+    upload_table();
+    int32_t* ragged_d;
+    HIP_OK(hipMalloc(&ragged_d, 64));
+    HIP_OK(hipMemcpy(ragged_d, batch.ragged_indptr.data(), (B + 1) * 4, hipMemcpyHostToDevice));
+
+    bits_t x_h = rand_bits((size_t)N * hidden, 1.0f);
+    HIP_OK(hipMemcpy(ws_d, x_h.data(), x_h.size() * 2, hipMemcpyHostToDevice));
+    prefill_h.plan(float_ws, 8 << 20, int_ws, 1 << 20, batch.ragged_indptr.data(), batch.ragged_indptr.data(), B, Hq, Hkv, D, P);
+    attn.forward(N, ragged_d, pt);
+    glu.forward(N);
+    HIP_OK(hipDeviceSynchronize());
+    bits_t res_gpu((size_t)N * hidden);
+    HIP_OK(hipMemcpy(res_gpu.data(), ws_d, res_gpu.size() * 2, hipMemcpyDeviceToHost));
+
+    // ---- the same on the CPU
+    const size_t plane = (size_t)max_pages * pt.stride_page;
+    bits_t pool_cpu(plane * layers, 0);
+    HIP_OK(hipMemcpy(pool_cpu.data(), cm.get_base_ptr(), pool_cpu.size() * 2, hipMemcpyDeviceToHost)); // untouched parts
+    bzo_paged_kv okv;
+    okv.k_base = pool_cpu.data() + plane; okv.v_base = pool_cpu.data() + plane + pt.stride_page / 2;
+    okv.indices = pt.indices.data(); okv.indptr = pt.indptr.data(); okv.last_page_len = pt.last_page_len.data();
+    okv.batch_size = B; okv.page_size = P; okv.num_kv_heads = Hkv; okv.head_dim = D;
+    okv.stride_page = pt.stride_page; okv.stride_n = pt.stride_n; okv.stride_h = pt.stride_h; okv.kv_dtype = 0;
+
+    const uint16_t *norm1 = w_h.data(), *wq = norm1 + hidden, *wk = wq + (size_t)Hq * D * hidden,
+                   *wv = wk + (size_t)Hkv * D * hidden, *wo = wv + (size_t)Hkv * D * hidden;
+    const uint16_t *norm2 = w_h.data() + attn_w, *wgu = norm2 + hidden, *wdn = wgu + 2 * (size_t)hidden * inter;
+    auto layer_cpu = [&](bits_t& resid, uint32_t n, bool prefill) {
+        std::vector<float> f((size_t)n * std::max<uint32_t>(hidden, std::max(inter, Hq * D)));
+        bits_t in((size_t)n * hidden), q((size_t)n * Hq * D), k((size_t)n * Hkv * D), v(k.size()), att(q.size());
+        bzo_rms_norm(resid.data(), norm1, 0, n, hidden, 1e-5f, f.data());
+        f.resize((size_t)n * hidden); round_to(f, in.data());
+        cpu_gemm(n, Hq * D, hidden, in.data(), wq, q.data());
+        cpu_gemm(n, Hkv * D, hidden, in.data(), wk, k.data());
+        cpu_gemm(n, Hkv * D, hidden, in.data(), wv, v.data());
+        std::vector<float> o((size_t)n * Hq * D);
+        if (prefill) {
+            bzo_store_prefill_kv(&okv, k.data(), v.data(), 0, batch.ragged_indptr.data(), 1, theta, nullptr, nullptr);
+            bzo_rope_ragged_inplace(q.data(), 0, batch.ragged_indptr.data(), B, Hq, D, theta);
+            bzo_rope_ragged_inplace(k.data(), 0, batch.ragged_indptr.data(), B, Hkv, D, theta);
+            bzo_batch_prefill_ragged(q.data(), k.data(), v.data(), 0, batch.ragged_indptr.data(), B, Hq, Hkv, D, 1, 0, theta,
+                                     1.0f / sqrtf((float)D), nullptr, 0, o.data());
+        } else {
+            bzo_append_decode_kv(&okv, k.data(), v.data(), 0, 1, theta, nullptr, nullptr);
+            bzo_rope_decode_q_inplace(q.data(), 0, &okv, Hq, theta);
+            bzo_batch_decode(q.data(), 0, &okv, Hq, 0, theta, 1.0f / sqrtf((float)D), nullptr, nullptr, o.data(), nullptr);
+        }
+        round_to(o, att.data());
+        bits_t oproj((size_t)n * hidden);
+        cpu_gemm(n, hidden, Hq * D, att.data(), wo, oproj.data());
+        // GLU
+        std::vector<float> g((size_t)n * hidden);
+        bzo_add_rms_norm(oproj.data(), resid.data(), norm2, 0, n, hidden, 1e-5f, g.data());
+        bits_t gin((size_t)n * hidden), gu((size_t)n * 2 * inter), st((size_t)n * inter), dn((size_t)n * hidden);
+        round_to(g, gin.data());
+        cpu_gemm(n, 2 * inter, hidden, gin.data(), wgu, gu.data());
+        std::vector<float> sf((size_t)n * inter);
+        bzo_silu_and_mul(gu.data(), 0, n, inter, sf.data());
+        round_to(sf, st.data());
+        cpu_gemm(n, hidden, inter, st.data(), wdn, dn.data());
+        bzo_add_residual(dn.data(), resid.data(), 0, (size_t)n * hidden);
+    };
+    bits_t res_cpu = x_h;
+    layer_cpu(res_cpu, N, true);
+    const double e1 = max_abs_diff(res_gpu.data(), res_cpu.data(), res_cpu.size());
+    printf("prefill layer: max |gpu - cpu| over the residual stream = %.3e\n", e1);
+
+    // ---- one decode step: the table grows by a slot per sequence, new token per sequence
+    batch.grow();
+    cm.set_layer(pt, 1); // grow() does not touch the plane pointers, but a real step resets them (src/blitz/stub.h:1349-1351)
+    upload_table();
+    okv.indices = pt.indices.data(); okv.indptr = pt.indptr.data(); okv.last_page_len = pt.last_page_len.data();
+    bits_t xd = rand_bits((size_t)B * hidden, 1.0f);
+    HIP_OK(hipMemcpy(ws_d, xd.data(), xd.size() * 2, hipMemcpyHostToDevice));
+    decode_h.plan(float_ws, 8 << 20, int_ws, 1 << 20, pt.indptr_h, pt.last_page_len_h, B, Hq, Hkv, D, P);
+    attn.forward(B, nullptr, pt);
+    glu.forward(B);
+    HIP_OK(hipDeviceSynchronize());
+    bits_t dres_gpu((size_t)B * hidden);
+    HIP_OK(hipMemcpy(dres_gpu.data(), ws_d, dres_gpu.size() * 2, hipMemcpyDeviceToHost));
+    bits_t dres_cpu = xd;
+    layer_cpu(dres_cpu, B, false);
+    const double e2 = max_abs_diff(dres_gpu.data(), dres_cpu.data(), dres_cpu.size());
+    printf("decode layer : max |gpu - cpu| over the residual stream = %.3e\n", e2);
+
+    // the two pools agree (K rotated on the way in: one f16 step on rare elements)
+    bits_t pool_gpu(pool_cpu.size());
+    HIP_OK(hipMemcpy(pool_gpu.data(), cm.get_base_ptr(), pool_gpu.size() * 2, hipMemcpyDeviceToHost));
+    const double e3 = max_abs_diff(pool_gpu.data() + plane, pool_cpu.data() + plane, plane);
+    size_t touched0 = 0;
+    for (size_t i = 0; i < plane; ++i) touched0 += pool_gpu[i] != pool_cpu[i];
+    printf("kv plane of layer 1: max diff %.3e; layer 0 plane differs in %zu elements\n", e3, touched0);
+
+    // error convention: std::runtime_error with the reference's message prefix
+    bool threw = false;
+    try {
+        blitz::kernel::BlitzBatchDecodeHandler<half_t, int32_t> fresh(blitz::kernel::create_flashinfer_decode_handler());
+        blitz::kernel::batch_decode_attention(fresh, ws_d, pt, ws_d, Hq);
+    } catch (const std::runtime_error& e) {
+        threw = strncmp(e.what(), "batchDecodeAttention error: ", 28) == 0;
+    }
+    // the activations are O(1); a chain of f16 roundings through four GEMMs stays within a few 1e-3
+    const bool ok = e1 < 2e-2 && e2 < 2e-2 && e3 < 5e-3 && touched0 == 0 && threw;
+    printf(ok ? "PASS\n" : "FAIL\n");
+    return ok ? 0 : 1;
+}

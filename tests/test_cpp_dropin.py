@@ -1,0 +1,39 @@
+"""The C++ drop-in headers (blitz_scale_amd/cpp) used the way the reference's worker uses its own:
+a hipcc-built program runs a prefill and a decode step of one layer and checks them against the CPU
+checker.  The binary is built on the CPU side (build_cpp_test) and only executed on the GPU box."""
+import os
+import subprocess
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+BIN = os.path.join(ROOT, "tests", "cpp", "test_dropin")
+
+
+def build_cpp_test():
+    import oracle
+    oracle.build()
+    cpp = os.path.join(ROOT, "blitz_scale_amd", "cpp")
+    cmd = ["/opt/rocm/bin/hipcc", "--offload-arch=gfx950", "-O2", "-std=c++17", "-Xclang", "-target-feature", "-Xclang",
+           "-packed-fp32-ops", "-I", os.path.join(ROOT, "include"), "-I", cpp, "-I", os.path.join(cpp, "kernel"),
+           os.path.join(ROOT, "tests", "cpp", "test_dropin.cpp"), "-o", BIN,
+           "-L", os.path.join(ROOT, "blitz_scale_amd", "lib"), "-lbz_hip", "-L", os.path.join(ROOT, "oracle"), "-lbz_oracle",
+           "-Wl,-rpath,$ORIGIN/../../blitz_scale_amd/lib", "-Wl,-rpath,$ORIGIN/../../oracle"]
+    out = subprocess.run(cmd, capture_output=True, text=True)
+    err = "\n".join(l for l in out.stderr.splitlines() if "packed-fp32-ops" not in l)
+    if out.returncode != 0:
+        raise RuntimeError("hipcc failed:\n" + err)
+    return BIN
+
+
+def test_headers_compile_and_link_without_a_gpu():
+    assert os.path.exists(build_cpp_test())
+
+
+@pytest.mark.gpu
+def test_layer_prefill_and_decode_through_the_cpp_headers():
+    if not os.path.exists(BIN):
+        build_cpp_test()
+    out = subprocess.run([BIN], capture_output=True, text=True, timeout=120)
+    print(out.stdout, out.stderr)
+    assert out.returncode == 0 and "PASS" in out.stdout

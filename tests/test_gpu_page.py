@@ -100,12 +100,14 @@ def test_fused_rope_store_prefill():
     want = p.pool.copy()
     oracle.store_prefill_kv(p.oracle_kv(want), k, v, dtype, ri, rope=True, rope_theta=theta)
     want_q = oracle.rope_ragged(q, dtype, ri, Hq, D, theta)
+    want_k = oracle.rope_ragged(k, dtype, ri, Hkv, D, theta)
     dev = DeviceDecode(p)
-    qd = to_dev(q, dtype)
-    K.store_prefill_kv_cache(dev.pt, to_dev(k, dtype), to_dev(v, dtype), to_dev(ri.view(np.float32), 3).view(torch.int32),
+    qd, kd = to_dev(q, dtype), to_dev(k, dtype)
+    K.store_prefill_kv_cache(dev.pt, kd, to_dev(v, dtype), to_dev(ri.view(np.float32), 3).view(torch.int32),
                              q=qd, num_qo_heads=Hq, rope=True, rope_theta=theta)
     torch.cuda.synchronize()
-    for g, w in ((to_host_bits(dev.pool), want), (to_host_bits(qd), want_q)):
+    # pool, q rows and the caller's k rows all carry the rotation
+    for g, w in ((to_host_bits(dev.pool), want), (to_host_bits(qd), want_q), (to_host_bits(kd), want_k)):
         assert np.abs(wl.to_f32(g, dtype) - wl.to_f32(w, dtype)).max() <= 2.0 ** -8
         assert (g != w).mean() < 2e-3
 
