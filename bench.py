@@ -1,12 +1,15 @@
-"""Headline benchmark: Llama-3-8B-shaped GQA paged decode (BASELINE config 3) on one MI355X.
+"""Benchmark of the paged-attention compute path on one MI355X.  Prints ONE JSON line.
 
-A step is one layer's decode-time attention block over the whole batch: the fused RoPE + KV append
-of the new token followed by batch decode over the paged KV cache (src/layer/attn.h:196-203 of the
-reference).  Steps cycle over several layer planes of the pool, as a model's layer loop does, so the
-KV a step reads has not just been read by the previous step.  plan() runs once per model step in the
-reference (src/model/llama.h:363-375), outside the layer loop, and is timed separately here.
+Default workload (the headline, BASELINE config 3): Llama-3-8B-shaped GQA paged decode, bf16, batch
+128, 32/8 heads, head_dim 128, page_size 16, log-normal contexts.  A step is one layer's decode-time
+attention block over the whole batch: the fused RoPE + KV append of the new token followed by batch
+decode over the paged KV cache (src/layer/attn.h:196-203 of the reference).  Steps cycle over several
+layer planes of the pool, as a model's layer loop does, so the KV a step reads has not just been read
+by the previous step.  plan() runs once per model step in the reference (src/model/llama.h:363-375),
+outside the layer loop, and is timed separately.
 
-Prints ONE JSON line.  One GPU only.
+--workload C2 | C4 | C5 run the other configurations (C2 adds the RMSNorm and SiLU-gate kernels of the
+layer, C4 is the ragged causal prefill + page store, C5 the e4m3-KV decode).  One GPU only.
 """
 import argparse
 import json
@@ -17,54 +20,103 @@ import time
 ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
-HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E
+HBM_PEAK_GBPS = 8000.0     # MI355X HBM3E
+MFMA_PEAK_TFLOPS = 2500.0  # dense f16 / bf16
 
 
-def main():
+def parse():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=400)
-    ap.add_argument("--warmup", type=int, default=40)
-    ap.add_argument("--layers", type=int, default=8, help="layer planes of the KV pool the steps cycle over")
+    ap.add_argument("--steps", type=int, default=None)
+    ap.add_argument("--warmup", type=int, default=None)
+    ap.add_argument("--workload", default="C3", choices=["C2", "C3", "C4", "C5"])
+    ap.add_argument("--layers", type=int, default=None, help="layer planes of the KV pool the steps cycle over")
     ap.add_argument("--seed", type=lambda s: int(s, 0), default=0x5EED)
-    ap.add_argument("--sigma", type=float, default=1.0, help="sigma of the log-normal context lengths")
+    ap.add_argument("--sigma", type=float, default=1.0, help="sigma of the log-normal context lengths (C3)")
     ap.add_argument("--split-tokens", type=int, default=2048)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on ONE GPU (--gpus 1); the path shards by kv head / by sequence "
                  "without any exchange inside attention, and nothing here launches a second rank.")
+    return args
 
+
+def pct(a):
+    import numpy as np
+    return {"mean": round(float(a.mean()) * 1e3, 3), "p10": round(float(np.percentile(a, 10)) * 1e3, 3),
+            "p50": round(float(np.percentile(a, 50)) * 1e3, 3), "p90": round(float(np.percentile(a, 90)) * 1e3, 3)}
+
+
+def timed(step, steps, warmup):
+    """W untimed steps, then exactly K steps between two device synchronisations; per-step HIP event pairs
+    (torch's current stream is the stream every launch goes to) bracket the dominant kernel."""
+    import numpy as np
+    import torch
+    for i in range(warmup):
+        step(i, None)
+    torch.cuda.synchronize()
+    events = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(steps)]
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(steps):
+        step(i, events[i])
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    return elapsed / steps * 1e3, np.array([a.elapsed_time(b) for a, b in events])
+
+
+def bench_decode(args, name):
     import numpy as np
     import torch
 
-    from blitz_scale_amd import _lib, kernel as K, workloads as wl
-    from blitz_scale_amd._lib import BZ_BF16, BZ_LAYOUT_HND, BZ_ROPE_NONE
+    from blitz_scale_amd import kernel as K, workloads as wl
+    from blitz_scale_amd._lib import BZ_BF16, BZ_E4M3, BZ_F16, BZ_LAYOUT_HND, BZ_ROPE_NONE
 
-    _lib.load()  # fails loudly if the HIP library is not built
-    torch.cuda.set_device(0)
     dev = "cuda"
-    cfg = dict(wl.CONFIGS["C3"])
+    cfg = dict(wl.CONFIGS[name])
     B, Hq, Hkv, D, P = cfg["batch"], cfg["Hq"], cfg["Hkv"], cfg["D"], cfg["P"]
     theta = cfg["rope_theta"]
+    tdt = torch.float16 if cfg["dtype"] == BZ_F16 else torch.bfloat16
+    fp8 = cfg["kv_dtype"] == BZ_E4M3
     rng = np.random.default_rng(args.seed)
-    ctx = wl.lognormal_ctx(rng, B, 1024.0, args.sigma, 64, 8192)
+    if name == "C3":
+        ctx = wl.lognormal_ctx(rng, B, 1024.0, args.sigma, 64, 8192)
+        ctx_desc = f"lognormal(mean 1024, sigma {args.sigma}) clipped [64,8192]"
+    else:
+        ctx = wl.ctx_lens_for(cfg, rng)
+        ctx_desc = str(cfg["ctx"])
     need = int(((ctx + P - 1) // P).sum())
-    pool_pages = int(np.ceil(need * cfg["oversub"]))
+    pool_pages = int(np.ceil(need * cfg.get("oversub", 1.0)))
     indices, indptr, lpl = wl.page_table_for(ctx, P, pool_pages, rng)
     stride_page, _, _ = wl.strides(BZ_LAYOUT_HND, Hkv, P, D)
-    L = args.layers
+    kv_bytes = 1 if fp8 else 2
+    plane = pool_pages * stride_page
+    L = args.layers or max(2, min(8, int(12e9 // (plane * kv_bytes))))
+    steps = args.steps or (400 if name == "C3" else 200)
+    warmup = args.warmup if args.warmup is not None else 40
 
     g = torch.Generator(device=dev)
     g.manual_seed(args.seed)
-    pool = torch.empty(L * pool_pages * stride_page, dtype=torch.bfloat16, device=dev)
-    plane = pool_pages * stride_page
-    for l in range(L):
-        pool[l * plane:(l + 1) * plane].normal_(generator=g)
-    q = torch.randn((B, Hq, D), dtype=torch.bfloat16, device=dev, generator=g)
-    k_new = torch.randn((B, Hkv, D), dtype=torch.bfloat16, device=dev, generator=g)
-    v_new = torch.randn((B, Hkv, D), dtype=torch.bfloat16, device=dev, generator=g)
-    out = torch.empty((B, Hq, D), dtype=torch.bfloat16, device=dev)
+    k_scale = v_scale = None
+    if fp8:
+        # N(0,1) values, per-kv-head scale amax/448 with amax taken as 5.5 sigma, stored as e4m3 bytes
+        scale = torch.full((Hkv,), 5.5 / 448.0, dtype=torch.float32, device=dev)
+        k_scale, v_scale = scale, scale.clone()
+        pool = torch.empty(L * plane, dtype=torch.uint8, device=dev)
+        chunk = 1 << 26
+        for off in range(0, L * plane, chunk):
+            n = min(chunk, L * plane - off)
+            x = torch.randn(n, dtype=torch.float32, device=dev, generator=g) / (5.5 / 448.0)
+            pool[off:off + n] = x.clamp_(-448, 448).to(torch.float8_e4m3fn).view(torch.uint8)
+    else:
+        pool = torch.empty(L * plane, dtype=tdt, device=dev)
+        for l in range(L):
+            pool[l * plane:(l + 1) * plane].normal_(generator=g)
+    q = torch.randn((B, Hq, D), dtype=tdt, device=dev, generator=g)
+    k_new = torch.randn((B, Hkv, D), dtype=tdt, device=dev, generator=g)
+    v_new = torch.randn((B, Hkv, D), dtype=tdt, device=dev, generator=g)
+    out = torch.empty((B, Hq, D), dtype=tdt, device=dev)
 
     pt = K.PageTable(B, P, Hkv, D, pool, layout=BZ_LAYOUT_HND)
     pt.indices, pt.indptr, pt.last_page_len = indices, indptr, lpl
@@ -84,84 +136,185 @@ def main():
     plan_ms = (time.perf_counter() - t0) / 10 * 1e3
     info = handler.info()
 
-    def step(i, ev=None):
+    extra = {}
+    if name == "C2":  # the layer's RMSNorm and SiLU-gate kernels ride along (hidden 4096, inter 11008)
+        h, I = cfg["hidden"], cfg["inter"]
+        x = torch.randn((B, h), dtype=tdt, device=dev, generator=g)
+        res = torch.randn((B, h), dtype=tdt, device=dev, generator=g)
+        w = (1 + 0.02 * torch.randn((h,), device=dev, generator=g)).to(tdt)
+        gate_up = torch.randn((B, 2 * I), dtype=tdt, device=dev, generator=g)
+        act = torch.empty((B, I), dtype=tdt, device=dev)
+        extra = {"hidden": h, "inter": I}
+
+    def step(i, ev):
         pt.set_layer(i % L, pool_pages)
-        K.append_decode_kv_cache(pt, k_new, v_new, q=q, num_qo_heads=Hq, rope=True, rope_theta=theta)
+        K.append_decode_kv_cache(pt, k_new, v_new, q=q, num_qo_heads=Hq, rope=theta is not None,
+                                 rope_theta=theta or 1e4, k_scale=k_scale, v_scale=v_scale)
         if ev is not None:
             ev[0].record()
-        K.batch_decode_attention(handler, q, pt, out, Hq, rope_mode=BZ_ROPE_NONE)
+        K.batch_decode_attention(handler, q, pt, out, Hq, rope_mode=BZ_ROPE_NONE, k_scale=k_scale, v_scale=v_scale)
         if ev is not None:
             ev[1].record()
+        if name == "C2":
+            K.add_rms_norm(x, res, w, B, h)
+            K.silu_and_mul(gate_up, act, B, I)
 
-    for i in range(args.warmup):
-        step(i)
-    torch.cuda.synchronize()
-    events = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(args.steps)]
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for i in range(args.steps):
-        step(i, events[i])
-    torch.cuda.synchronize()
-    elapsed = time.perf_counter() - t0
-    ms_per_step = elapsed / args.steps * 1e3
-    dec_ms = np.array([a.elapsed_time(b) for a, b in events])
-
-    alg_bytes = wl.decode_algorithmic_bytes(ctx, Hq, Hkv, D, 2, 2, P)
-    dec_avg_s = float(dec_ms.mean()) * 1e-3
-    achieved = alg_bytes / dec_avg_s / 1e9
-
-    res = {
-        "metric": "paged_decode_us_per_step",
-        "value": round(ms_per_step * 1e3, 3),
-        "unit": "us/step",
-        "n_gpus": 1,
-        "steps": args.steps,
-        "warmup": args.warmup,
-        "ms_per_step": round(ms_per_step, 6),
-        "higher_is_better": False,
-        "scaling": "weak",
-        "vs_baseline": None,
-        "dtype": "bf16",
-        "data": "synthetic",
-        "config": {
-            "workload": "C3: Llama-3-8B-shaped GQA paged decode, one layer per step (fused RoPE+append, batch decode)",
-            "batch": B, "num_qo_heads": Hq, "num_kv_heads": Hkv, "head_dim": D, "page_size": P,
-            "ctx": f"lognormal(mean 1024, sigma {args.sigma}) clipped [64,8192]", "sum_ctx": int(ctx.sum()),
-            "max_ctx": int(ctx.max()), "pool_pages_per_layer": pool_pages, "layer_planes_cycled": L,
-            "kv_layout": "HND", "rope_theta": theta, "split_tokens": args.split_tokens, "seed": hex(args.seed),
-            "plan": info,
-        },
+    ms_per_step, dec_ms = timed(step, steps, warmup)
+    alg_bytes = wl.decode_algorithmic_bytes(ctx, Hq, Hkv, D, kv_bytes, 2, P)
+    achieved = alg_bytes / (float(dec_ms.mean()) * 1e-3) / 1e9
+    res_json = {
+        "metric": "paged_decode_us_per_step", "value": round(ms_per_step * 1e3, 3), "unit": "us/step",
+        "n_gpus": 1, "steps": steps, "warmup": warmup, "ms_per_step": round(ms_per_step, 6),
+        "higher_is_better": False, "scaling": "weak", "vs_baseline": None,
+        "dtype": ("bf16" if tdt == torch.bfloat16 else "f16") + (" q, e4m3 kv" if fp8 else ""), "data": "synthetic",
+        "config": dict({
+            "workload": {"C2": "C2: Llama-2-7B-shaped MHA decode step of one layer (fused RoPE+append, batch decode, "
+                               "add+RMSNorm, SiLU-gate)",
+                         "C3": "C3: Llama-3-8B-shaped GQA paged decode, one layer per step (fused RoPE+append, batch decode)",
+                         "C5": "C5: Llama-3-70B-shaped GQA decode with e4m3 KV, one layer per step (quantising append, "
+                               "batch decode)"}[name],
+            "batch": B, "num_qo_heads": Hq, "num_kv_heads": Hkv, "head_dim": D, "page_size": P, "ctx": ctx_desc,
+            "sum_ctx": int(ctx.sum()), "max_ctx": int(ctx.max()), "pool_pages_per_layer": pool_pages,
+            "layer_planes_cycled": L, "kv_layout": "HND", "rope_theta": theta, "split_tokens": args.split_tokens,
+            "seed": hex(args.seed), "plan": info}, **extra),
         "tokens_per_s": round(B / (ms_per_step * 1e-3), 1),
         "plan_ms_per_model_step": round(plan_ms, 4),
-        "decode_kernel_us": {"mean": round(float(dec_ms.mean()) * 1e3, 3),
-                             "p10": round(float(np.percentile(dec_ms, 10)) * 1e3, 3),
-                             "p50": round(float(np.percentile(dec_ms, 50)) * 1e3, 3),
-                             "p90": round(float(np.percentile(dec_ms, 90)) * 1e3, 3)},
+        "decode_kernel_us": pct(dec_ms),
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": None,
                      "algorithmic_bytes_per_launch": int(alg_bytes),
-                     "kernel": "batch decode (main kernel + split-K combine), HIP events on the launch stream"},
+                     "kernel": "batch decode (decode kernel + split-K combine), HIP events on the launch stream"},
     }
-
     if not args.no_cpu_baseline:
         import oracle  # the checker, used here only as the timed CPU baseline
-        plane0 = pool[:plane].view(torch.int16).cpu().numpy().view(np.uint16)
+        sb = B if name != "C5" else 16  # bounded sample: C5 in full would be minutes of CPU time
+        odt = oracle.E4M3 if fp8 else (oracle.F16 if tdt == torch.float16 else oracle.BF16)
+        plane0 = pool[:plane]
+        plane0 = plane0.cpu().numpy() if fp8 else plane0.view(torch.int16).cpu().numpy().view(np.uint16)
         qh = q.view(torch.int16).cpu().numpy().view(np.uint16)
         sp, sn, sh = wl.strides(BZ_LAYOUT_HND, Hkv, P, D)
-        kv = oracle.PagedKV(plane0, plane0[sp // 2:], indices, indptr, lpl, P, Hkv, D, sp, sn, sh, oracle.BF16)
+        kv = oracle.PagedKV(plane0, plane0[sp // 2:], indices[:int(indptr[sb])], indptr[:sb + 1], lpl[:sb], P, Hkv, D, sp,
+                            sn, sh, odt)
+        ks = k_scale.cpu().numpy() if fp8 else None
+        vs = v_scale.cpu().numpy() if fp8 else None
+        qdt = oracle.F16 if tdt == torch.float16 else oracle.BF16
         t0 = time.perf_counter()
-        ref = oracle.batch_decode(qh, oracle.BF16, kv, Hq, parallel=True)
+        ref = oracle.batch_decode(qh[:sb], qdt, kv, Hq, k_scale=ks, v_scale=vs, parallel=True)
         cpu_s = time.perf_counter() - t0
-        # the same call on the GPU for the same plane, as a last sanity check of what was timed
         pt.set_layer(0, pool_pages)
         out32 = torch.empty((B, Hq, D), dtype=torch.float32, device=dev)
-        K.batch_decode_attention(handler, q, pt, out32, Hq, rope_mode=BZ_ROPE_NONE)
+        K.batch_decode_attention(handler, q, pt, out32, Hq, rope_mode=BZ_ROPE_NONE, k_scale=k_scale, v_scale=v_scale)
         torch.cuda.synchronize()
-        res["max_abs_err_vs_cpu"] = float(np.abs(out32.cpu().numpy() - ref).max())
-        res["cpu_baseline"] = {"value": round(cpu_s * 1e6, 1), "unit": "us/step", "cores": oracle.num_threads(True),
-                               "kind": "port",
-                               "sample": "full C3 batch, decode only (no append), 1 repetition, OpenMP over sequences",
-                               "host_cpus": os.cpu_count()}
+        res_json["max_abs_err_vs_cpu"] = float(np.abs(out32[:sb].cpu().numpy() - ref).max())
+        scale_up = float(ctx.sum()) / float(ctx[:sb].sum())
+        res_json["cpu_baseline"] = {
+            "value": round(cpu_s * scale_up * 1e6, 1), "unit": "us/step", "cores": oracle.num_threads(True),
+            "kind": "port",
+            "sample": f"batch decode only (no append) of the first {sb} of {B} sequences, 1 repetition, OpenMP over "
+                      f"sequences, {cpu_s:.2f} s measured, scaled by total/sample context tokens ({scale_up:.2f}x)",
+            "host_cpus": os.cpu_count()}
+    return res_json
+
+
+def bench_prefill(args):
+    import numpy as np
+    import torch
+
+    from blitz_scale_amd import kernel as K, workloads as wl
+    from blitz_scale_amd._lib import BZ_LAYOUT_HND, BZ_ROPE_NONE
+
+    dev = "cuda"
+    cfg = wl.CONFIGS["C4"]
+    B, Hq, Hkv, D, P, theta = cfg["batch"], cfg["Hq"], cfg["Hkv"], cfg["D"], cfg["P"], cfg["rope_theta"]
+    rng = np.random.default_rng(args.seed)
+    lens = wl.ctx_lens_for(cfg, rng)
+    indptr = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+    N = int(indptr[-1])
+    # page table with the reference's len+1 reservation, seeded page placement
+    need = int(((lens + 1 + P - 1) // P).sum())
+    pool_pages = int(np.ceil(need * cfg["oversub"]))
+    indices, pindptr, lpl = wl.page_table_for(lens + 1, P, pool_pages, rng)
+    stride_page, _, _ = wl.strides(BZ_LAYOUT_HND, Hkv, P, D)
+    steps = args.steps or 20
+    warmup = args.warmup if args.warmup is not None else 3
+    g = torch.Generator(device=dev)
+    g.manual_seed(args.seed)
+    q0 = torch.randn((N, Hq, D), dtype=torch.float16, device=dev, generator=g)
+    k0 = torch.randn((N, Hkv, D), dtype=torch.float16, device=dev, generator=g)
+    v = torch.randn((N, Hkv, D), dtype=torch.float16, device=dev, generator=g)
+    q, k = q0.clone(), k0.clone()
+    out = torch.empty_like(q)
+    pool = torch.zeros(pool_pages * stride_page, dtype=torch.float16, device=dev)
+    pt = K.PageTable(B, P, Hkv, D, pool, layout=BZ_LAYOUT_HND)
+    pt.indices, pt.indptr, pt.last_page_len = indices, pindptr, lpl
+    pt.upload()
+    ip = torch.from_numpy(indptr).to(dev)
+    float_ws = torch.empty(128 << 20, dtype=torch.uint8, device=dev)
+    int_ws = torch.empty(8 << 20, dtype=torch.uint8, device=dev)
+    handler = K.BatchPrefillRaggedHandler()
+    t0 = time.perf_counter()
+    for _ in range(10):
+        handler.plan(float_ws, float_ws.numel(), int_ws, int_ws.numel(), indptr, indptr, B, Hq, Hkv, D, P)
+    torch.cuda.synchronize()
+    plan_ms = (time.perf_counter() - t0) / 10 * 1e3
+
+    def step(i, ev):
+        # fused RoPE (q, k in place) + page store, then attention on the rotated rows.  q and k are rotated
+        # again every step; rotations keep the N(0,1) statistics, so the work is the same each time.
+        K.store_prefill_kv_cache(pt, k, v, ip, num_tokens=N, q=q, num_qo_heads=Hq, rope=True, rope_theta=theta)
+        if ev is not None:
+            ev[0].record()
+        K.batch_prefill_attention(handler, q, ip, k, v, ip, out, B, Hq, Hkv, D, causal=True, rope_mode=BZ_ROPE_NONE)
+        if ev is not None:
+            ev[1].record()
+
+    ms_per_step, att_ms = timed(step, steps, warmup)
+    flops = float(sum(Hq * 4 * D * int(l) * (int(l) + 1) / 2 for l in lens))
+    achieved = flops / (float(att_ms.mean()) * 1e-3) / 1e12
+    res_json = {
+        "metric": "ragged_causal_prefill_ms_per_step", "value": round(ms_per_step, 4), "unit": "ms/step",
+        "n_gpus": 1, "steps": steps, "warmup": warmup, "ms_per_step": round(ms_per_step, 6),
+        "higher_is_better": False, "scaling": "weak", "vs_baseline": None, "dtype": "f16", "data": "synthetic",
+        "config": {"workload": "C4: Llama-2-13B-shaped ragged causal prefill with fused RoPE + KV page store, one layer per step",
+                   "batch": B, "num_qo_heads": Hq, "num_kv_heads": Hkv, "head_dim": D, "page_size": P,
+                   "lens": "uniform[128,4096]", "tokens": N, "pool_pages": pool_pages, "rope_theta": theta,
+                   "seed": hex(args.seed)},
+        "tokens_per_s": round(N / (ms_per_step * 1e-3), 1),
+        "plan_ms_per_model_step": round(plan_ms, 4),
+        "attention_kernel_us": pct(att_ms),
+        "roofline": {"bound": "mfma", "achieved": round(achieved, 1), "peak": MFMA_PEAK_TFLOPS, "unit": "TFLOP/s",
+                     "frac": round(achieved / MFMA_PEAK_TFLOPS, 4), "traffic": None,
+                     "algorithmic_flops_per_launch": flops,
+                     "kernel": "ragged causal prefill attention, HIP events on the launch stream"},
+    }
+    if not args.no_cpu_baseline:
+        import oracle
+        rows = np.sort(rng.choice(N, size=24, replace=False)).astype(np.int32)
+        qh, kh, vh = (t.view(torch.int16).cpu().numpy().view(np.uint16) for t in (q, k, v))
+        K.batch_prefill_attention(handler, q, ip, k, v, ip, out, B, Hq, Hkv, D, causal=True, rope_mode=BZ_ROPE_NONE)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        ref = oracle.batch_prefill_ragged(qh, kh, vh, oracle.F16, indptr, Hq, Hkv, D, causal=True, rows=rows, parallel=True)
+        cpu_s = time.perf_counter() - t0
+        res_json["max_abs_err_vs_cpu"] = float(np.abs(out[torch.from_numpy(rows.astype(np.int64)).to(dev)].float().cpu().numpy() - ref).max())
+        seen = sum(int(r - indptr[np.searchsorted(indptr, r, side="right") - 1]) + 1 for r in rows)
+        total = sum(int(l) * (int(l) + 1) // 2 for l in lens)
+        res_json["cpu_baseline"] = {
+            "value": round(cpu_s * total / seen * 1e3, 1), "unit": "ms/step", "cores": oracle.num_threads(True),
+            "kind": "port",
+            "sample": f"{len(rows)} seeded rows x all heads ({seen} of {total} row-key pairs), attention only, OpenMP "
+                      f"over rows, {cpu_s:.2f} s measured, scaled by pairs",
+            "host_cpus": os.cpu_count()}
+    return res_json
+
+
+def main():
+    args = parse()
+    import torch
+    from blitz_scale_amd import _lib
+    _lib.load()  # fails loudly if the HIP library is not built
+    torch.cuda.set_device(0)
+    res = bench_prefill(args) if args.workload == "C4" else bench_decode(args, args.workload)
     print(json.dumps(res))
 
 
