@@ -289,7 +289,8 @@ static void launch_zero(const DecodePlan* p, void* out, uint32_t row_elems, hipS
 
 int decode_fast_path(const DecodePlan* p, const void* q, void* out, float* lse, int q_dtype, int out_dtype,
                      int rope_mode, float sm_scale_log2, const RopeFreqs& freqs, const bz_paged_kv_t* kv,
-                     uint32_t num_qo_heads, hipStream_t s); // bz_decode_mfma.hip
+                     uint32_t num_qo_heads, const float* k_scale, const float* v_scale,
+                     hipStream_t s); // bz_decode_mfma.hip
 
 } // namespace bz
 
@@ -332,10 +333,9 @@ extern "C" int bz_batch_decode(bz_decode_plan_t* plan_, const void* q, int q_dty
 
     if (p->num_segments > 0) {
         int rc = BZ_ERR_UNSUPPORTED;
-        const bool used_fast = !p->force_general && !k_scale && !v_scale;
-        if (used_fast)
+        if (!p->force_general)
             rc = decode_fast_path(p, q, out, lse, q_dtype, out_dtype, rope_mode, a.sm_scale_log2, a.freqs, kv,
-                                  num_qo_heads, s);
+                                  num_qo_heads, k_scale, v_scale, s);
         if (rc == 0) {
             // the MFMA path brings its own combine; only empty sequences are left to do
             if (p->num_empty > 0) {

@@ -44,6 +44,8 @@ struct MfmaDecodeArgs {
     uint32_t page_size, num_qo_heads, group;
     int rope_q;
     float sm_scale_log2;
+    const float* k_scale; // e4m3 pool only: per-kv-head dequantisation factors (nullptr = 1)
+    const float* v_scale;
     RopeFreqs freqs;
 };
 
@@ -79,6 +81,24 @@ template <> struct Mma<false> {
 
 __device__ __forceinline__ uint32_t& u4(uint4& v, int i) { return reinterpret_cast<uint32_t*>(&v)[i]; }
 
+// Four OCP e4m3 bytes -> four values of the 16-bit MFMA operand type.  Every e4m3 value is exactly
+// representable in f16 and in bf16, so the conversion through fp32 loses nothing.
+template <bool BF16> __device__ __forceinline__ uint2 fp8x4_to_op(uint32_t w) {
+    const auto lo = __builtin_amdgcn_cvt_pk_f32_fp8(w, false);
+    const auto hi = __builtin_amdgcn_cvt_pk_f32_fp8(w, true);
+    if (BF16) { // the upper halves of the two fp32 values, side by side
+        return make_uint2(__builtin_amdgcn_perm(__float_as_uint(lo[1]), __float_as_uint(lo[0]), 0x07060302u),
+                          __builtin_amdgcn_perm(__float_as_uint(hi[1]), __float_as_uint(hi[0]), 0x07060302u));
+    }
+    return make_uint2(Mma<false>::pack2(lo[0], lo[1]), Mma<false>::pack2(hi[0], hi[1]));
+}
+// bytes 8e .. 8e+7 of a 16-byte register -> one 8-element MFMA operand
+template <bool BF16> __device__ __forceinline__ uint4 fp8x8_to_op(const uint4& r, int e) {
+    const uint32_t w0 = e ? r.z : r.x, w1 = e ? r.w : r.y;
+    const uint2 a = fp8x4_to_op<BF16>(w0), b = fp8x4_to_op<BF16>(w1);
+    return make_uint4(a.x, a.y, b.x, b.y);
+}
+
 // The read-only inputs are separate __restrict__ parameters so that wave-uniform reads go through
 // the scalar unit.
 //
@@ -99,7 +119,11 @@ __device__ __forceinline__ void wave_lds_sync() {
 
 constexpr int kInfoInts = 12; // per-tile description kept in LDS (see fetch_info)
 
-template <bool BF16, typename OT, bool ROPE_Q>
+// KV8: the pool holds e4m3 bytes.  K and V are widened to the 16-bit type of q in registers (exactly)
+// on their way to the matrix cores; the per-head scales are folded into the softmax scale and into
+// the final normalisation.  A lane then fetches 16 bytes = 16 elements of a K row, so the contraction
+// index of MFMA step ks, lane group j, element i is d = 64*(ks/2) + 16*j + 8*(ks%2) + i (q follows).
+template <bool BF16, typename OT, bool ROPE_Q, bool KV8>
 __global__ __launch_bounds__(64, 2) void decode_mfma_kernel(MfmaDecodeArgs a, const char* __restrict__ q_ptr,
                                                             const char* __restrict__ k_data,
                                                             const char* __restrict__ v_data,
@@ -115,7 +139,9 @@ __global__ __launch_bounds__(64, 2) void decode_mfma_kernel(MfmaDecodeArgs a, co
     const int n = lane & 15; // query head (scores) / d column (output) / token row (K operand)
     const int j = lane >> 4; // lane group: which 8-wide slice of the MFMA contraction
     const int P = (int)a.page_size;
-    const size_t row_bytes = (size_t)a.stride_n * 2;
+    constexpr int ES = KV8 ? 1 : 2; // bytes per pool element
+    const size_t row_bytes = (size_t)a.stride_n * ES;
+    auto d_of = [&](int ks) { return KV8 ? 64 * (ks >> 1) + 16 * j + 8 * (ks & 1) : 32 * ks + 8 * j; };
     const int G = (int)a.group;
 
     const int g_begin = tile_ptr[blockIdx.x], g_end = tile_ptr[blockIdx.x + 1];
@@ -179,17 +205,30 @@ __global__ __launch_bounds__(64, 2) void decode_mfma_kernel(MfmaDecodeArgs a, co
 #pragma unroll
         for (int s = 0; s < 2; ++s) {
             const int slot0 = (u.t * kTileTok + 16 * s) % P; // a subtile past the last page reads the last page, masked later
-            base[s] = ((size_t)pid[s] * a.stride_page + (size_t)slot0 * a.stride_n + (size_t)u.kvh * a.stride_h) * 2;
+            base[s] = ((size_t)pid[s] * a.stride_page + (size_t)slot0 * a.stride_n + (size_t)u.kvh * a.stride_h) * ES;
         }
+        if constexpr (KV8) {
 #pragma unroll
-        for (int ks = 0; ks < 4; ++ks) {
-            kreg[0][ks] = *reinterpret_cast<const uint4*>(k_data + base[0] + (size_t)n * row_bytes + ks * 64 + j * 16);
-            kreg[1][ks] = *reinterpret_cast<const uint4*>(k_data + base[1] + (size_t)n * row_bytes + ks * 64 + j * 16);
-        }
+            for (int p = 0; p < 2; ++p) { // 16 bytes feed MFMA steps 2p and 2p+1
+                kreg[0][p] = *reinterpret_cast<const uint4*>(k_data + base[0] + (size_t)n * row_bytes + p * 64 + j * 16);
+                kreg[1][p] = *reinterpret_cast<const uint4*>(k_data + base[1] + (size_t)n * row_bytes + p * 64 + j * 16);
+            }
 #pragma unroll
-        for (int w = 0; w < 8; ++w) { // rows 4w..4w+3 of the tile, 16 lanes x 16 B per row
-            const int row = 4 * w + j;
-            vreg[w] = *reinterpret_cast<const uint4*>(v_data + base[row >> 4] + (size_t)(row & 15) * row_bytes + n * 16);
+            for (int w = 0; w < 4; ++w) { // rows 8w..8w+7 of the tile, 8 lanes x 16 B per 128-byte row
+                const int row = 8 * w + (lane >> 3);
+                vreg[w] = *reinterpret_cast<const uint4*>(v_data + base[row >> 4] + (size_t)(row & 15) * row_bytes + (lane & 7) * 16);
+            }
+        } else {
+#pragma unroll
+            for (int ks = 0; ks < 4; ++ks) {
+                kreg[0][ks] = *reinterpret_cast<const uint4*>(k_data + base[0] + (size_t)n * row_bytes + ks * 64 + j * 16);
+                kreg[1][ks] = *reinterpret_cast<const uint4*>(k_data + base[1] + (size_t)n * row_bytes + ks * 64 + j * 16);
+            }
+#pragma unroll
+            for (int w = 0; w < 8; ++w) { // rows 4w..4w+3 of the tile, 16 lanes x 16 B per row
+                const int row = 4 * w + j;
+                vreg[w] = *reinterpret_cast<const uint4*>(v_data + base[row >> 4] + (size_t)(row & 15) * row_bytes + n * 16);
+            }
         }
     };
     // q rows of a piece as MFMA B operand: lane (head n, group j) holds q[head][32*ks + 8*j .. +7]
@@ -199,7 +238,7 @@ __global__ __launch_bounds__(64, 2) void decode_mfma_kernel(MfmaDecodeArgs a, co
         if (n < G) {
             const char* qrow = q_ptr + ((size_t)u.seq * a.num_qo_heads + (size_t)u.kvh * G + n) * 256;
 #pragma unroll
-            for (int ks = 0; ks < 4; ++ks) qnext[ks] = *reinterpret_cast<const uint4*>(qrow + ks * 64 + j * 16);
+            for (int ks = 0; ks < 4; ++ks) qnext[ks] = *reinterpret_cast<const uint4*>(qrow + d_of(ks) * 2);
         }
     };
 
@@ -226,6 +265,7 @@ __global__ __launch_bounds__(64, 2) void decode_mfma_kernel(MfmaDecodeArgs a, co
         if (i == 8 && chunk_base + 32 < g_end) dnext = fetch_info(chunk_base + 32);
         if (i == 24 && chunk_base + 32 < g_end) { stash_info(dnext, buf ^ 1); wave_lds_sync(); }
         const int t = uc.t, tok_end = uc.tok_end, seq_len = uc.seq_len;
+        const float score_scale = a.sm_scale_log2 * ((KV8 && a.k_scale) ? a.k_scale[uc.kvh] : 1.0f);
 
         if (uc.flags & 1) { // ================= first tile of a piece =================
 #pragma unroll
@@ -244,7 +284,7 @@ __global__ __launch_bounds__(64, 2) void decode_mfma_kernel(MfmaDecodeArgs a, co
 #pragma unroll
                         for (int e = 0; e < 2; ++e) {
                             float s, c;
-                            sincosf(pos * a.freqs.f[32 * ks + 8 * j + 2 * w + e], &s, &c);
+                            sincosf(pos * a.freqs.f[d_of(ks) + 2 * w + e], &s, &c);
                             xr[e] = x[e] * c - y[e] * s;
                             yr[e] = y[e] * c + x[e] * s;
                         }
@@ -272,18 +312,33 @@ __global__ __launch_bounds__(64, 2) void decode_mfma_kernel(MfmaDecodeArgs a, co
           for (int w = 0; w < 8; ++w) x ^= vreg[w].x ^ vreg[w].y ^ vreg[w].z ^ vreg[w].w;
           acc[1][0] += __uint_as_float(x & 0x3fffffu); }
 #else
+        if constexpr (KV8) {
 #pragma unroll
-        for (int w = 0; w < 8; ++w) {
-            uint4 v = vreg[w];
-            if (ragged && tile_tok0 + 4 * w + j >= tok_end) v = make_uint4(0, 0, 0, 0); // 0 * garbage must be 0
-            *reinterpret_cast<uint4*>(v_lds + (4 * w + j) * kVRowBytes + n * 16) = v;
+            for (int w = 0; w < 4; ++w) { // 16 e4m3 bytes -> 16 operand-type values -> 32 B of the LDS row
+                uint4 v = vreg[w];
+                const int row = 8 * w + (lane >> 3);
+                if (ragged && tile_tok0 + row >= tok_end) v = make_uint4(0, 0, 0, 0); // 0 * garbage must be 0
+                unsigned char* dst = v_lds + row * kVRowBytes + (lane & 7) * 32;
+                *reinterpret_cast<uint4*>(dst) = fp8x8_to_op<BF16>(v, 0);
+                *reinterpret_cast<uint4*>(dst + 16) = fp8x8_to_op<BF16>(v, 1);
+            }
+        } else {
+#pragma unroll
+            for (int w = 0; w < 8; ++w) {
+                uint4 v = vreg[w];
+                if (ragged && tile_tok0 + 4 * w + j >= tok_end) v = make_uint4(0, 0, 0, 0); // 0 * garbage must be 0
+                *reinterpret_cast<uint4*>(v_lds + (4 * w + j) * kVRowBytes + n * 16) = v;
+            }
         }
 #endif
         uint4 kcur[2][4];
 #pragma unroll
         for (int u = 0; u < 2; ++u)
 #pragma unroll
-            for (int ks = 0; ks < 4; ++ks) kcur[u][ks] = kreg[u][ks];
+            for (int ks = 0; ks < 4; ++ks) {
+                if constexpr (KV8) kcur[u][ks] = fp8x8_to_op<BF16>(kreg[u][ks >> 1], ks & 1);
+                else kcur[u][ks] = kreg[u][ks];
+            }
         if (g + 1 < g_end) {
             if (i + 1 == 32) { chunk_base += 32; buf ^= 1; }
             un = read_info(buf, (g + 1) - chunk_base);
@@ -320,7 +375,7 @@ __global__ __launch_bounds__(64, 2) void decode_mfma_kernel(MfmaDecodeArgs a, co
         for (int u = 0; u < 2; ++u)
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
-                float v = s[u][r] * a.sm_scale_log2;
+                float v = s[u][r] * score_scale;
                 if (ragged && tile_tok0 + 16 * u + 4 * j + r >= tok_end) v = -INFINITY;
                 s[u][r] = v;
                 tmax = fmaxf(tmax, v);
@@ -388,7 +443,7 @@ __global__ __launch_bounds__(64, 2) void decode_mfma_kernel(MfmaDecodeArgs a, co
             ++exp_pieces;
 #endif
             const int b = uc.seq, kvh = uc.kvh, partial = uc.partial;
-            const float inv_l = l_run > 0.f ? 1.0f / l_run : 0.f;
+            const float inv_l = (l_run > 0.f ? 1.0f / l_run : 0.f) * ((KV8 && a.v_scale) ? a.v_scale[kvh] : 1.0f);
             const float lse2 = l_run > 0.f ? m_run + log2f(l_run) : -INFINITY;
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
@@ -471,16 +526,21 @@ __global__ __launch_bounds__(128) void decode_mfma_combine_kernel(const MfmaComb
 
 struct DecodeArgs; // general-kernel argument block (bz_decode.hip); only its scalar fields are forwarded here
 
-template <bool BF16, typename OT, bool ROPE_Q>
+template <bool BF16, typename OT, bool ROPE_Q, bool KV8>
 static void launch_mfma_k(const DecodePlan* p, const MfmaDecodeArgs& a, hipStream_t s) {
-    hipLaunchKernelGGL((decode_mfma_kernel<BF16, OT, ROPE_Q>), dim3(p->mfma_slots), dim3(64), 0, s, a,
+    hipLaunchKernelGGL((decode_mfma_kernel<BF16, OT, ROPE_Q, KV8>), dim3(p->mfma_slots), dim3(64), 0, s, a,
                        (const char*)a.q, a.k_data, a.v_data, a.indices, a.pieces, a.tiles, a.tile_ptr);
 }
 
 template <bool BF16, typename OT>
-static int launch_mfma(const DecodePlan* p, const MfmaDecodeArgs& a, hipStream_t s) {
-    if (a.rope_q) launch_mfma_k<BF16, OT, true>(p, a, s);
-    else launch_mfma_k<BF16, OT, false>(p, a, s);
+static int launch_mfma(const DecodePlan* p, const MfmaDecodeArgs& a, bool kv8, hipStream_t s) {
+    if (kv8) {
+        if (a.rope_q) launch_mfma_k<BF16, OT, true, true>(p, a, s);
+        else launch_mfma_k<BF16, OT, false, true>(p, a, s);
+    } else {
+        if (a.rope_q) launch_mfma_k<BF16, OT, true, false>(p, a, s);
+        else launch_mfma_k<BF16, OT, false, false>(p, a, s);
+    }
     BZ_LAUNCH_CHECK();
     if (p->mfma_combos > 0) {
         hipLaunchKernelGGL((decode_mfma_combine_kernel<OT>), dim3(p->mfma_combos, a.group), dim3(128), 0, s,
@@ -492,10 +552,13 @@ static int launch_mfma(const DecodePlan* p, const MfmaDecodeArgs& a, hipStream_t
 
 int decode_fast_path(const DecodePlan* p, const void* q, void* out, float* lse, int q_dtype, int out_dtype,
                      int rope_mode, float sm_scale_log2, const RopeFreqs& freqs, const bz_paged_kv_t* kv,
-                     uint32_t num_qo_heads, hipStream_t s) {
+                     uint32_t num_qo_heads, const float* k_scale, const float* v_scale, hipStream_t s) {
     if (!p->mfma_ok || p->mfma_slots == 0) return BZ_ERR_UNSUPPORTED;
-    if (kv->kv_dtype != q_dtype || rope_mode == BZ_ROPE_FULL) return BZ_ERR_UNSUPPORTED;
-    if ((kv->stride_n * 2) % 16 || (kv->stride_h * 2) % 16 || (kv->stride_page * 2) % 16) return BZ_ERR_UNSUPPORTED;
+    const bool kv8 = kv->kv_dtype == BZ_E4M3;
+    if ((!kv8 && kv->kv_dtype != q_dtype) || rope_mode == BZ_ROPE_FULL) return BZ_ERR_UNSUPPORTED;
+    if (!kv8 && (k_scale || v_scale)) return BZ_ERR_UNSUPPORTED;
+    const uint64_t es = kv8 ? 1 : 2;
+    if ((kv->stride_n * es) % 16 || (kv->stride_h * es) % 16 || (kv->stride_page * es) % 16) return BZ_ERR_UNSUPPORTED;
     if (((uintptr_t)kv->k_data | (uintptr_t)kv->v_data | (uintptr_t)q) % 16) return BZ_ERR_UNSUPPORTED;
     MfmaDecodeArgs a;
     a.q = q; a.out = out; a.lse = lse;
@@ -507,10 +570,11 @@ int decode_fast_path(const DecodePlan* p, const void* q, void* out, float* lse, 
     a.page_size = kv->page_size; a.num_qo_heads = num_qo_heads; a.group = num_qo_heads / kv->num_kv_heads;
     a.rope_q = rope_mode == BZ_ROPE_Q_ONLY;
     a.sm_scale_log2 = sm_scale_log2;
+    a.k_scale = k_scale; a.v_scale = v_scale;
     a.freqs = freqs;
     if (q_dtype == BZ_BF16)
-        return out_dtype == BZ_F32 ? launch_mfma<true, float>(p, a, s) : launch_mfma<true, bf16_t>(p, a, s);
-    return out_dtype == BZ_F32 ? launch_mfma<false, float>(p, a, s) : launch_mfma<false, f16_t>(p, a, s);
+        return out_dtype == BZ_F32 ? launch_mfma<true, float>(p, a, kv8, s) : launch_mfma<true, bf16_t>(p, a, kv8, s);
+    return out_dtype == BZ_F32 ? launch_mfma<false, float>(p, a, kv8, s) : launch_mfma<false, f16_t>(p, a, kv8, s);
 }
 
 } // namespace bz
