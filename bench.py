@@ -35,6 +35,8 @@ def parse():
     ap.add_argument("--sigma", type=float, default=1.0, help="sigma of the log-normal context lengths (C3)")
     ap.add_argument("--split-tokens", type=int, default=2048)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also launch a few plain device copies of 1 GiB (reference point for rocprofv3 --pmc byte counters)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on ONE GPU (--gpus 1); the path shards by kv head / by sequence "
@@ -314,6 +316,13 @@ def main():
     from blitz_scale_amd import _lib
     _lib.load()  # fails loudly if the HIP library is not built
     torch.cuda.set_device(0)
+    if args.calibrate_copy:
+        src = torch.empty(1 << 29, dtype=torch.bfloat16, device="cuda").normal_()  # 1 GiB read + 1 GiB written per copy
+        dst = torch.empty_like(src)
+        for _ in range(5):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
     res = bench_prefill(args) if args.workload == "C4" else bench_decode(args, args.workload)
     print(json.dumps(res))
 

@@ -35,11 +35,11 @@ constexpr int kVRow = 320;     // LDS row stride of the V tile (256 B + 64: 4 ro
 constexpr int kKTile = kBN * kKRow;
 constexpr int kVTile = kBN * kVRow;
 
-struct PrefillItem {
+struct PrefillItem { // one workgroup's job, in launch order
     int32_t tok0; // global index of the request's first token
-    int32_t len;  // tokens in the request
+    int32_t len;  // tokens in the request (0: padding entry, nothing to do)
     int32_t q0;   // first q row of this tile, relative to the request
-    int32_t pad;
+    int32_t head; // q head
 };
 
 struct PrefillPlan {
@@ -99,7 +99,8 @@ __global__ __launch_bounds__(256, 2) void prefill_kernel(PrefillArgs a, const ch
     unsigned char* v_lds = smem + 2 * kKTile; // [2][kVTile]
 
     const PrefillItem it = a.items[blockIdx.x];
-    const int head = blockIdx.y;
+    if (it.len <= 0) return;
+    const int head = it.head;
     const int Hq = (int)a.num_qo_heads, Hkv = (int)a.num_kv_heads;
     const int kvh = head / (Hq / Hkv);
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
@@ -176,18 +177,27 @@ __global__ __launch_bounds__(256, 2) void prefill_kernel(PrefillArgs a, const ch
             // ---- scale, mask, online softmax.  Element 4b+r of block kb is token kv0 + 32kb + 8b + 4h + r.
             const bool need_mask = (a.causal && kv0 + kBN - 1 > wave_q_lo) || (kv0 + kBN > L);
             float tmax = -INFINITY;
+            if (need_mask) { // wave-uniform; selects, not branches, per element
+                const int kv_max = a.causal ? min(q_pos, L - 1) : L - 1; // last token this row may see
 #pragma unroll
-            for (int kb = 0; kb < 2; ++kb)
+                for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
-                for (int i = 0; i < 16; ++i) {
-                    float v = s[kb][i] * a.sm_scale_log2;
-                    if (need_mask) {
+                    for (int i = 0; i < 16; ++i) {
                         const int kv = kv0 + 32 * kb + 8 * (i >> 2) + 4 * h + (i & 3);
-                        if (kv >= L || (a.causal && kv > q_pos)) v = -INFINITY;
+                        const float v = kv > kv_max ? -INFINITY : s[kb][i] * a.sm_scale_log2;
+                        s[kb][i] = v;
+                        tmax = fmaxf(tmax, v);
                     }
-                    s[kb][i] = v;
-                    tmax = fmaxf(tmax, v);
-                }
+            } else {
+#pragma unroll
+                for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+                    for (int i = 0; i < 16; ++i) {
+                        const float v = s[kb][i] * a.sm_scale_log2;
+                        s[kb][i] = v;
+                        tmax = fmaxf(tmax, v);
+                    }
+            }
             tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
             const float m_new = fmaxf(m_run, tmax); // finite from the first tile on: token 0 is visible to every row
             const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
@@ -210,10 +220,12 @@ __global__ __launch_bounds__(256, 2) void prefill_kernel(PrefillArgs a, const ch
             psum += __shfl_xor(psum, 32, 64);
             l_run = l_run * alpha + psum;
             m_run = m_new;
+            if (__any(alpha != 1.0f)) { // the running maximum settles after a few tiles
 #pragma unroll
-            for (int db = 0; db < 4; ++db)
+                for (int db = 0; db < 4; ++db)
 #pragma unroll
-                for (int i = 0; i < 16; ++i) acc[db][i] *= alpha;
+                    for (int i = 0; i < 16; ++i) acc[db][i] *= alpha;
+            }
 
             // ---- O^T += V^T P^T.  A operand through the transposing LDS read: a 16-lane group fetches
             // 4 token rows x 16 d columns and every lane ends up with the 4 tokens of its own d column.
@@ -363,16 +375,35 @@ extern "C" int bz_prefill_plan(bz_prefill_plan_t* plan_, void* float_buffer, siz
     // self-attention only: the reference passes the same array twice (src/layer/attn.h:175-187)
     for (uint32_t b = 0; b <= batch_size; ++b)
         if (qo_indptr_h[b] != kv_indptr_h[b]) return BZ_ERR_UNSUPPORTED;
-    std::vector<PrefillItem> items;
-    for (uint32_t b = 0; b < batch_size; ++b) {
-        const int32_t len = qo_indptr_h[b + 1] - qo_indptr_h[b];
-        if (len < 0) return BZ_ERR_BAD_ARG;
-        for (int32_t q0 = 0; q0 < len; q0 += kBM) items.push_back({qo_indptr_h[b], len, q0, 0});
-    }
-    // longest first: a tile's work grows with the number of tokens its rows can see
-    std::stable_sort(items.begin(), items.end(), [](const PrefillItem& x, const PrefillItem& y) {
-        return std::min(x.len, x.q0 + kBM) > std::min(y.len, y.q0 + kBM);
+    // One entry per workgroup, in launch order.  Workgroups are dealt round-robin to the 8 XCDs, each
+    // with its own L2, so launch index i runs on XCD i % 8.  Every (request, q head) pair is given to one
+    // XCD as a run of consecutive jobs: its q tiles then execute together on that XCD and share the
+    // pair's K/V (up to 2 MiB for 4096 tokens) through that L2 instead of each fetching it from HBM.
+    // Pairs go to the XCDs in turn, longest requests first and tiles from the last (most keys) to the
+    // first, so every XCD gets the same mix of work.
+    for (uint32_t b = 0; b < batch_size; ++b)
+        if (qo_indptr_h[b + 1] < qo_indptr_h[b]) return BZ_ERR_BAD_ARG;
+    std::vector<uint32_t> order(batch_size);
+    for (uint32_t b = 0; b < batch_size; ++b) order[b] = b;
+    std::stable_sort(order.begin(), order.end(), [&](uint32_t x, uint32_t y) {
+        return qo_indptr_h[x + 1] - qo_indptr_h[x] > qo_indptr_h[y + 1] - qo_indptr_h[y];
     });
+    constexpr int kXcd = 8;
+    std::vector<PrefillItem> per_xcd[kXcd];
+    uint32_t pair = 0;
+    for (uint32_t b : order) {
+        const int32_t len = qo_indptr_h[b + 1] - qo_indptr_h[b];
+        if (len == 0) continue;
+        const int32_t last_q0 = (len - 1) / kBM * kBM;
+        for (uint32_t h = 0; h < num_qo_heads; ++h, ++pair)
+            for (int32_t q0 = last_q0; q0 >= 0; q0 -= kBM)
+                per_xcd[pair % kXcd].push_back({qo_indptr_h[b], len, q0, (int32_t)h});
+    }
+    size_t longest = 0;
+    for (auto& v : per_xcd) longest = std::max(longest, v.size());
+    std::vector<PrefillItem> items(longest * kXcd, PrefillItem{0, 0, 0, 0});
+    for (int x = 0; x < kXcd; ++x)
+        for (size_t k = 0; k < per_xcd[x].size(); ++k) items[k * kXcd + x] = per_xcd[x][k];
     const size_t bytes = pf_align_up(items.size() * sizeof(PrefillItem), 256);
     if (bytes > int_buffer_bytes) return BZ_ERR_WORKSPACE;
     hipStream_t s = (hipStream_t)stream;
@@ -411,7 +442,7 @@ static int launch_prefill(const PrefillPlan* p, const PrefillArgs& a, const void
         BZ_CHECK_HIP(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
         attr_done = true;
     }
-    hipLaunchKernelGGL(kern, dim3(p->num_items, a.num_qo_heads), dim3(256), smem, s, a, (const char*)q, (const char*)k,
+    hipLaunchKernelGGL(kern, dim3(p->num_items), dim3(256), smem, s, a, (const char*)q, (const char*)k,
                        (const char*)v);
     BZ_LAUNCH_CHECK();
     return 0;
