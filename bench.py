@@ -44,15 +44,39 @@ def parse():
     return args
 
 
+class HipEvents:
+    """Plain HIP events (ctypes on the HIP runtime torch already loaded), for timing a launch on the
+    stream it is issued to from inside the library."""
+
+    def __init__(self, n):
+        import ctypes as C
+        self.C = C
+        self.hip = C.CDLL("libamdhip64.so")
+        self.ev = []
+        for _ in range(2 * n):
+            e = C.c_void_p()
+            assert self.hip.hipEventCreate(C.byref(e)) == 0
+            self.ev.append(e)
+
+    def pair(self, i):
+        return self.ev[2 * i], self.ev[2 * i + 1]
+
+    def elapsed_ms(self, i):
+        ms = self.C.c_float()
+        assert self.hip.hipEventElapsedTime(self.C.byref(ms), self.ev[2 * i], self.ev[2 * i + 1]) == 0
+        return ms.value
+
+
 def pct(a):
     import numpy as np
     return {"mean": round(float(a.mean()) * 1e3, 3), "p10": round(float(np.percentile(a, 10)) * 1e3, 3),
             "p50": round(float(np.percentile(a, 50)) * 1e3, 3), "p90": round(float(np.percentile(a, 90)) * 1e3, 3)}
 
 
-def timed(step, steps, warmup):
-    """W untimed steps, then exactly K steps between two device synchronisations; per-step HIP event pairs
-    (torch's current stream is the stream every launch goes to) bracket the dominant kernel."""
+def timed(step, steps, warmup, torch_events=True):
+    """W untimed steps, then exactly K steps between two device synchronisations.  step(i, ev) gets a pair
+    of torch events (recorded on torch's current stream, the stream every launch goes to) to bracket the
+    dominant kernel, or True when the step brings its own events."""
     import numpy as np
     import torch
     for i in range(warmup):
@@ -62,10 +86,22 @@ def timed(step, steps, warmup):
     torch.cuda.synchronize()
     t0 = time.perf_counter()
     for i in range(steps):
-        step(i, events[i])
+        step(i, events[i] if torch_events else True)
     torch.cuda.synchronize()
     elapsed = time.perf_counter() - t0
-    return elapsed / steps * 1e3, np.array([a.elapsed_time(b) for a, b in events])
+    return elapsed / steps * 1e3, (np.array([a.elapsed_time(b) for a, b in events]) if torch_events else None)
+
+
+def measured_traffic(name, args):
+    """HBM bytes per launch of the dominant kernel, measured offline with rocprofv3 --pmc (profiles/*.md);
+    only reported for the exact workload it was measured on."""
+    if args.seed != 0x5EED or args.sigma != 1.0 or args.split_tokens != 2048:
+        return None
+    try:
+        with open(os.path.join(ROOT, "blitz_scale_amd", "measured_traffic.json")) as f:
+            return json.load(f)["bytes_per_launch"].get(name)
+    except OSError:
+        return None
 
 
 def bench_decode(args, name):
@@ -148,22 +184,35 @@ def bench_decode(args, name):
         act = torch.empty((B, I), dtype=tdt, device=dev)
         extra = {"hidden": h, "inter": I}
 
+    kev = HipEvents(steps)  # recorded by the library around the decode kernel launch itself
+
     def step(i, ev):
         pt.set_layer(i % L, pool_pages)
         K.append_decode_kv_cache(pt, k_new, v_new, q=q, num_qo_heads=Hq, rope=theta is not None,
                                  rope_theta=theta or 1e4, k_scale=k_scale, v_scale=v_scale)
-        if ev is not None:
-            ev[0].record()
+        if ev == "call":      # informational pass: torch events around the whole decode call
+            call_ev[i][0].record()
+        elif ev is not None:  # timed pass: the library records a HIP event pair around the decode kernel launch
+            handler.set_timing_events(*kev.pair(i))
         K.batch_decode_attention(handler, q, pt, out, Hq, rope_mode=BZ_ROPE_NONE, k_scale=k_scale, v_scale=v_scale)
-        if ev is not None:
-            ev[1].record()
+        if ev == "call":
+            call_ev[i][1].record()
         if name == "C2":
             K.add_rms_norm(x, res, w, B, h)
             K.silu_and_mul(gate_up, act, B, I)
 
-    ms_per_step, dec_ms = timed(step, steps, warmup)
+    ms_per_step, _ = timed(step, steps, warmup, torch_events=False)
+    handler.set_timing_events(None, None)
+    kern_ms = np.array([kev.elapsed_ms(i) for i in range(steps)])
+    ncall = min(steps, 100)
+    call_ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(ncall)]
+    for i in range(ncall):
+        step(i, "call")
+    torch.cuda.synchronize()
+    dec_ms = np.array([a.elapsed_time(b) for a, b in call_ev])
     alg_bytes = wl.decode_algorithmic_bytes(ctx, Hq, Hkv, D, kv_bytes, 2, P)
-    achieved = alg_bytes / (float(dec_ms.mean()) * 1e-3) / 1e9
+    achieved = alg_bytes / (float(kern_ms.mean()) * 1e-3) / 1e9
+    traffic = measured_traffic(name, args)
     res_json = {
         "metric": "paged_decode_us_per_step", "value": round(ms_per_step * 1e3, 3), "unit": "us/step",
         "n_gpus": 1, "steps": steps, "warmup": warmup, "ms_per_step": round(ms_per_step, 6),
@@ -181,11 +230,13 @@ def bench_decode(args, name):
             "seed": hex(args.seed), "plan": info}, **extra),
         "tokens_per_s": round(B / (ms_per_step * 1e-3), 1),
         "plan_ms_per_model_step": round(plan_ms, 4),
-        "decode_kernel_us": pct(dec_ms),
+        "decode_call_us": pct(dec_ms),
+        "decode_kernel_us": pct(kern_ms),
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                     "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": None,
+                     "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": traffic,
                      "algorithmic_bytes_per_launch": int(alg_bytes),
-                     "kernel": "batch decode (decode kernel + split-K combine), HIP events on the launch stream"},
+                     "kernel": "decode kernel (bz::decode_mfma_kernel), HIP events recorded by the library on the launch "
+                               "stream right around its launch; decode_call_us also holds the split-K combine launch"},
     }
     if not args.no_cpu_baseline:
         import oracle  # the checker, used here only as the timed CPU baseline
@@ -200,9 +251,11 @@ def bench_decode(args, name):
         ks = k_scale.cpu().numpy() if fp8 else None
         vs = v_scale.cpu().numpy() if fp8 else None
         qdt = oracle.F16 if tdt == torch.float16 else oracle.BF16
-        t0 = time.perf_counter()
-        ref = oracle.batch_decode(qh[:sb], qdt, kv, Hq, k_scale=ks, v_scale=vs, parallel=True)
-        cpu_s = time.perf_counter() - t0
+        reps, t0 = 0, time.perf_counter()
+        while reps == 0 or (time.perf_counter() - t0 < 10.0 and reps < 200):  # about 10 s of CPU work
+            ref = oracle.batch_decode(qh[:sb], qdt, kv, Hq, k_scale=ks, v_scale=vs, parallel=True)
+            reps += 1
+        cpu_s = (time.perf_counter() - t0) / reps
         pt.set_layer(0, pool_pages)
         out32 = torch.empty((B, Hq, D), dtype=torch.float32, device=dev)
         K.batch_decode_attention(handler, q, pt, out32, Hq, rope_mode=BZ_ROPE_NONE, k_scale=k_scale, v_scale=v_scale)
@@ -212,8 +265,8 @@ def bench_decode(args, name):
         res_json["cpu_baseline"] = {
             "value": round(cpu_s * scale_up * 1e6, 1), "unit": "us/step", "cores": oracle.num_threads(True),
             "kind": "port",
-            "sample": f"batch decode only (no append) of the first {sb} of {B} sequences, 1 repetition, OpenMP over "
-                      f"sequences, {cpu_s:.2f} s measured, scaled by total/sample context tokens ({scale_up:.2f}x)",
+            "sample": f"batch decode only (no append) of the first {sb} of {B} sequences, mean of {reps} repetitions "
+                      f"({cpu_s:.2f} s each), OpenMP over sequences, scaled by total/sample context tokens ({scale_up:.2f}x)",
             "host_cpus": os.cpu_count()}
     return res_json
 
@@ -285,7 +338,7 @@ def bench_prefill(args):
         "plan_ms_per_model_step": round(plan_ms, 4),
         "attention_kernel_us": pct(att_ms),
         "roofline": {"bound": "mfma", "achieved": round(achieved, 1), "peak": MFMA_PEAK_TFLOPS, "unit": "TFLOP/s",
-                     "frac": round(achieved / MFMA_PEAK_TFLOPS, 4), "traffic": None,
+                     "frac": round(achieved / MFMA_PEAK_TFLOPS, 4), "traffic": measured_traffic("C4", args),
                      "algorithmic_flops_per_launch": flops,
                      "kernel": "ragged causal prefill attention, HIP events on the launch stream"},
     }

@@ -349,12 +349,14 @@ extern "C" int bz_batch_decode(bz_decode_plan_t* plan_, const void* q, int q_dty
         }
         if (rc == BZ_ERR_UNSUPPORTED) {
             dim3 grid(p->num_segments, kv->num_kv_heads);
+            if (p->time_start) BZ_CHECK_HIP(hipEventRecord(p->time_start, s));
             if (q_dtype == BZ_F16)
                 rc = (out_dtype == BZ_F32) ? launch_general_kv<f16_t, float>(a, kv->kv_dtype, q_dtype, D, G, grid, s)
                                            : launch_general_kv<f16_t, f16_t>(a, kv->kv_dtype, q_dtype, D, G, grid, s);
             else
                 rc = (out_dtype == BZ_F32) ? launch_general_kv<bf16_t, float>(a, kv->kv_dtype, q_dtype, D, G, grid, s)
                                            : launch_general_kv<bf16_t, bf16_t>(a, kv->kv_dtype, q_dtype, D, G, grid, s);
+            if (rc == 0 && p->time_stop) BZ_CHECK_HIP(hipEventRecord(p->time_stop, s));
         }
         if (rc) return rc;
     }

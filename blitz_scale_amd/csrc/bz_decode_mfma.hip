@@ -534,6 +534,7 @@ static void launch_mfma_k(const DecodePlan* p, const MfmaDecodeArgs& a, hipStrea
 
 template <bool BF16, typename OT>
 static int launch_mfma(const DecodePlan* p, const MfmaDecodeArgs& a, bool kv8, hipStream_t s) {
+    if (p->time_start) BZ_CHECK_HIP(hipEventRecord(p->time_start, s));
     if (kv8) {
         if (a.rope_q) launch_mfma_k<BF16, OT, true, true>(p, a, s);
         else launch_mfma_k<BF16, OT, false, true>(p, a, s);
@@ -542,6 +543,7 @@ static int launch_mfma(const DecodePlan* p, const MfmaDecodeArgs& a, bool kv8, h
         else launch_mfma_k<BF16, OT, false, false>(p, a, s);
     }
     BZ_LAUNCH_CHECK();
+    if (p->time_stop) BZ_CHECK_HIP(hipEventRecord(p->time_stop, s));
     if (p->mfma_combos > 0) {
         hipLaunchKernelGGL((decode_mfma_combine_kernel<OT>), dim3(p->mfma_combos, a.group), dim3(128), 0, s,
                            p->mfma_combos_d, a.part_o, a.part_lse, a.out, a.lse, a.num_qo_heads, a.group);

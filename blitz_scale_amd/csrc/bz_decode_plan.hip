@@ -282,3 +282,11 @@ extern "C" int bz_decode_plan_info(const bz_decode_plan_t* plan_, uint32_t* num_
     if (num_workgroups) *num_workgroups = mfma ? p->mfma_slots : p->num_workgroups;
     return 0;
 }
+
+extern "C" int bz_decode_plan_set_timing_events(bz_decode_plan_t* plan_, void* start_event, void* stop_event) {
+    DecodePlan* p = reinterpret_cast<DecodePlan*>(plan_);
+    if (!p || ((start_event == nullptr) != (stop_event == nullptr))) return BZ_ERR_BAD_ARG;
+    p->time_start = (hipEvent_t)start_event;
+    p->time_stop = (hipEvent_t)stop_event;
+    return 0;
+}

@@ -68,6 +68,7 @@ struct DecodePlan {
     void* staging = nullptr;
     size_t staging_bytes = 0;
     hipEvent_t upload_done = nullptr;
+    hipEvent_t time_start = nullptr, time_stop = nullptr; // optional: bracket the decode kernel launch
     int device = -1;
 };
 

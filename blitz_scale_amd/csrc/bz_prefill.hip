@@ -184,7 +184,7 @@ __global__ __launch_bounds__(256, 2) void prefill_kernel(PrefillArgs a, const ch
 #pragma unroll
                     for (int i = 0; i < 16; ++i) {
                         const int kv = kv0 + 32 * kb + 8 * (i >> 2) + 4 * h + (i & 3);
-                        const float v = kv > kv_max ? -INFINITY : s[kb][i] * a.sm_scale_log2;
+                        const float v = kv > kv_max ? -INFINITY : s[kb][i];
                         s[kb][i] = v;
                         tmax = fmaxf(tmax, v);
                     }
@@ -192,13 +192,11 @@ __global__ __launch_bounds__(256, 2) void prefill_kernel(PrefillArgs a, const ch
 #pragma unroll
                 for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
-                    for (int i = 0; i < 16; ++i) {
-                        const float v = s[kb][i] * a.sm_scale_log2;
-                        s[kb][i] = v;
-                        tmax = fmaxf(tmax, v);
-                    }
+                    for (int i = 0; i < 16; ++i) tmax = fmaxf(tmax, s[kb][i]);
             }
-            tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
+            // the scores stay unscaled in registers: the (positive) softmax scale is applied to the maximum
+            // here and to every score inside the fused multiply-add that feeds exp2
+            tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64)) * a.sm_scale_log2;
             const float m_new = fmaxf(m_run, tmax); // finite from the first tile on: token 0 is visible to every row
             const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
             float psum = 0.f;
@@ -209,8 +207,8 @@ __global__ __launch_bounds__(256, 2) void prefill_kernel(PrefillArgs a, const ch
 #pragma unroll
                 for (int w = 0; w < 4; ++w) { // elements e = 2w, 2w+1 of the operand: block b0 + e/4, r = e%4
                     const int i0 = 4 * (b0 + (w >> 1)) + 2 * (w & 1);
-                    const float p0 = __builtin_amdgcn_exp2f(s[kb][i0] - m_new);
-                    const float p1 = __builtin_amdgcn_exp2f(s[kb][i0 + 1] - m_new);
+                    const float p0 = __builtin_amdgcn_exp2f(fmaf(s[kb][i0], a.sm_scale_log2, -m_new));
+                    const float p1 = __builtin_amdgcn_exp2f(fmaf(s[kb][i0 + 1], a.sm_scale_log2, -m_new));
                     psum += p0 + p1;
                     const uint32_t hw = M::pack2(p0, p1);
                     pf_u4(pa[st], w) = hw;

@@ -123,6 +123,10 @@ class BlitzBatchDecodeHandler:
         check(rc, "Handler plan")
         self._keep = (float_buffer, int_buffer)
 
+    def set_timing_events(self, start=None, stop=None):
+        """hipEvent_t handles recorded right before / after the decode kernel launch (None: off)."""
+        check(_lib.load().bz_decode_plan_set_timing_events(self._h, start, stop), "Handler timing events")
+
     def info(self):
         a, b, c = C.c_uint32(), C.c_uint32(), C.c_uint32()
         check(_lib.load().bz_decode_plan_info(self._h, C.byref(a), C.byref(b), C.byref(c)), "Handler info")

@@ -105,6 +105,12 @@ int bz_decode_plan(bz_decode_plan_t* plan, void* float_buffer, size_t float_buff
 int bz_decode_plan_info(const bz_decode_plan_t* plan, uint32_t* num_segments, uint32_t* num_split_seqs,
                         uint32_t* num_workgroups);
 
+/* Profiling aid (no counterpart in the reference): when both handles are non-NULL hipEvent_t values,
+ * the next bz_batch_decode calls on this plan record them on the launch stream immediately before
+ * and after the decode kernel itself (the split-K combine launch that may follow is outside the
+ * pair).  Pass NULL, NULL to switch it off. */
+int bz_decode_plan_set_timing_events(bz_decode_plan_t* plan, void* start_event, void* stop_event);
+
 /*
  * batch_decode_attention (src/kernel/attention.h:24-31, attention_decode.cu:13-40).
  * q, out: [batch, num_qo_heads, head_dim] of q_dtype (out_dtype may be BZ_F32 for tests).
