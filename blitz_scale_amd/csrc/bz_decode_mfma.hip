@@ -199,14 +199,20 @@ __global__ __launch_bounds__(64, 2) void decode_mfma_kernel(MfmaDecodeArgs a, co
     };
 
     uint4 kreg[2][4], vreg[8], qnext[4];
-    auto issue_loads = [&](const TileUni& u) {
-        size_t base[2];
+    // byte offsets of the two 16-token subtiles of a tile inside the pool
+    struct TileBase { size_t b[2]; };
+    auto tile_base = [&](const TileUni& u) -> TileBase {
+        TileBase r;
         const int pid[2] = {u.pid0, u.pid1};
 #pragma unroll
         for (int s = 0; s < 2; ++s) {
             const int slot0 = (u.t * kTileTok + 16 * s) % P; // a subtile past the last page reads the last page, masked later
-            base[s] = ((size_t)pid[s] * a.stride_page + (size_t)slot0 * a.stride_n + (size_t)u.kvh * a.stride_h) * ES;
+            r.b[s] = ((size_t)pid[s] * a.stride_page + (size_t)slot0 * a.stride_n + (size_t)u.kvh * a.stride_h) * ES;
         }
+        return r;
+    };
+    auto issue_loads = [&](const TileBase& tb) {
+        const size_t base[2] = {tb.b[0], tb.b[1]};
         if constexpr (KV8) {
 #pragma unroll
             for (int p = 0; p < 2; ++p) { // 16 bytes feed MFMA steps 2p and 2p+1
@@ -251,7 +257,7 @@ __global__ __launch_bounds__(64, 2) void decode_mfma_kernel(MfmaDecodeArgs a, co
     Desc dnext;
     TileUni un = read_info(0, 0); // description of the tile whose loads are issued next
     issue_q(un);
-    issue_loads(un);
+    issue_loads(tile_base(un));
 
 
     uint4 qhi[4], qlo[4];
@@ -261,6 +267,16 @@ __global__ __launch_bounds__(64, 2) void decode_mfma_kernel(MfmaDecodeArgs a, co
     for (int g = g_begin; g < g_end; ++g) {
         const TileUni uc = un; // the tile computed in this iteration (its loads are in flight or done)
         const int i = g - chunk_base;
+        // The description and the addresses of the next tile come first, while this tile's data is
+        // still on its way: the time between its arrival and the next loads is time in which this
+        // wave has nothing in flight.
+        TileBase nb;
+        if (g + 1 < g_end) {
+            const int nbuf = (i + 1 == 32) ? buf ^ 1 : buf;
+            un = read_info(nbuf, (i + 1) & 31);
+            nb = tile_base(un);
+        }
+        __builtin_amdgcn_sched_barrier(0);
         // descriptions of the next 32 tiles: fetched at i == 8, parked in the other LDS buffer at i == 24
         if (i == 8 && chunk_base + 32 < g_end) dnext = fetch_info(chunk_base + 32);
         if (i == 24 && chunk_base + 32 < g_end) { stash_info(dnext, buf ^ 1); wave_lds_sync(); }
@@ -341,11 +357,10 @@ __global__ __launch_bounds__(64, 2) void decode_mfma_kernel(MfmaDecodeArgs a, co
             }
         if (g + 1 < g_end) {
             if (i + 1 == 32) { chunk_base += 32; buf ^= 1; }
-            un = read_info(buf, (g + 1) - chunk_base);
 #if !(defined(BZ_EXP) && BZ_EXP == 4)
             if (un.flags & 1) issue_q(un); // next tile opens a new piece
 #endif
-            issue_loads(un);
+            issue_loads(nb);
         }
 #if defined(BZ_EXP) && (BZ_EXP == 1 || BZ_EXP == 2 || BZ_EXP == 4)
         { // experiment: loads only
