@@ -197,8 +197,13 @@ __global__ __launch_bounds__(256, 2) void prefill_kernel(PrefillArgs a, const ch
             // the scores stay unscaled in registers: the (positive) softmax scale is applied to the maximum
             // here and to every score inside the fused multiply-add that feeds exp2
             tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64)) * a.sm_scale_log2;
-            const float m_new = fmaxf(m_run, tmax); // finite from the first tile on: token 0 is visible to every row
-            const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
+            // The reference maximum only moves when some row's maximum has grown by more than 2^8 since
+            // it was last set (wave-uniform decision): until then exp2(s - m_run) is at most 256, which
+            // fp32 sums and 16-bit operands hold without loss, and the accumulators need no rescaling.
+            // Token 0 is visible to every row, so the first tile always sets a finite maximum.
+            const bool move_max = __any(tmax > m_run + 8.0f);
+            const float m_new = move_max ? fmaxf(m_run, tmax) : m_run;
+            const float alpha = move_max ? __builtin_amdgcn_exp2f(m_run - m_new) : 1.0f;
             float psum = 0.f;
             uint4 pa[4], pb[4]; // P^T operands of the four 16-token steps (head, and tail when SPLIT_P)
 #pragma unroll
@@ -218,7 +223,7 @@ __global__ __launch_bounds__(256, 2) void prefill_kernel(PrefillArgs a, const ch
             psum += __shfl_xor(psum, 32, 64);
             l_run = l_run * alpha + psum;
             m_run = m_new;
-            if (__any(alpha != 1.0f)) { // the running maximum settles after a few tiles
+            if (move_max) {
 #pragma unroll
                 for (int db = 0; db < 4; ++db)
 #pragma unroll
