@@ -31,6 +31,7 @@ HIPCC_FLAGS = [
     "-fPIC",
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     "-Wno-unused-result",
+    "-Wno-inline-asm",
 ]
 
 

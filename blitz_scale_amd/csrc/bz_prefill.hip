@@ -12,8 +12,11 @@
 // tile joins the two half-waves).
 #include <algorithm>
 #include <cmath>
+#include <cstdio>
+#include <cstdlib>
 #include <cstring>
 #include <new>
+#include <type_traits>
 #include <vector>
 
 #include "bz_common.hpp"
@@ -30,10 +33,18 @@ typedef __attribute__((ext_vector_type(4))) short pf_s16x4;
 
 constexpr int kBM = 128;       // q rows per workgroup
 constexpr int kBN = 64;        // kv tokens per tile
-constexpr int kKRow = 272;     // LDS row stride of the K tile (256 B + 16: 16 rows cover all banks)
-constexpr int kVRow = 320;     // LDS row stride of the V tile (256 B + 64: 4 rows x 64 B cover all banks)
-constexpr int kKTile = kBN * kKRow;
-constexpr int kVTile = kBN * kVRow;
+constexpr int kTile = kBN * 256; // bytes of one K or V tile in LDS (rows unpadded); LDS holds K0 K1 V0 V1
+constexpr int kORow = 272;       // LDS row stride of the output transpose in the epilogue (256 B + 16)
+
+// 16 bytes per lane from global memory straight into LDS: lane l's data lands at lds_addr + 16*l.
+// The compiler does not know that this is a load (it would otherwise wait for every such load before
+// any later LDS read, the ones of the tile in use included); the kernel waits for it explicitly.
+__device__ __forceinline__ void lds_direct_load16(const char* uniform_base, uint32_t lane_offset, uint32_t lds_addr) {
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
+                 :
+                 : "s"(lds_addr), "v"(lane_offset), "s"(uniform_base)
+                 : "memory", "m0");
+}
 
 struct PrefillItem { // one workgroup's job, in launch order
     int32_t tok0; // global index of the request's first token
@@ -79,7 +90,8 @@ template <> struct PfMma<true> {
                                                        c, 0, 0, 0);
     }
     __device__ static __forceinline__ uint32_t pack2(float lo, float hi) {
-        return (uint32_t)f32_to_bf16_bits(lo) | ((uint32_t)f32_to_bf16_bits(hi) << 16);
+        const pf_bf16x2 b = __builtin_convertvector(pf_f32x2{lo, hi}, pf_bf16x2); // v_cvt_pk_bf16_f32, round to nearest even
+        return __builtin_bit_cast(uint32_t, b);
     }
     __device__ static __forceinline__ float lo(uint32_t w) { return __uint_as_float(w << 16); }
     __device__ static __forceinline__ float hi(uint32_t w) { return __uint_as_float(w & 0xffff0000u); }
@@ -95,9 +107,10 @@ __global__ __launch_bounds__(256, 2) void prefill_kernel(PrefillArgs a, const ch
                                                          const char* __restrict__ v_ptr) {
     using M = PfMma<BF16>;
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
-    unsigned char* k_lds = smem;              // [2][kKTile]
-    unsigned char* v_lds = smem + 2 * kKTile; // [2][kVTile]
 
+#if defined(BZ_PF_EXP) && BZ_PF_EXP == 7
+    const long long wg_c0 = clock64(), wg_w0 = wall_clock64();
+#endif
     const PrefillItem it = a.items[blockIdx.x];
     if (it.len <= 0) return;
     const int head = it.head;
@@ -121,27 +134,50 @@ __global__ __launch_bounds__(256, 2) void prefill_kernel(PrefillArgs a, const ch
 
     const int kv_limit = a.causal ? min(L, it.q0 + kBM) : L; // tokens any row of this workgroup can see
     const int n_tiles = (kv_limit + kBN - 1) / kBN;
+    // tiles this wave computes: under the causal mask its rows see nothing past token wave_q_hi
+    const int n_w = a.causal ? min(n_tiles, wave_q_hi / kBN + 1) : n_tiles;
 
-    // ---- global -> register -> LDS staging of one K/V tile: thread i moves 16 B of rows i/16 + 16*r,
-    // r = 0..3.  Rows past the end of the request re-read its last row (valid memory; masked later).
-    uint4 kg0, kg1, kg2, kg3, vg0, vg1, vg2, vg3;
-    const int st_row = tid >> 4, st_col = (tid & 15) * 16;
-#define BZ_PF_LOAD_ROW(t_, r_, kreg_, vreg_)                                                              \
-    {                                                                                                     \
-        const size_t tok = (size_t)it.tok0 + (size_t)min((t_) * kBN + st_row + 16 * (r_), L - 1);          \
-        const size_t off = (tok * Hkv + kvh) * 256 + (size_t)st_col;                                       \
-        kreg_ = *reinterpret_cast<const uint4*>(k_ptr + off);                                              \
-        vreg_ = *reinterpret_cast<const uint4*>(v_ptr + off);                                              \
-    }
-#define BZ_PF_LOAD_TILE(t_)                                                                               \
-    BZ_PF_LOAD_ROW(t_, 0, kg0, vg0) BZ_PF_LOAD_ROW(t_, 1, kg1, vg1) BZ_PF_LOAD_ROW(t_, 2, kg2, vg2)        \
-    BZ_PF_LOAD_ROW(t_, 3, kg3, vg3)
-#define BZ_PF_STASH_ROW(buf_, r_, kreg_, vreg_)                                                           \
-    *reinterpret_cast<uint4*>(k_lds + (buf_) * kKTile + (st_row + 16 * (r_)) * kKRow + st_col) = kreg_;     \
-    *reinterpret_cast<uint4*>(v_lds + (buf_) * kVTile + (st_row + 16 * (r_)) * kVRow + st_col) = vreg_;
-#define BZ_PF_STASH_TILE(buf_)                                                                            \
-    BZ_PF_STASH_ROW(buf_, 0, kg0, vg0) BZ_PF_STASH_ROW(buf_, 1, kg1, vg1) BZ_PF_STASH_ROW(buf_, 2, kg2, vg2) \
-    BZ_PF_STASH_ROW(buf_, 3, kg3, vg3)
+    // ---- global -> LDS staging of a K/V tile with LDS-direct loads (no registers, no LDS stores): a
+    // wave instruction moves 64 x 16 B to 1 KiB of consecutive LDS, i.e. 4 unpadded 256-byte rows; wave w
+    // moves rows 16w .. 16w+15 of the tile with four instructions each for K and V.  What keeps the
+    // operand reads free of bank conflicts is an XOR on the 16-byte column chunk instead of padding:
+    //   K: chunk c of row r sits at position c ^ (r % 16)      (8 lanes read 8 rows, one chunk each)
+    //   V: chunk c of row r sits at position c ^ 2*(r % 4)     (a 16-lane group reads 4 rows x 32 B)
+    // and a lane of the copy simply fetches the chunk that belongs at its position.  Rows past the end
+    // of the request re-read its last row (valid memory; masked later).
+    const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) unsigned char*)smem;
+    const int wv = __builtin_amdgcn_readfirstlane(wave);
+    const int r4 = lane >> 4, p16 = lane & 15;
+    const uint32_t row_stride = (uint32_t)Hkv * 256u;
+    uint32_t kcol[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) kcol[i] = (uint32_t)((p16 ^ ((4 * i + r4) & 15)) * 16);
+    const uint32_t vcol = (uint32_t)((p16 ^ (r4 << 1)) * 16);
+    auto issue_tile = [&](int t, int buf) __attribute__((always_inline)) {
+        const size_t base = (((size_t)it.tok0 + (size_t)t * kBN) * Hkv + kvh) * 256; // wave-uniform
+        const uint32_t m0k = lds0 + (uint32_t)(buf * kTile + 16 * wv * 256);
+        if ((t + 1) * kBN <= L) { // the whole tile lies inside the request: only scalar arithmetic
+            const uint32_t lane_row = (uint32_t)r4 * row_stride;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const size_t rows = base + (size_t)(16 * wv + 4 * i) * row_stride;
+                lds_direct_load16(k_ptr + rows, lane_row + kcol[i], m0k + i * 1024);
+                lds_direct_load16(v_ptr + rows, lane_row + vcol, m0k + 2 * kTile + i * 1024);
+            }
+        } else {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int row = min(t * kBN + 16 * wv + 4 * i + r4, L - 1) - t * kBN;
+                lds_direct_load16(k_ptr + base, (uint32_t)row * row_stride + kcol[i], m0k + i * 1024);
+                lds_direct_load16(v_ptr + base, (uint32_t)row * row_stride + vcol, m0k + 2 * kTile + i * 1024);
+            }
+        }
+    };
+    // the copies of this wave have landed; after the barrier so have everyone's
+    auto publish = [&]() __attribute__((always_inline)) {
+        __builtin_amdgcn_s_waitcnt(0x0F70); // vmcnt(0)
+        __syncthreads();
+    };
 
     float m_run = -INFINITY, l_run = 0.f;
     pf_f32x16 acc[4]; // O^T: block db covers d = 32*db .. +31; element 4b+r is d = 32*db + 8b + 4h + r
@@ -150,31 +186,77 @@ __global__ __launch_bounds__(256, 2) void prefill_kernel(PrefillArgs a, const ch
 #pragma unroll
         for (int i = 0; i < 16; ++i) acc[db][i] = 0.f;
 
-    BZ_PF_LOAD_TILE(0)
-    BZ_PF_STASH_TILE(0)
-    __syncthreads();
+    issue_tile(0, 0);
+    publish();
 
-    for (int t = 0; t < n_tiles; ++t) {
-        const int buf = t & 1;
+    // operand read offsets inside a tile (lane constants).  K: row qn (+32 for the second block), chunk
+    // 2*ks + h.  V, through the transposing LDS read: a 16-lane group fetches 4 token rows x 16 d columns
+    // and every lane ends up with the 4 tokens of its own d column; the lane's row is 4h + srow (+16 per
+    // step, +8 for the second half) and its chunk 4*db + 2*(lane/16 % 2) + (lane % 4)/2.
+    uint32_t koff[8], voff[4];
+    {
+        const int y = h ^ (qn & 15);
+#pragma unroll
+        for (int ks = 0; ks < 8; ++ks) koff[ks] = (uint32_t)(qn * 256 + (((2 * ks) ^ y) * 16));
+        const int srow = (lane & 15) >> 2;
+        const int zl = ((((lane >> 4) & 1) << 1) | ((lane & 3) >> 1)) ^ (srow << 1);
+#pragma unroll
+        for (int db = 0; db < 4; ++db)
+            voff[db] = (uint32_t)((4 * h + srow) * 256 + ((((db << 2)) ^ zl) * 16) + (lane & 1) * 8);
+    }
+
+#if defined(BZ_PF_EXP) && BZ_PF_EXP == 7
+    long long ts_acc[6] = {0, 0, 0, 0, 0, 0}, ts_last = clock64();
+    const long long wg_c1 = ts_last;
+#define BZ_PF_TS(k_) { const long long now_ = clock64(); ts_acc[k_] += now_ - ts_last; ts_last = now_; }
+#else
+#define BZ_PF_TS(k_)
+#endif
+    // the arithmetic of tile t (K/V in LDS buffer BUF = t % 2, a compile-time constant so that the buffer
+    // and step offsets fold into the immediate field of the LDS reads)
+    auto compute_tile = [&](int t, auto which) __attribute__((always_inline)) {
+        constexpr int BUF = decltype(which)::value;
         const int kv0 = t * kBN;
-        if (t + 1 < n_tiles) { BZ_PF_LOAD_TILE(t + 1) }
-
-        const bool skip = a.causal && kv0 > wave_q_hi; // nothing in this tile is visible to the wave's rows
-        if (!skip) {
+        if (t < n_w) {
+            // Both contractions are scheduled by hand.  An LDS read takes several times as long as a
+            // matrix instruction, so the operand reads run kDK / kDV matrix instructions ahead of their
+            // use (rings ka / va); scheduling barriers keep the steps in this order.
+            constexpr int kDK = 4, kDV = 4;
+            uint4 ka[kDK], va[kDV];
+            auto k_read = [&](int i) __attribute__((always_inline)) { // operand of score step i: block i/8, d step i%8
+                return *reinterpret_cast<const uint4*>(smem + BUF * kTile + (i >> 3) * 32 * 256 + koff[i & 7]);
+            };
+            auto v_read = [&](int i) __attribute__((always_inline)) { // operand of step i: tokens 16*(i/4).., d block i%4
+                const unsigned char* vb = smem + (2 + BUF) * kTile + (i >> 2) * 16 * 256 + voff[i & 3];
+                const pf_s16x4 t0 =
+                    __builtin_amdgcn_ds_read_tr16_b64_v4i16((pf_s16x4 __attribute__((address_space(3)))*)(vb));
+                const pf_s16x4 t1 = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+                    (pf_s16x4 __attribute__((address_space(3)))*)(vb + 8 * 256));
+                const uint2 w0 = __builtin_bit_cast(uint2, t0), w1 = __builtin_bit_cast(uint2, t1);
+                return make_uint4(w0.x, w0.y, w1.x, w1.y);
+            };
             // ---- S^T = K Q^T: two 32-token blocks, eight 16-wide steps over d
             pf_f32x16 s[2];
 #pragma unroll
-            for (int kb = 0; kb < 2; ++kb) {
+            for (int i = 0; i < kDK; ++i) ka[i] = k_read(i);
+            __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-                for (int i = 0; i < 16; ++i) s[kb][i] = 0.f;
-                const unsigned char* krow = k_lds + buf * kKTile + (32 * kb + qn) * kKRow + h * 16;
+            for (int i = 0; i < 16; ++i) {
+                if ((i & 7) == 0) {
+                    pf_f32x16 zero;
 #pragma unroll
-                for (int ks = 0; ks < 8; ++ks) {
-                    const uint4 ka = *reinterpret_cast<const uint4*>(krow + ks * 32);
-                    s[kb] = M::run(ka, qreg[ks], s[kb]);
+                    for (int e = 0; e < 16; ++e) zero[e] = 0.f;
+                    s[i >> 3] = M::run(ka[i % kDK], qreg[i & 7], zero);
+                } else {
+                    s[i >> 3] = M::run(ka[i % kDK], qreg[i & 7], s[i >> 3]);
                 }
+                if (i + kDK < 16) ka[i % kDK] = k_read(i + kDK);
+                else va[i + kDK - 16] = v_read(i + kDK - 16); // the first V operands arrive during the softmax
+                __builtin_amdgcn_sched_barrier(0);
             }
-            // ---- scale, mask, online softmax.  Element 4b+r of block kb is token kv0 + 32kb + 8b + 4h + r.
+            static_assert(kDV == kDK, "the tail of the score steps fills the whole V ring");
+            BZ_PF_TS(1)
+            // ---- mask, maximum.  Element 4b+r of block kb is token kv0 + 32kb + 8b + 4h + r.
             const bool need_mask = (a.causal && kv0 + kBN - 1 > wave_q_lo) || (kv0 + kBN > L);
             float tmax = -INFINITY;
             if (need_mask) { // wave-uniform; selects, not branches, per element
@@ -201,9 +283,16 @@ __global__ __launch_bounds__(256, 2) void prefill_kernel(PrefillArgs a, const ch
             // it was last set (wave-uniform decision): until then exp2(s - m_run) is at most 256, which
             // fp32 sums and 16-bit operands hold without loss, and the accumulators need no rescaling.
             // Token 0 is visible to every row, so the first tile always sets a finite maximum.
-            const bool move_max = __any(tmax > m_run + 8.0f);
-            const float m_new = move_max ? fmaxf(m_run, tmax) : m_run;
-            const float alpha = move_max ? __builtin_amdgcn_exp2f(m_run - m_new) : 1.0f;
+            if (__any(tmax > m_run + 8.0f)) {
+                const float m_new = fmaxf(m_run, tmax);
+                const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
+                m_run = m_new;
+                l_run *= alpha;
+#pragma unroll
+                for (int db = 0; db < 4; ++db)
+#pragma unroll
+                    for (int i = 0; i < 16; ++i) acc[db][i] *= alpha;
+            }
             float psum = 0.f;
             uint4 pa[4], pb[4]; // P^T operands of the four 16-token steps (head, and tail when SPLIT_P)
 #pragma unroll
@@ -212,8 +301,8 @@ __global__ __launch_bounds__(256, 2) void prefill_kernel(PrefillArgs a, const ch
 #pragma unroll
                 for (int w = 0; w < 4; ++w) { // elements e = 2w, 2w+1 of the operand: block b0 + e/4, r = e%4
                     const int i0 = 4 * (b0 + (w >> 1)) + 2 * (w & 1);
-                    const float p0 = __builtin_amdgcn_exp2f(fmaf(s[kb][i0], a.sm_scale_log2, -m_new));
-                    const float p1 = __builtin_amdgcn_exp2f(fmaf(s[kb][i0 + 1], a.sm_scale_log2, -m_new));
+                    const float p0 = __builtin_amdgcn_exp2f(fmaf(s[kb][i0], a.sm_scale_log2, -m_run));
+                    const float p1 = __builtin_amdgcn_exp2f(fmaf(s[kb][i0 + 1], a.sm_scale_log2, -m_run));
                     psum += p0 + p1;
                     const uint32_t hw = M::pack2(p0, p1);
                     pf_u4(pa[st], w) = hw;
@@ -221,54 +310,59 @@ __global__ __launch_bounds__(256, 2) void prefill_kernel(PrefillArgs a, const ch
                 }
             }
             psum += __shfl_xor(psum, 32, 64);
-            l_run = l_run * alpha + psum;
-            m_run = m_new;
-            if (move_max) {
+            l_run += psum;
+            __builtin_amdgcn_sched_barrier(0);
+            BZ_PF_TS(2)
+            // ---- O^T += V^T P^T: step i takes tokens 16*(i/4) .. +15 and d block i%4
 #pragma unroll
-                for (int db = 0; db < 4; ++db)
-#pragma unroll
-                    for (int i = 0; i < 16; ++i) acc[db][i] *= alpha;
+            for (int i = 0; i < 16; ++i) {
+                acc[i & 3] = M::run(va[i % kDV], pa[i >> 2], acc[i & 3]);
+                if (SPLIT_P) acc[i & 3] = M::run(va[i % kDV], pb[i >> 2], acc[i & 3]);
+                if (i + kDV < 16) va[i % kDV] = v_read(i + kDV);
+                __builtin_amdgcn_sched_barrier(0);
             }
-
-            // ---- O^T += V^T P^T.  A operand through the transposing LDS read: a 16-lane group fetches
-            // 4 token rows x 16 d columns and every lane ends up with the 4 tokens of its own d column.
-            const int grp_d = ((lane >> 4) & 1) * 16; // d columns 0..15 or 16..31 of the block
-            const int srow = (lane & 15) >> 2, scol = (lane & 3) * 4;
-#pragma unroll
-            for (int st = 0; st < 4; ++st) {
-                const unsigned char* vbase = v_lds + buf * kVTile + (16 * st + 4 * h + srow) * kVRow + (grp_d + scol) * 2;
-#pragma unroll
-                for (int db = 0; db < 4; ++db) {
-                    uint4 va;
-                    const pf_s16x4 t0 = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-                        (pf_s16x4 __attribute__((address_space(3)))*)(vbase + db * 64));
-                    const pf_s16x4 t1 = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-                        (pf_s16x4 __attribute__((address_space(3)))*)(vbase + 8 * kVRow + db * 64));
-                    const uint2 w0 = __builtin_bit_cast(uint2, t0), w1 = __builtin_bit_cast(uint2, t1);
-                    va = make_uint4(w0.x, w0.y, w1.x, w1.y);
-                    acc[db] = M::run(va, pa[st], acc[db]);
-                    if (SPLIT_P) acc[db] = M::run(va, pb[st], acc[db]);
-                }
-            }
+            BZ_PF_TS(3)
         }
-        if (t + 1 < n_tiles) { BZ_PF_STASH_TILE(buf ^ 1) }
-        __syncthreads();
+    };
+    for (int t = 0; t < n_tiles; t += 2) {
+        if (t + 1 < n_tiles) issue_tile(t + 1, 1); // buffer 1 was last read before the previous barrier
+        BZ_PF_TS(0)
+        compute_tile(t, std::integral_constant<int, 0>{});
+        BZ_PF_TS(4)
+        publish();
+        BZ_PF_TS(5)
+        if (t + 1 < n_tiles) {
+            if (t + 2 < n_tiles) issue_tile(t + 2, 0);
+            BZ_PF_TS(0)
+            compute_tile(t + 1, std::integral_constant<int, 1>{});
+            BZ_PF_TS(4)
+            publish();
+            BZ_PF_TS(5)
+        }
     }
+#if defined(BZ_PF_EXP) && BZ_PF_EXP == 7
+    if (lane == 0) {
+        long long* dbg = reinterpret_cast<long long*>(reinterpret_cast<char*>(const_cast<PrefillItem*>(a.items)) + (1 << 20)) +
+                         ((size_t)blockIdx.x * 4 + wave) * 8;
+#pragma unroll
+        for (int k = 0; k < 6; ++k) dbg[k] = ts_acc[k];
+        dbg[6] = n_tiles;
+        dbg[7] = n_w;
+    }
+    const long long wg_c2 = clock64();
+#endif
+#undef BZ_PF_TS
 
-#undef BZ_PF_LOAD_ROW
-#undef BZ_PF_LOAD_TILE
-#undef BZ_PF_STASH_ROW
-#undef BZ_PF_STASH_TILE
     // ---- epilogue: normalise, transpose the wave's 32 x 128 block through LDS, store whole rows
     const float inv_l = l_run > 0.f ? 1.0f / l_run : 0.f;
-    unsigned char* o_lds = smem + wave * (32 * kKRow); // the K buffers are free now (barrier above)
+    unsigned char* o_lds = smem + wave * (32 * kORow); // the tiles are free now (barrier above)
 #pragma unroll
     for (int db = 0; db < 4; ++db)
 #pragma unroll
         for (int b = 0; b < 4; ++b) {
             const uint32_t w0 = M::pack2(acc[db][4 * b] * inv_l, acc[db][4 * b + 1] * inv_l);
             const uint32_t w1 = M::pack2(acc[db][4 * b + 2] * inv_l, acc[db][4 * b + 3] * inv_l);
-            *reinterpret_cast<uint2*>(o_lds + qn * kKRow + (32 * db + 8 * b + 4 * h) * 2) = make_uint2(w0, w1);
+            *reinterpret_cast<uint2*>(o_lds + qn * kORow + (32 * db + 8 * b + 4 * h) * 2) = make_uint2(w0, w1);
         }
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
     __builtin_amdgcn_wave_barrier();
@@ -278,11 +372,22 @@ __global__ __launch_bounds__(256, 2) void prefill_kernel(PrefillArgs a, const ch
         const int row = 4 * ps + (lane >> 4);
         const int pos = wave_q_lo + row;
         if (pos < L) {
-            const uint4 v = *reinterpret_cast<const uint4*>(o_lds + row * kKRow + (lane & 15) * 16);
+            const uint4 v = *reinterpret_cast<const uint4*>(o_lds + row * kORow + (lane & 15) * 16);
             char* orow = (char*)a.out + (((size_t)it.tok0 + pos) * Hq + head) * 256;
             *reinterpret_cast<uint4*>(orow + (lane & 15) * 16) = v;
         }
     }
+#if defined(BZ_PF_EXP) && BZ_PF_EXP == 7
+    if (lane == 0) {
+        long long* dbg2 = reinterpret_cast<long long*>(reinterpret_cast<char*>(const_cast<PrefillItem*>(a.items)) + (4 << 20)) +
+                          ((size_t)blockIdx.x * 4 + wave) * 8;
+        unsigned hwid, xcc;
+        asm volatile("s_getreg_b32 %0, hwreg(HW_REG_HW_ID)" : "=s"(hwid));
+        asm volatile("s_getreg_b32 %0, hwreg(HW_REG_XCC_ID)" : "=s"(xcc));
+        dbg2[0] = wg_w0; dbg2[1] = wall_clock64(); dbg2[2] = wg_c1 - wg_c0; dbg2[3] = wg_c2 - wg_c1; dbg2[4] = clock64() - wg_c2;
+        dbg2[5] = hwid; dbg2[6] = xcc & 0xf; dbg2[7] = n_tiles;
+    }
+#endif
 }
 
 // ---- in-place RoPE of ragged q and k rows (used when the caller asks the attention call itself to rotate)
@@ -438,12 +543,18 @@ extern "C" int bz_prefill_plan(bz_prefill_plan_t* plan_, void* float_buffer, siz
 template <bool BF16, bool SPLIT_P>
 static int launch_prefill(const PrefillPlan* p, const PrefillArgs& a, const void* q, const void* k, const void* v,
                           hipStream_t s) {
-    const size_t smem = 2 * (size_t)(kKTile + kVTile);
+    size_t smem = 4 * (size_t)kTile;
+    if (const char* e = getenv("BZ_PREFILL_SMEM_PAD")) smem += (size_t)atoi(e);
     auto kern = prefill_kernel<BF16, SPLIT_P>;
     static bool attr_done = false; // raising the dynamic LDS limit is idempotent; a repeated call is harmless
     if (!attr_done) {
         BZ_CHECK_HIP(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
         attr_done = true;
+        if (getenv("BZ_PREFILL_DEBUG")) {
+            int nb = -1;
+            (void)hipOccupancyMaxActiveBlocksPerMultiprocessor(&nb, (const void*)kern, 256, smem);
+            fprintf(stderr, "prefill: %d workgroups per CU, %zu B of LDS each, %u workgroups\n", nb, smem, p->num_items);
+        }
     }
     hipLaunchKernelGGL(kern, dim3(p->num_items), dim3(256), smem, s, a, (const char*)q, (const char*)k,
                        (const char*)v);
