@@ -149,22 +149,26 @@ __global__ __launch_bounds__(256, 2) void prefill_kernel(PrefillArgs a, const ch
     const int wv = __builtin_amdgcn_readfirstlane(wave);
     const int r4 = lane >> 4, p16 = lane & 15;
     const uint32_t row_stride = (uint32_t)Hkv * 256u;
-    uint32_t kcol[4];
+    uint32_t kcol[4], kfast[4], vfast[4];
 #pragma unroll
     for (int i = 0; i < 4; ++i) kcol[i] = (uint32_t)((p16 ^ ((4 * i + r4) & 15)) * 16);
     const uint32_t vcol = (uint32_t)((p16 ^ (r4 << 1)) * 16);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) { // lane offsets of copy i inside the wave's 16 rows when no row needs clamping
+        kfast[i] = (uint32_t)(4 * i + r4) * row_stride + kcol[i];
+        vfast[i] = (uint32_t)(4 * i + r4) * row_stride + vcol;
+    }
     auto issue_tile = [&](int t, int buf) __attribute__((always_inline)) {
-        const size_t base = (((size_t)it.tok0 + (size_t)t * kBN) * Hkv + kvh) * 256; // wave-uniform
         const uint32_t m0k = lds0 + (uint32_t)(buf * kTile + 16 * wv * 256);
-        if ((t + 1) * kBN <= L) { // the whole tile lies inside the request: only scalar arithmetic
-            const uint32_t lane_row = (uint32_t)r4 * row_stride;
+        if ((t + 1) * kBN <= L) { // the whole tile lies inside the request: one wave-uniform base for K, one for V
+            const size_t base = (((size_t)it.tok0 + (size_t)(t * kBN + 16 * wv)) * Hkv + kvh) * 256;
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
-                const size_t rows = base + (size_t)(16 * wv + 4 * i) * row_stride;
-                lds_direct_load16(k_ptr + rows, lane_row + kcol[i], m0k + i * 1024);
-                lds_direct_load16(v_ptr + rows, lane_row + vcol, m0k + 2 * kTile + i * 1024);
+                lds_direct_load16(k_ptr + base, kfast[i], m0k + i * 1024);
+                lds_direct_load16(v_ptr + base, vfast[i], m0k + 2 * kTile + i * 1024);
             }
         } else {
+            const size_t base = (((size_t)it.tok0 + (size_t)t * kBN) * Hkv + kvh) * 256;
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
                 const int row = min(t * kBN + 16 * wv + 4 * i + r4, L - 1) - t * kBN;
