@@ -146,11 +146,6 @@ __global__ __launch_bounds__(64, 2) void decode_mfma_kernel(MfmaDecodeArgs a, co
 
     const int g_begin = tile_ptr[blockIdx.x], g_end = tile_ptr[blockIdx.x + 1];
     if (g_begin >= g_end) return;
-#if defined(BZ_EXP) && BZ_EXP >= 3
-    long long* ts_buf = reinterpret_cast<long long*>(reinterpret_cast<char*>(a.part_o) + (64u << 20));
-    if (lane == 0) ts_buf[blockIdx.x * 4 + 0] = wall_clock64();
-    int exp_pieces = 0;
-#endif
 
     // ---- descriptions of 32 tiles at a time: lane l < 32 fetches the record of tile base+l, the two
     // page ids it points at and the piece it belongs to, and leaves 12 ints in LDS:
@@ -322,12 +317,6 @@ __global__ __launch_bounds__(64, 2) void decode_mfma_kernel(MfmaDecodeArgs a, co
         const int tile_tok0 = t * kTileTok;
         const bool ragged = tile_tok0 + kTileTok > tok_end; // wave-uniform
         wave_lds_sync(); // transposed reads of the previous tile come before V is overwritten
-#if defined(BZ_EXP) && BZ_EXP == 4
-        { uint32_t x = 0;
-#pragma unroll
-          for (int w = 0; w < 8; ++w) x ^= vreg[w].x ^ vreg[w].y ^ vreg[w].z ^ vreg[w].w;
-          acc[1][0] += __uint_as_float(x & 0x3fffffu); }
-#else
         if constexpr (KV8) {
 #pragma unroll
             for (int w = 0; w < 4; ++w) { // 16 e4m3 bytes -> 16 operand-type values -> 32 B of the LDS row
@@ -346,7 +335,6 @@ __global__ __launch_bounds__(64, 2) void decode_mfma_kernel(MfmaDecodeArgs a, co
                 *reinterpret_cast<uint4*>(v_lds + (4 * w + j) * kVRowBytes + n * 16) = v;
             }
         }
-#endif
         uint4 kcur[2][4];
 #pragma unroll
         for (int u = 0; u < 2; ++u)
@@ -357,22 +345,9 @@ __global__ __launch_bounds__(64, 2) void decode_mfma_kernel(MfmaDecodeArgs a, co
             }
         if (g + 1 < g_end) {
             if (i + 1 == 32) { chunk_base += 32; buf ^= 1; }
-#if !(defined(BZ_EXP) && BZ_EXP == 4)
             if (un.flags & 1) issue_q(un); // next tile opens a new piece
-#endif
             issue_loads(nb);
         }
-#if defined(BZ_EXP) && (BZ_EXP == 1 || BZ_EXP == 2 || BZ_EXP == 4)
-        { // experiment: loads only
-            uint32_t x = 0;
-#pragma unroll
-            for (int u = 0; u < 2; ++u)
-#pragma unroll
-                for (int ks = 0; ks < 4; ++ks) x ^= kcur[u][ks].x ^ kcur[u][ks].y ^ kcur[u][ks].z ^ kcur[u][ks].w;
-            acc[0][0] += __uint_as_float(x & 0x3fffffu);
-            l_run = 1.f; m_run = 0.f;
-        }
-#else
         // ---- scores: S^T[token][head], lane (head n, group j) gets tokens 16u + 4j + r
         f32x4_t s[2];
 #pragma unroll
@@ -446,17 +421,8 @@ __global__ __launch_bounds__(64, 2) void decode_mfma_kernel(MfmaDecodeArgs a, co
             acc[d] = M::run(pa, vb, acc[d]);
             acc[d] = M::run(pb, vb, acc[d]);
         }
-#endif
 
-#if defined(BZ_EXP) && BZ_EXP == 4
-        if ((uc.flags & 2) && g + 1 == g_end && acc[0][0] + acc[1][0] == 1.2345f) a.part_lse[0] = acc[0][0];
-        if (false) {
-#else
         if (uc.flags & 2) { // ================= last tile of a piece: final rows, or the split-K partial
-#endif
-#if defined(BZ_EXP) && BZ_EXP >= 3
-            ++exp_pieces;
-#endif
             const int b = uc.seq, kvh = uc.kvh, partial = uc.partial;
             const float inv_l = (l_run > 0.f ? 1.0f / l_run : 0.f) * ((KV8 && a.v_scale) ? a.v_scale[kvh] : 1.0f);
             const float lse2 = l_run > 0.f ? m_run + log2f(l_run) : -INFINITY;
@@ -485,16 +451,6 @@ __global__ __launch_bounds__(64, 2) void decode_mfma_kernel(MfmaDecodeArgs a, co
             }
         }
     }
-#if defined(BZ_EXP) && BZ_EXP >= 3
-    if (lane == 0) {
-        ts_buf[blockIdx.x * 4 + 1] = wall_clock64();
-        unsigned hwid, xcc;
-        asm volatile("s_getreg_b32 %0, hwreg(HW_REG_HW_ID)" : "=s"(hwid));
-        asm volatile("s_getreg_b32 %0, hwreg(HW_REG_XCC_ID)" : "=s"(xcc));
-        ts_buf[blockIdx.x * 4 + 2] = hwid;
-        ts_buf[blockIdx.x * 4 + 3] = (long long)(xcc & 0xf) | ((long long)exp_pieces << 8) | ((long long)(g_end - g_begin) << 20);
-    }
-#endif
 }
 
 // Combine the partials of one split (sequence, kv head): o = sum_i o_i 2^(lse_i - M) / sum_i 2^(lse_i - M).

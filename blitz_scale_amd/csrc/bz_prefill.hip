@@ -108,9 +108,6 @@ __global__ __launch_bounds__(256, 2) void prefill_kernel(PrefillArgs a, const ch
     using M = PfMma<BF16>;
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
 
-#if defined(BZ_PF_EXP) && BZ_PF_EXP == 7
-    const long long wg_c0 = clock64(), wg_w0 = wall_clock64();
-#endif
     const PrefillItem it = a.items[blockIdx.x];
     if (it.len <= 0) return;
     const int head = it.head;
@@ -209,13 +206,6 @@ __global__ __launch_bounds__(256, 2) void prefill_kernel(PrefillArgs a, const ch
             voff[db] = (uint32_t)((4 * h + srow) * 256 + ((((db << 2)) ^ zl) * 16) + (lane & 1) * 8);
     }
 
-#if defined(BZ_PF_EXP) && BZ_PF_EXP == 7
-    long long ts_acc[6] = {0, 0, 0, 0, 0, 0}, ts_last = clock64();
-    const long long wg_c1 = ts_last;
-#define BZ_PF_TS(k_) { const long long now_ = clock64(); ts_acc[k_] += now_ - ts_last; ts_last = now_; }
-#else
-#define BZ_PF_TS(k_)
-#endif
     // the arithmetic of tile t (K/V in LDS buffer BUF = t % 2, a compile-time constant so that the buffer
     // and step offsets fold into the immediate field of the LDS reads)
     auto compute_tile = [&](int t, auto which) __attribute__((always_inline)) {
@@ -259,7 +249,6 @@ __global__ __launch_bounds__(256, 2) void prefill_kernel(PrefillArgs a, const ch
                 __builtin_amdgcn_sched_barrier(0);
             }
             static_assert(kDV == kDK, "the tail of the score steps fills the whole V ring");
-            BZ_PF_TS(1)
             // ---- mask, maximum.  Element 4b+r of block kb is token kv0 + 32kb + 8b + 4h + r.
             const bool need_mask = (a.causal && kv0 + kBN - 1 > wave_q_lo) || (kv0 + kBN > L);
             float tmax = -INFINITY;
@@ -316,7 +305,6 @@ __global__ __launch_bounds__(256, 2) void prefill_kernel(PrefillArgs a, const ch
             psum += __shfl_xor(psum, 32, 64);
             l_run += psum;
             __builtin_amdgcn_sched_barrier(0);
-            BZ_PF_TS(2)
             // ---- O^T += V^T P^T: step i takes tokens 16*(i/4) .. +15 and d block i%4
 #pragma unroll
             for (int i = 0; i < 16; ++i) {
@@ -325,37 +313,18 @@ __global__ __launch_bounds__(256, 2) void prefill_kernel(PrefillArgs a, const ch
                 if (i + kDV < 16) va[i % kDV] = v_read(i + kDV);
                 __builtin_amdgcn_sched_barrier(0);
             }
-            BZ_PF_TS(3)
         }
     };
     for (int t = 0; t < n_tiles; t += 2) {
         if (t + 1 < n_tiles) issue_tile(t + 1, 1); // buffer 1 was last read before the previous barrier
-        BZ_PF_TS(0)
         compute_tile(t, std::integral_constant<int, 0>{});
-        BZ_PF_TS(4)
         publish();
-        BZ_PF_TS(5)
         if (t + 1 < n_tiles) {
             if (t + 2 < n_tiles) issue_tile(t + 2, 0);
-            BZ_PF_TS(0)
             compute_tile(t + 1, std::integral_constant<int, 1>{});
-            BZ_PF_TS(4)
             publish();
-            BZ_PF_TS(5)
         }
     }
-#if defined(BZ_PF_EXP) && BZ_PF_EXP == 7
-    if (lane == 0) {
-        long long* dbg = reinterpret_cast<long long*>(reinterpret_cast<char*>(const_cast<PrefillItem*>(a.items)) + (1 << 20)) +
-                         ((size_t)blockIdx.x * 4 + wave) * 8;
-#pragma unroll
-        for (int k = 0; k < 6; ++k) dbg[k] = ts_acc[k];
-        dbg[6] = n_tiles;
-        dbg[7] = n_w;
-    }
-    const long long wg_c2 = clock64();
-#endif
-#undef BZ_PF_TS
 
     // ---- epilogue: normalise, transpose the wave's 32 x 128 block through LDS, store whole rows
     const float inv_l = l_run > 0.f ? 1.0f / l_run : 0.f;
@@ -381,17 +350,6 @@ __global__ __launch_bounds__(256, 2) void prefill_kernel(PrefillArgs a, const ch
             *reinterpret_cast<uint4*>(orow + (lane & 15) * 16) = v;
         }
     }
-#if defined(BZ_PF_EXP) && BZ_PF_EXP == 7
-    if (lane == 0) {
-        long long* dbg2 = reinterpret_cast<long long*>(reinterpret_cast<char*>(const_cast<PrefillItem*>(a.items)) + (4 << 20)) +
-                          ((size_t)blockIdx.x * 4 + wave) * 8;
-        unsigned hwid, xcc;
-        asm volatile("s_getreg_b32 %0, hwreg(HW_REG_HW_ID)" : "=s"(hwid));
-        asm volatile("s_getreg_b32 %0, hwreg(HW_REG_XCC_ID)" : "=s"(xcc));
-        dbg2[0] = wg_w0; dbg2[1] = wall_clock64(); dbg2[2] = wg_c1 - wg_c0; dbg2[3] = wg_c2 - wg_c1; dbg2[4] = clock64() - wg_c2;
-        dbg2[5] = hwid; dbg2[6] = xcc & 0xf; dbg2[7] = n_tiles;
-    }
-#endif
 }
 
 // ---- in-place RoPE of ragged q and k rows (used when the caller asks the attention call itself to rotate)
@@ -547,18 +505,12 @@ extern "C" int bz_prefill_plan(bz_prefill_plan_t* plan_, void* float_buffer, siz
 template <bool BF16, bool SPLIT_P>
 static int launch_prefill(const PrefillPlan* p, const PrefillArgs& a, const void* q, const void* k, const void* v,
                           hipStream_t s) {
-    size_t smem = 4 * (size_t)kTile;
-    if (const char* e = getenv("BZ_PREFILL_SMEM_PAD")) smem += (size_t)atoi(e);
+    const size_t smem = 4 * (size_t)kTile;
     auto kern = prefill_kernel<BF16, SPLIT_P>;
     static bool attr_done = false; // raising the dynamic LDS limit is idempotent; a repeated call is harmless
     if (!attr_done) {
         BZ_CHECK_HIP(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
         attr_done = true;
-        if (getenv("BZ_PREFILL_DEBUG")) {
-            int nb = -1;
-            (void)hipOccupancyMaxActiveBlocksPerMultiprocessor(&nb, (const void*)kern, 256, smem);
-            fprintf(stderr, "prefill: %d workgroups per CU, %zu B of LDS each, %u workgroups\n", nb, smem, p->num_items);
-        }
     }
     hipLaunchKernelGGL(kern, dim3(p->num_items), dim3(256), smem, s, a, (const char*)q, (const char*)k,
                        (const char*)v);
