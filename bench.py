@@ -29,7 +29,7 @@ def parse():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=None)
     ap.add_argument("--warmup", type=int, default=None)
-    ap.add_argument("--workload", default="C3", choices=["C2", "C3", "C4", "C5"])
+    ap.add_argument("--workload", default="C3", choices=["C2", "C3", "C4", "C5", "ENDS"])
     ap.add_argument("--layers", type=int, default=None, help="layer planes of the KV pool the steps cycle over")
     ap.add_argument("--seed", type=lambda s: int(s, 0), default=0x5EED)
     ap.add_argument("--sigma", type=float, default=1.0, help="sigma of the log-normal context lengths (C3)")
@@ -363,6 +363,58 @@ def bench_prefill(args):
     return res_json
 
 
+def bench_ends(args):
+    """The row gathers and the greedy argmax either side of the layer loop (embedding, gather_last_token,
+    batch_find_max) at Llama-3-8B sizes: each is one pass over its rows, reported in us and GB/s."""
+    import numpy as np
+    import torch
+
+    import oracle
+    from blitz_scale_amd import kernel as K
+
+    vocab, hidden, ntok, batch = 128256, 4096, 8192, 128
+    rng = np.random.default_rng(args.seed)
+    g = torch.Generator(device="cuda")
+    g.manual_seed(args.seed)
+    w = torch.randn((vocab, hidden), dtype=torch.bfloat16, device="cuda", generator=g)
+    ids = torch.from_numpy(rng.integers(0, vocab, size=ntok).astype(np.int32)).cuda()
+    rows = torch.empty((ntok, hidden), dtype=torch.bfloat16, device="cuda")
+    indptr = torch.from_numpy((np.arange(batch + 1) * (ntok // batch)).astype(np.int32)).cuda()
+    last = torch.empty((batch, hidden), dtype=torch.bfloat16, device="cuda")
+    logits = torch.randn((batch, vocab), dtype=torch.bfloat16, device="cuda", generator=g)
+    arg = torch.empty(batch, dtype=torch.int32, device="cuda")
+    steps = args.steps or 200
+    warmup = args.warmup if args.warmup is not None else 20
+    ops = {
+        "embedding": (lambda: K.embedding(rows, ids, w, ntok, hidden), 2 * ntok * hidden * 2 + 4 * ntok),
+        "gather_last_token": (lambda: K.gather_last_token(last, rows, indptr, ntok, batch, hidden),
+                              2 * batch * hidden * 2 + 4 * (batch + 1)),
+        "batch_find_max": (lambda: K.batch_find_max(arg, logits, batch, vocab), batch * vocab * 2 + 4 * batch),
+    }
+    out = {}
+    total_ms = 0.0
+    for name, (fn, nbytes) in ops.items():
+        ms, ev = timed(lambda i, e: (e[0].record(), fn(), e[1].record()) if e is not None else fn(), steps, warmup)
+        out[name] = {"us": pct(ev)["mean"], "algorithmic_bytes": nbytes,
+                     "GB_per_s": round(nbytes / (float(ev.mean()) * 1e-3) / 1e9, 1)}
+        total_ms += ms
+    # parity on the spot (bit-exact)
+    torch.cuda.synchronize()
+    lg = logits.view(torch.int16).cpu().numpy().view(np.uint16)
+    from blitz_scale_amd._lib import BZ_BF16
+    ok = bool(np.array_equal(arg.cpu().numpy().view(np.uint32), oracle.batch_find_max(lg, BZ_BF16)))
+    dom = out["batch_find_max"]
+    return {"metric": "model_ends_us_per_step", "value": round(total_ms * 1e3, 3), "unit": "us/step", "n_gpus": 1,
+            "steps": steps, "warmup": warmup, "ms_per_step": round(total_ms, 6), "higher_is_better": False,
+            "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+            "config": {"workload": "ENDS: embedding of 8192 tokens, last-token gather and greedy argmax for 128 "
+                                   "sequences, Llama-3-8B sizes (hidden 4096, vocabulary 128256)"},
+            "ops": out, "argmax_bit_exact_vs_cpu": ok,
+            "roofline": {"bound": "hbm", "achieved": dom["GB_per_s"], "peak": 8000.0, "unit": "GB/s",
+                         "frac": round(dom["GB_per_s"] / 8000.0, 4), "traffic": None,
+                         "kernel": "bz::batch_find_max_kernel (the largest of the three)"}}
+
+
 def main():
     args = parse()
     import torch
@@ -376,7 +428,10 @@ def main():
             dst.copy_(src)
         torch.cuda.synchronize()
         del src, dst
-    res = bench_prefill(args) if args.workload == "C4" else bench_decode(args, args.workload)
+    if args.workload == "ENDS":
+        res = bench_ends(args)
+    else:
+        res = bench_prefill(args) if args.workload == "C4" else bench_decode(args, args.workload)
     print(json.dumps(res))
 
 

@@ -63,6 +63,9 @@ SIGNATURES = {
     "bz_add_rms_norm": (_i32, [_vp, _vp, _vp, _i32, _u32, _u32, _f32, _vp]),
     "bz_silu_and_mul": (_i32, [_vp, _vp, _i32, _u32, _u32, _vp]),
     "bz_add_residual": (_i32, [_vp, _vp, _i32, _u32, _u32, _vp]),
+    "bz_embedding": (_i32, [_vp, _vp, _vp, _vp, _i32, _u32, _u32, _vp]),
+    "bz_gather_last_token": (_i32, [_vp, _vp, _vp, _i32, _u32, _u32, _u32, _vp]),
+    "bz_batch_find_max": (_i32, [_vp, _vp, _i32, _u32, _u32, _vp]),
     "bz_cm_create": (_i32, [C.POINTER(_vp), _u32, _u32, _u32, _u32, _u32, _i32, _i32, _i32]),
     "bz_cm_destroy": (None, [_vp]),
     "bz_cm_batch_prefill": (_i32, [_vp, _vp, _u32, C.POINTER(_i32)]),

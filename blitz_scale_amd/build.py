@@ -20,6 +20,7 @@ SOURCES = [
     "bz_prefill.hip",
     "bz_page.hip",
     "bz_elementwise.hip",
+    "bz_sampler.hip",
     "bz_host.hip",
 ]
 

@@ -238,3 +238,24 @@ def add_residual(input, residual, num_tokens, dim, *, stream=None):
     """src/kernel/add.h:8-14."""
     rc = _lib.load().bz_add_residual(_ptr(input), _ptr(residual), bz_dtype(input), num_tokens, dim, _stream(stream))
     check(rc, "AddKernel")
+
+
+def embedding(output, token_ids, weight, num_tokens, hidden_size, *, out_loc=None, stream=None):
+    """src/kernel/embedding.h:7-36: output[loc] = weight[token_ids[t]]; loc = t or out_loc[t]."""
+    rc = _lib.load().bz_embedding(_ptr(output), _ptr(token_ids), _ptr(out_loc) if out_loc is not None else None,
+                                  _ptr(weight), bz_dtype(weight), num_tokens, hidden_size, _stream(stream))
+    check(rc, "EmbeddingKernel")
+
+
+def gather_last_token(output, tokens, ragged_indptr, num_tokens, batch_size, hidden_size, *, stream=None):
+    """src/kernel/sampler.h:8-16: output[b] = tokens[ragged_indptr[b+1] - 1]."""
+    rc = _lib.load().bz_gather_last_token(_ptr(output), _ptr(tokens), _ptr(ragged_indptr), bz_dtype(tokens),
+                                          num_tokens, batch_size, hidden_size, _stream(stream))
+    check(rc, "GatherLastTokenKernel")
+
+
+def batch_find_max(output_indices, input, batch_size, length, *, stream=None):
+    """src/kernel/sampler.h:18-26: output_indices[b] = argmax(input[b])."""
+    rc = _lib.load().bz_batch_find_max(_ptr(output_indices), _ptr(input), bz_dtype(input), batch_size, length,
+                                       _stream(stream))
+    check(rc, "BatchFindMaxKernel")

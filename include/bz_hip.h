@@ -185,6 +185,25 @@ int bz_add_residual(const void* input, void* residual, int dtype, uint32_t num_t
                     void* stream);
 
 /* ---------------------------------------------------------------------------------------
+ * row gathers and greedy sampling either side of the layer loop (src/model/llama.h)
+ * ------------------------------------------------------------------------------------- */
+/* embedding (src/kernel/embedding.h:7-36, embedding.cu:7-47): output[loc] = weight[token_ids[t]] for
+ * t < num_tokens, rows of hidden_size 16-bit elements (hidden_size % 8 == 0); loc = t, or out_loc[t]
+ * when out_loc is given (the tensor-parallel variant that scatters into a zeroed buffer). */
+int bz_embedding(void* output, const uint32_t* token_ids, const int32_t* out_loc, const void* weight, int dtype,
+                 uint32_t num_tokens, uint32_t hidden_size, void* stream);
+/* gather_last_token (src/kernel/sampler.h:8-16, sampler.cu:7-54): output[b] = tokens[ragged_indptr[b+1]-1],
+ * the whole row (the reference's kernel drops the lane offset on the destination, sampler.cu:21-24);
+ * a request without tokens yields a zero row. */
+int bz_gather_last_token(void* output, const void* tokens, const int32_t* ragged_indptr, int dtype,
+                         uint32_t num_tokens, uint32_t batch_size, uint32_t hidden_size, void* stream);
+/* batch_find_max (src/kernel/sampler.h:18-26, sampler.cu:80-135): output_indices[b] = argmax_i input[b][i]
+ * over rows of `length` 16-bit elements: the smallest index of the largest non-NaN value, 0 for a row
+ * that has none (the reference leaves ties to a race and the index undefined below -65400). */
+int bz_batch_find_max(uint32_t* output_indices, const void* input, int dtype, uint32_t batch_size, uint32_t length,
+                      void* stream);
+
+/* ---------------------------------------------------------------------------------------
  * Host page-table logic: pool owner, first-fit page allocator and per-batch page tables in pinned
  * memory.  Replaces the integer semantics of src/blitz/cache_manager.h:123-324 and of the page-table
  * parts of src/blitz/batch.h (prefill constructor :206-276, update :280-295, filter :297-418,

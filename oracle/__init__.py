@@ -226,6 +226,33 @@ def add_residual(in_bits, res_bits, dtype):
     return res
 
 
+def embedding(token_ids, weight_bits, out_rows=None, out_loc=None):
+    """out[loc] = weight[token_ids[t]]; returns the output (rows not written stay zero)."""
+    ids = _c(token_ids, np.uint32)
+    w = _c(weight_bits, np.uint16)
+    hidden = w.shape[1]
+    out = np.zeros((len(ids) if out_rows is None else out_rows, hidden), np.uint16)
+    loc = _c(out_loc, np.int32) if out_loc is not None else None
+    lib().bzo_embedding(_p(out), _p(ids), _p(loc) if loc is not None else None, _p(w), C.c_size_t(len(ids)),
+                        C.c_size_t(hidden))
+    return out
+
+
+def gather_last_token(tokens_bits, ragged_indptr):
+    t = _c(tokens_bits, np.uint16)
+    ip = _c(ragged_indptr, np.int32)
+    out = np.empty((len(ip) - 1, t.shape[1]), np.uint16)
+    lib().bzo_gather_last_token(_p(out), _p(t), _p(ip), C.c_size_t(len(ip) - 1), C.c_size_t(t.shape[1]))
+    return out
+
+
+def batch_find_max(input_bits, dtype):
+    x = _c(input_bits, np.uint16)
+    out = np.empty(x.shape[0], np.uint32)
+    lib().bzo_batch_find_max(_p(out), _p(x), dtype, C.c_size_t(x.shape[0]), C.c_size_t(x.shape[1]))
+    return out
+
+
 def prefill_reservation(lens, page_size):
     lens = _c(lens, np.int32)
     B = len(lens)

@@ -15,6 +15,8 @@
  *   rms_norm / add_rms_norm .......... src/kernel/rms_norm.h:11-34, norm.cu:7-39
  *   silu_and_mul ..................... src/kernel/activation.h:7-16, activation.cu:9
  *   add_residual ..................... src/kernel/add.h:8-14, add.cu:13-38
+ *   embedding ........................ src/kernel/embedding.h:7-36, embedding.cu:7-47
+ *   gather_last_token / batch_find_max src/kernel/sampler.h:8-26, sampler.cu:7-25,80-109
  *   host page table build / grow ..... src/blitz/batch.h:236-257,
  *                                      src/blitz/cache_manager.h:161-184,197-324
  *
@@ -487,6 +489,42 @@ void bzo_add_residual(const void* input, void* residual, int dtype, size_t n) {
     for (size_t i = 0; i < n; ++i) {
         double s = (double)load_as_f32(input, dtype, i) + (double)load_as_f32(residual, dtype, i);
         ((uint16_t*)residual)[i] = round_f64_to_16(s, dtype);
+    }
+}
+
+/* embedding (embedding.cu:7-47): out row (out_loc ? out_loc[t] : t) <- weight row token_ids[t] */
+void bzo_embedding(uint16_t* out, const uint32_t* token_ids, const int32_t* out_loc, const uint16_t* weight,
+                   size_t num_tokens, size_t hidden) {
+    for (size_t t = 0; t < num_tokens; ++t) {
+        const size_t d = out_loc ? (size_t)out_loc[t] : t;
+        for (size_t i = 0; i < hidden; ++i) out[d * hidden + i] = weight[(size_t)token_ids[t] * hidden + i];
+    }
+}
+
+/* gather_last_token (sampler.h:8-16): out row b <- tokens row ragged_indptr[b+1]-1, the whole row
+ * (what the header documents; the reference's kernel drops the lane offset on the destination,
+ * sampler.cu:21-24).  A request without tokens yields a zero row. */
+void bzo_gather_last_token(uint16_t* out, const uint16_t* tokens, const int32_t* ragged_indptr, size_t batch,
+                           size_t hidden) {
+    for (size_t b = 0; b < batch; ++b)
+        for (size_t i = 0; i < hidden; ++i)
+            out[b * hidden + i] =
+                ragged_indptr[b + 1] > ragged_indptr[b] ? tokens[(size_t)(ragged_indptr[b + 1] - 1) * hidden + i] : 0;
+}
+
+/* batch_find_max (sampler.h:18-26): argmax of each row: the smallest index of the largest non-NaN
+ * value, 0 if the row has none (sampler.cu:87-108 leaves ties to a race and starts from -65400). */
+void bzo_batch_find_max(uint32_t* out, const void* input, int dtype, size_t batch, size_t length) {
+    for (size_t b = 0; b < batch; ++b) {
+        float best = 0.f;
+        int have = 0;
+        uint32_t bi = 0;
+        for (size_t i = 0; i < length; ++i) {
+            const float v = load_as_f32(input, dtype, b * length + i);
+            if (v != v) continue;
+            if (!have || v > best) { best = v; bi = (uint32_t)i; have = 1; }
+        }
+        out[b] = bi;
     }
 }
 

@@ -15,7 +15,9 @@
 #include "kernel/activation.h"
 #include "kernel/add.h"
 #include "kernel/attention.h"
+#include "kernel/embedding.h"
 #include "kernel/rms_norm.h"
+#include "kernel/sampler.h"
 #include "layer/attn.h"
 #include "layer/glu.h"
 
@@ -34,6 +36,9 @@ void bzo_rms_norm(const void*, const void*, int, int, int, float, float*);
 void bzo_add_rms_norm(const void*, void*, const void*, int, int, int, float, float*);
 void bzo_silu_and_mul(const void*, int, int, int, float*);
 void bzo_add_residual(const void*, void*, int, size_t);
+void bzo_embedding(uint16_t*, const uint32_t*, const int32_t*, const uint16_t*, size_t, size_t);
+void bzo_gather_last_token(uint16_t*, const uint16_t*, const int32_t*, size_t, size_t);
+void bzo_batch_find_max(uint32_t*, const void*, int, size_t, size_t);
 void bzo_rope_ragged_inplace(void*, int, const int32_t*, int, int, int, float);
 void bzo_rope_decode_q_inplace(void*, int, const bzo_paged_kv*, int, float);
 void bzo_store_prefill_kv(const bzo_paged_kv*, const void*, const void*, int, const int32_t*, int, float, const float*,
@@ -247,6 +252,43 @@ int main() {
     for (size_t i = 0; i < plane; ++i) touched0 += pool_gpu[i] != pool_cpu[i];
     printf("kv plane of layer 1: max diff %.3e; layer 0 plane differs in %zu elements\n", e3, touched0);
 
+    // ---- the two ends of Llama::forward (src/model/llama.h): embedding rows in, last-token rows and
+    // greedy token ids out, through the reference's template names
+    bool ends_ok = true;
+    {
+        const uint32_t vocab = 1000, ntok = (uint32_t)N, nb = (uint32_t)B;
+        std::vector<int32_t> indptr_tok(batch.ragged_indptr.begin(), batch.ragged_indptr.end()); // the prompts' rows
+        bits_t emb = rand_bits((size_t)vocab * hidden, 1.0f);
+        std::vector<uint32_t> ids(ntok);
+        for (uint32_t t = 0; t < ntok; ++t) ids[t] = (t * 7919u + 13u) % vocab;
+        half_t *emb_d, *rows_d, *last_d;
+        uint32_t *ids_d, *arg_d;
+        int32_t* ip_d;
+        HIP_OK(hipMalloc(&emb_d, emb.size() * 2));
+        HIP_OK(hipMalloc(&rows_d, (size_t)ntok * hidden * 2));
+        HIP_OK(hipMalloc(&last_d, (size_t)nb * hidden * 2));
+        HIP_OK(hipMalloc(&ids_d, ntok * 4));
+        HIP_OK(hipMalloc(&arg_d, nb * 4));
+        HIP_OK(hipMalloc(&ip_d, (nb + 1) * 4));
+        HIP_OK(hipMemcpy(emb_d, emb.data(), emb.size() * 2, hipMemcpyHostToDevice));
+        HIP_OK(hipMemcpy(ids_d, ids.data(), ntok * 4, hipMemcpyHostToDevice));
+        HIP_OK(hipMemcpy(ip_d, indptr_tok.data(), (nb + 1) * 4, hipMemcpyHostToDevice));
+        blitz::kernel::embedding(rows_d, ids_d, emb_d, ntok, (uint32_t)hidden);
+        blitz::kernel::gather_last_token(last_d, rows_d, ip_d, ntok, nb, (uint32_t)hidden);
+        blitz::kernel::batch_find_max(arg_d, last_d, nb, (uint32_t)hidden);
+        HIP_OK(hipDeviceSynchronize());
+        bits_t rows_g((size_t)ntok * hidden), last_g((size_t)nb * hidden), rows_c(rows_g.size()), last_c(last_g.size());
+        std::vector<uint32_t> arg_g(nb), arg_c(nb);
+        HIP_OK(hipMemcpy(rows_g.data(), rows_d, rows_g.size() * 2, hipMemcpyDeviceToHost));
+        HIP_OK(hipMemcpy(last_g.data(), last_d, last_g.size() * 2, hipMemcpyDeviceToHost));
+        HIP_OK(hipMemcpy(arg_g.data(), arg_d, nb * 4, hipMemcpyDeviceToHost));
+        bzo_embedding(rows_c.data(), ids.data(), nullptr, emb.data(), ntok, hidden);
+        bzo_gather_last_token(last_c.data(), rows_c.data(), indptr_tok.data(), nb, hidden);
+        bzo_batch_find_max(arg_c.data(), last_c.data(), 0, nb, hidden);
+        ends_ok = rows_g == rows_c && last_g == last_c && arg_g == arg_c;
+        printf("embedding / gather_last_token / batch_find_max: %s\n", ends_ok ? "bit-exact" : "MISMATCH");
+    }
+
     // error convention: std::runtime_error with the reference's message prefix
     bool threw = false;
     try {
@@ -256,7 +298,7 @@ int main() {
         threw = strncmp(e.what(), "batchDecodeAttention error: ", 28) == 0;
     }
     // the activations are O(1); a chain of f16 roundings through four GEMMs stays within a few 1e-3
-    const bool ok = e1 < 2e-2 && e2 < 2e-2 && e3 < 5e-3 && touched0 == 0 && threw;
+    const bool ok = e1 < 2e-2 && e2 < 2e-2 && e3 < 5e-3 && touched0 == 0 && threw && ends_ok;
     printf(ok ? "PASS\n" : "FAIL\n");
     return ok ? 0 : 1;
 }
