@@ -1,0 +1,190 @@
+// One Llama-2-7B-shaped decoder layer (hidden 4096, 32 heads, intermediate 11008) stepping a decode
+// batch of 64 sequences through the C++ drop-in headers with every GEMM on hipBLASLt: what SURVEY's C2
+// workload calls "a single-layer decode step", with the four GEMMs in.  Checks
+//   1. blitz::util::HipblasLtGemm against a naive fp32-accumulate GEMM on a few shapes,
+//   2. the layer's residual stream against the same layer run with the naive GEMM,
+// and prints the time of a layer step.  Runs on the GPU box; built without a GPU.
+#include <algorithm>
+#include <cmath>
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <vector>
+
+#include <hip/hip_runtime.h>
+
+#include "blitz/cache_manager.h"
+#include "kernel/attention.h"
+#include "layer/attn.h"
+#include "layer/glu.h"
+#include "util/hipblaslt_gemm.h"
+
+#define HIP_OK(x)                                                                         \
+    do {                                                                                  \
+        hipError_t e_ = (x);                                                              \
+        if (e_ != hipSuccess) {                                                           \
+            printf("HIP error %s at %s:%d\n", hipGetErrorString(e_), __FILE__, __LINE__); \
+            exit(2);                                                                      \
+        }                                                                                 \
+    } while (0)
+
+using half_t = __half;
+
+// naive row-major GEMM, fp32 accumulate in index order, one rounding to f16: test infrastructure only
+__global__ void naive_gemm(int m, int n, int k, const __half* A, const __half* B, __half* C) {
+    const int col = blockIdx.x * blockDim.x + threadIdx.x, row = blockIdx.y;
+    if (col >= n) return;
+    float acc = 0.f;
+    for (int i = 0; i < k; ++i) acc += __half2float(A[(size_t)row * k + i]) * __half2float(B[(size_t)i * n + col]);
+    C[(size_t)row * n + col] = __float2half_rn(acc);
+}
+struct NaiveGemm : blitz::util::GemmWrapper {
+    void gemm(int m, int n, int k, const void* A, const void* B, void* C) override {
+        hipLaunchKernelGGL(naive_gemm, dim3((n + 127) / 128, m), dim3(128), 0, 0, m, n, k, (const __half*)A,
+                           (const __half*)B, (__half*)C);
+    }
+};
+// device fill: uniform(-scale, scale) + mean from a counter hash (no host buffers of gigabytes)
+__global__ void fill_uniform(__half* p, size_t n, float scale, float mean, uint64_t seed) {
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x) {
+        uint64_t z = seed + (i + 1) * 0x9E3779B97F4A7C15ull;
+        z = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ull;
+        z = (z ^ (z >> 27)) * 0x94D049BB133111EBull;
+        z ^= z >> 31;
+        p[i] = __float2half_rn(mean + scale * (float)((double)(z >> 11) / 9007199254740992.0 * 2.0 - 1.0));
+    }
+}
+static void fill(__half* p, size_t n, float scale, float mean, uint64_t seed) {
+    hipLaunchKernelGGL(fill_uniform, dim3(2048), dim3(256), 0, 0, p, n, scale, mean, seed);
+}
+static double max_abs_diff_dev(const __half* a, const __half* b, size_t n, double* max_ref) {
+    std::vector<__half> ha(n), hb(n);
+    HIP_OK(hipMemcpy(ha.data(), a, n * 2, hipMemcpyDeviceToHost));
+    HIP_OK(hipMemcpy(hb.data(), b, n * 2, hipMemcpyDeviceToHost));
+    double m = 0, r = 0;
+    for (size_t i = 0; i < n; ++i) {
+        const double x = __half2float(ha[i]), y = __half2float(hb[i]);
+        if (!(x == x) || !(y == y)) return INFINITY;
+        m = fmax(m, fabs(x - y));
+        r = fmax(r, fabs(y));
+    }
+    if (max_ref) *max_ref = r;
+    return m;
+}
+
+int main() {
+    bool ok = true;
+    blitz::util::HipblasLtGemm lt(HIP_R_16F);
+    NaiveGemm naive;
+
+    // ---- 1. the GEMM wrapper against the naive product (inputs O(1)/sqrt(k): results O(1))
+    const int shapes[][3] = {{64, 512, 256}, {7, 1024, 384}, {1, 4096, 4096}, {64, 12288, 4096}, {57, 264, 128}};
+    for (auto& s : shapes) {
+        const int m = s[0], n = s[1], k = s[2];
+        __half *A, *B, *C0, *C1;
+        HIP_OK(hipMalloc(&A, (size_t)m * k * 2));
+        HIP_OK(hipMalloc(&B, (size_t)k * n * 2));
+        HIP_OK(hipMalloc(&C0, (size_t)m * n * 2));
+        HIP_OK(hipMalloc(&C1, (size_t)m * n * 2));
+        fill(A, (size_t)m * k, 1.0f, 0.f, 11);
+        fill(B, (size_t)k * n, 1.7f / sqrtf((float)k), 0.f, 12);
+        naive.gemm(m, n, k, A, B, C0);
+        lt.gemm(m, n, k, A, B, C1);
+        HIP_OK(hipDeviceSynchronize());
+        double ref = 0;
+        const double e = max_abs_diff_dev(C1, C0, (size_t)m * n, &ref);
+        // both accumulate in fp32 and round once; the summation order differs: a few f16 steps at |c| ~ 2
+        const bool good = e <= 4e-3 * fmax(1.0, ref);
+        printf("gemm %5d x %5d x %5d: max |hipblaslt - naive| = %.3e (max |c| %.2f) %s\n", m, n, k, e, ref, good ? "ok" : "BAD");
+        ok = ok && good;
+        (void)hipFree(A); (void)hipFree(B); (void)hipFree(C0); (void)hipFree(C1);
+    }
+
+    // ---- 2. a Llama-2-7B-shaped layer, decode batch of 64, contexts U[512, 2048]
+    const uint32_t hidden = 4096, Hq = 32, Hkv = 32, D = 128, inter = 11008, P = 16, B = 64;
+    blitz::kernel::attention_options().rope_theta = 1e4f;
+    std::vector<int32_t> lens(B);
+    uint64_t st = 0x5EED;
+    uint32_t need = 0;
+    for (auto& l : lens) {
+        st = st * 6364136223846793005ull + 1442695040888963407ull;
+        l = 512 + (int32_t)((st >> 33) % 1537);
+        need += (l + 2 + P - 1) / P;
+    }
+    const uint32_t max_pages = need + 16;
+    blitz::CacheManager<half_t, int32_t> cm(Hkv, 1, D, P, max_pages, BZ_LAYOUT_HND, true, 1 << 20);
+    fill((half_t*)cm.get_base_ptr(), (size_t)max_pages * 2 * Hkv * P * D, 1.0f, 0.f, 21); // a context of N(0,~0.58) keys/values
+    blitz::HostBatch<half_t, int32_t> batch(&cm, lens); // reserves len+1 slots: a batch right after its prefill
+    auto& pt = batch.page_table;
+    cm.set_layer(pt, 0);
+    int32_t* table_d;
+    HIP_OK(hipMalloc(&table_d, 4 << 20));
+    const size_t tn = pt.indices.size() + pt.indptr.size() + pt.last_page_len.size();
+    HIP_OK(hipMemcpy(table_d, pt.indices_h, tn * 4, hipMemcpyHostToDevice));
+    pt.indices_d = table_d;
+    pt.indptr_d = table_d + pt.indices.size();
+    pt.last_page_len_d = pt.indptr_d + pt.indptr.size();
+
+    const size_t attn_w = hidden + 2 * (size_t)Hq * D * hidden + 2 * (size_t)Hkv * D * hidden;
+    const size_t glu_w = hidden + 3 * (size_t)hidden * inter;
+    half_t* w_d;
+    HIP_OK(hipMalloc(&w_d, (attn_w + glu_w) * 2));
+    fill(w_d, attn_w + glu_w, 1.7f / sqrtf((float)hidden), 0.f, 31);
+    fill(w_d, hidden, 0.02f, 1.0f, 32);          // input norm
+    fill(w_d + attn_w, hidden, 0.02f, 1.0f, 33); // post-attention norm
+    void *float_ws, *int_ws;
+    HIP_OK(hipMalloc(&float_ws, 128 << 20));
+    HIP_OK(hipMalloc(&int_ws, 8 << 20));
+    blitz::kernel::BatchPrefillRaggedHandler<half_t, int32_t> prefill_h(blitz::kernel::create_flashinfer_prefill_handler());
+    blitz::kernel::BlitzBatchDecodeHandler<half_t, int32_t> decode_h(blitz::kernel::create_flashinfer_decode_handler());
+    const size_t ws_elems = (size_t)B * (hidden + 3 * (size_t)std::max<uint32_t>(hidden, inter) + (size_t)(2 * Hq + 2 * Hkv) * D);
+    half_t *ws_lt, *ws_nv, *x_d;
+    HIP_OK(hipMalloc(&ws_lt, ws_elems * 2));
+    HIP_OK(hipMalloc(&ws_nv, ws_elems * 2));
+    HIP_OK(hipMalloc(&x_d, (size_t)B * hidden * 2));
+    fill(x_d, (size_t)B * hidden, 1.7f, 0.f, 41);
+    decode_h.plan(float_ws, 128 << 20, int_ws, 8 << 20, pt.indptr_h, pt.last_page_len_h, B, Hq, Hkv, D, P);
+
+    auto run_layer = [&](blitz::util::GemmWrapper* g, half_t* ws) {
+        half_t* seg = w_d;
+        blitz::layer::Attention<half_t, int32_t> attn(g, &prefill_h, &decode_h, D, hidden, Hq, Hkv, ws, &seg);
+        blitz::layer::GatedLinearUnit<half_t> glu(g, hidden, inter, ws, &seg);
+        HIP_OK(hipMemcpy(ws, x_d, (size_t)B * hidden * 2, hipMemcpyDeviceToDevice));
+        attn.forward(B, nullptr, pt);
+        glu.forward(B);
+        HIP_OK(hipDeviceSynchronize());
+    };
+    // both runs append the same new K/V at the same slot, so the second one sees the pool the first one left
+    run_layer(&naive, ws_nv);
+    run_layer(&lt, ws_lt);
+    double ref = 0;
+    const double e = max_abs_diff_dev(ws_lt, ws_nv, (size_t)B * hidden, &ref);
+    const bool good = e <= 2e-2 * fmax(1.0, ref);
+    printf("layer decode step, residual stream: max |hipblaslt - naive gemm| = %.3e (max |x| %.2f) %s\n", e, ref, good ? "ok" : "BAD");
+    ok = ok && good;
+
+    // ---- time of a layer step (events on the null stream, which everything here uses)
+    {
+        half_t* seg = w_d;
+        blitz::layer::Attention<half_t, int32_t> attn(&lt, &prefill_h, &decode_h, D, hidden, Hq, Hkv, ws_lt, &seg);
+        blitz::layer::GatedLinearUnit<half_t> glu(&lt, hidden, inter, ws_lt, &seg);
+        hipEvent_t e0, e1;
+        HIP_OK(hipEventCreate(&e0));
+        HIP_OK(hipEventCreate(&e1));
+        const int warm = 10, steps = 100;
+        for (int i = 0; i < warm + steps; ++i) {
+            if (i == warm) HIP_OK(hipEventRecord(e0, 0));
+            attn.forward(B, nullptr, pt);
+            glu.forward(B);
+        }
+        HIP_OK(hipEventRecord(e1, 0));
+        HIP_OK(hipEventSynchronize(e1));
+        float ms = 0;
+        HIP_OK(hipEventElapsedTime(&ms, e0, e1));
+        const double weights = (double)(attn_w + glu_w) * 2;
+        printf("layer decode step (B 64, ctx U[512,2048], 7B shapes, all GEMMs on hipBLASLt): %.1f us; weights %.1f MB -> %.0f GB/s "
+               "if the step were only the weight stream\n", ms * 1e3 / steps, weights / 1e6, weights / (ms * 1e-3 / steps) / 1e9);
+    }
+    printf(ok ? "PASS\n" : "FAIL\n");
+    return ok ? 0 : 1;
+}

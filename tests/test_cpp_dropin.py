@@ -8,6 +8,7 @@ import pytest
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 BIN = os.path.join(ROOT, "tests", "cpp", "test_dropin")
+LAYER_BIN = os.path.join(ROOT, "tests", "cpp", "layer_step")
 
 
 def build_cpp_test():
@@ -23,11 +24,20 @@ def build_cpp_test():
     err = "\n".join(l for l in out.stderr.splitlines() if "packed-fp32-ops" not in l)
     if out.returncode != 0:
         raise RuntimeError("hipcc failed:\n" + err)
+    # the layer step with every GEMM on hipBLASLt (blitz_scale_amd/cpp/util/hipblaslt_gemm.h)
+    cmd2 = cmd[:cmd.index(os.path.join(ROOT, "tests", "cpp", "test_dropin.cpp"))] + [
+        os.path.join(ROOT, "tests", "cpp", "layer_step.cpp"), "-o", LAYER_BIN,
+        "-L", os.path.join(ROOT, "blitz_scale_amd", "lib"), "-lbz_hip", "-L", "/opt/rocm/lib", "-lhipblaslt",
+        "-Wl,-rpath,$ORIGIN/../../blitz_scale_amd/lib"]
+    out = subprocess.run(cmd2, capture_output=True, text=True)
+    err = "\n".join(l for l in out.stderr.splitlines() if "packed-fp32-ops" not in l)
+    if out.returncode != 0:
+        raise RuntimeError("hipcc failed:\n" + err)
     return BIN
 
 
 def test_headers_compile_and_link_without_a_gpu():
-    assert os.path.exists(build_cpp_test())
+    assert os.path.exists(build_cpp_test()) and os.path.exists(LAYER_BIN)
 
 
 @pytest.mark.gpu
@@ -35,5 +45,14 @@ def test_layer_prefill_and_decode_through_the_cpp_headers():
     if not os.path.exists(BIN):
         build_cpp_test()
     out = subprocess.run([BIN], capture_output=True, text=True, timeout=120)
+    print(out.stdout, out.stderr)
+    assert out.returncode == 0 and "PASS" in out.stdout
+
+
+@pytest.mark.gpu
+def test_layer_decode_step_with_hipblaslt_gemms():
+    if not os.path.exists(LAYER_BIN):
+        build_cpp_test()
+    out = subprocess.run([LAYER_BIN], capture_output=True, text=True, timeout=300)
     print(out.stdout, out.stderr)
     assert out.returncode == 0 and "PASS" in out.stdout
