@@ -1,6 +1,6 @@
 // One Llama-2-7B-shaped decoder layer (hidden 4096, 32 heads, intermediate 11008) stepping a decode
-// batch of 64 sequences through the C++ drop-in headers with every GEMM on hipBLASLt: what SURVEY's C2
-// workload calls "a single-layer decode step", with the four GEMMs in.  Checks
+// batch of 64 sequences through the C++ drop-in headers with every GEMM on hipBLASLt: the "single-layer decode step" of
+// a Llama-2-7B decode benchmark with the four GEMMs in.  Checks
 //   1. blitz::util::HipblasLtGemm against a naive fp32-accumulate GEMM on a few shapes,
 //   2. the layer's residual stream against the same layer run with the naive GEMM,
 // and prints the time of a layer step.  Runs on the GPU box; built without a GPU.
