@@ -66,6 +66,9 @@ SIGNATURES = {
     "bz_embedding": (_i32, [_vp, _vp, _vp, _vp, _i32, _u32, _u32, _vp]),
     "bz_gather_last_token": (_i32, [_vp, _vp, _vp, _i32, _u32, _u32, _u32, _vp]),
     "bz_batch_find_max": (_i32, [_vp, _vp, _i32, _u32, _u32, _vp]),
+    "bz_kv_wire_bytes": (_u64, [_u32, _u32, _kvp, _i32]),
+    "bz_kv_pages_pack": (_i32, [_vp, _u64, _kvp, _vp, _u32, _u32, _u32, _vp, _i32, _vp, _vp, _vp]),
+    "bz_kv_pages_unpack": (_i32, [_vp, _u64, _kvp, _vp, _u32, _u32, _u32, _vp, _i32, _vp, _vp, _vp]),
     "bz_cm_create": (_i32, [C.POINTER(_vp), _u32, _u32, _u32, _u32, _u32, _i32, _i32, _i32]),
     "bz_cm_destroy": (None, [_vp]),
     "bz_cm_batch_prefill": (_i32, [_vp, _vp, _u32, C.POINTER(_i32)]),

@@ -21,6 +21,7 @@ SOURCES = [
     "bz_page.hip",
     "bz_elementwise.hip",
     "bz_sampler.hip",
+    "bz_wire.hip",
     "bz_host.hip",
 ]
 

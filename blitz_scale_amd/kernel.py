@@ -259,3 +259,33 @@ def batch_find_max(output_indices, input, batch_size, length, *, stream=None):
     rc = _lib.load().bz_batch_find_max(_ptr(output_indices), _ptr(input), bz_dtype(input), batch_size, length,
                                        _stream(stream))
     check(rc, "BatchFindMaxKernel")
+
+
+def kv_wire_bytes(page_table, num_pages, layer_cnt, wire_dtype=None):
+    """Bytes of the migration buffer for num_pages pages of layer_cnt layers."""
+    s = page_table.as_struct()
+    wd = page_table.kv_dtype if wire_dtype is None else wire_dtype
+    return int(_lib.load().bz_kv_wire_bytes(num_pages, layer_cnt, C.byref(s), wd))
+
+
+def pack_kv_pages(page_table, max_num_pages, page_ids, start_layer, layer_cnt, wire, *, wire_dtype=None,
+                  k_scale=None, v_scale=None, stream=None):
+    """The messages of MigrationManager::send_multi_layer_fast (src/blitz/migration_manager.h:455-467),
+    page by page and layer by layer, concatenated into `wire`.  page_table.base is layer 0 of the pool."""
+    s = page_table.as_struct()
+    wd = page_table.kv_dtype if wire_dtype is None else wire_dtype
+    rc = _lib.load().bz_kv_pages_pack(_ptr(page_table.base), max_num_pages, C.byref(s), _ptr(page_ids),
+                                      page_ids.numel(), start_layer, layer_cnt, _ptr(wire), wd, _ptr(k_scale),
+                                      _ptr(v_scale), _stream(stream))
+    check(rc, "PackKVPages")
+
+
+def unpack_kv_pages(page_table, max_num_pages, page_ids, start_layer, layer_cnt, wire, *, wire_dtype=None,
+                    k_scale=None, v_scale=None, stream=None):
+    """The receiving side: chunk i*layer_cnt + l of `wire` goes to page page_ids[i] of layer start_layer + l."""
+    s = page_table.as_struct()
+    wd = page_table.kv_dtype if wire_dtype is None else wire_dtype
+    rc = _lib.load().bz_kv_pages_unpack(_ptr(page_table.base), max_num_pages, C.byref(s), _ptr(page_ids),
+                                        page_ids.numel(), start_layer, layer_cnt, _ptr(wire), wd, _ptr(k_scale),
+                                        _ptr(v_scale), _stream(stream))
+    check(rc, "UnpackKVPages")

@@ -204,6 +204,30 @@ int bz_batch_find_max(uint32_t* output_indices, const void* input, int dtype, ui
                       void* stream);
 
 /* ---------------------------------------------------------------------------------------
+ * KV page wire format for migration between instances.  The reference sends one message of
+ * stride_page elements per (page, layer) straight from the pool, request by request, prompt block by
+ * prompt block, layer by layer (src/blitz/migration_manager.h:86-92 get_page_ptr, :455-467 send loop;
+ * the receive loops mirror it).  bz_kv_pages_pack writes that byte stream into ONE contiguous device
+ * buffer, so that one large transfer replaces the per-(page, layer) sends: chunk c = i*layer_cnt + l of
+ * `wire` is page page_ids[i] of layer start_layer + l (stride_page elements, the page's in-pool
+ * order).  bz_kv_pages_unpack scatters such a buffer to the receiver's own page ids.
+ *   pool_base : layer 0 of a pool laid out [layer][page][...] with max_pages pages per layer
+ *   kv        : geometry only (num_kv_heads, stride_page, stride_h, kv_dtype); its pointers are not read
+ *   page_ids  : device array [num_pages], in the order the pages are to appear on the wire
+ *   wire_dtype: the pool's type (bit copy), or BZ_E4M3 for a 16-bit pool: elements travel as
+ *               e4m3(x / scale) and arrive as e4m3 * scale, scale = k_scale / v_scale[l*num_kv_heads +
+ *               head] (device arrays [layer_cnt][num_kv_heads]; NULL = 1), half the bytes.
+ * Pages listed twice in an unpack race.  Launch only; no allocation, copy or synchronisation.
+ * ------------------------------------------------------------------------------------- */
+uint64_t bz_kv_wire_bytes(uint32_t num_pages, uint32_t layer_cnt, const bz_paged_kv_t* kv, int wire_dtype);
+int bz_kv_pages_pack(const void* pool_base, uint64_t max_pages, const bz_paged_kv_t* kv, const int32_t* page_ids,
+                     uint32_t num_pages, uint32_t start_layer, uint32_t layer_cnt, void* wire, int wire_dtype,
+                     const float* k_scale, const float* v_scale, void* stream);
+int bz_kv_pages_unpack(void* pool_base, uint64_t max_pages, const bz_paged_kv_t* kv, const int32_t* page_ids,
+                       uint32_t num_pages, uint32_t start_layer, uint32_t layer_cnt, const void* wire,
+                       int wire_dtype, const float* k_scale, const float* v_scale, void* stream);
+
+/* ---------------------------------------------------------------------------------------
  * Host page-table logic: pool owner, first-fit page allocator and per-batch page tables in pinned
  * memory.  Replaces the integer semantics of src/blitz/cache_manager.h:123-324 and of the page-table
  * parts of src/blitz/batch.h (prefill constructor :206-276, update :280-295, filter :297-418,

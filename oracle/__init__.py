@@ -253,6 +253,64 @@ def batch_find_max(input_bits, dtype):
     return out
 
 
+def _wire_scales(kv_dtype, wire_dtype, stride_page, stride_h, Hkv, layer_cnt, k_scale, v_scale):
+    """Per-element scale of one (page, layer) chunk for every layer: [layer_cnt][stride_page] fp32, or None."""
+    if wire_dtype == kv_dtype or (k_scale is None and v_scale is None):
+        return None
+    half = stride_page // 2
+    head = (np.arange(half) // stride_h) % Hkv
+    ks = np.ones((layer_cnt, Hkv), np.float32) if k_scale is None else _c(k_scale, np.float32).reshape(layer_cnt, Hkv)
+    vs = np.ones((layer_cnt, Hkv), np.float32) if v_scale is None else _c(v_scale, np.float32).reshape(layer_cnt, Hkv)
+    return np.concatenate([ks[:, head], vs[:, head]], axis=1)
+
+
+def kv_pages_pack(pool_bits, kv_dtype, max_pages, stride_page, page_ids, start_layer, layer_cnt, wire_dtype=None,
+                  num_kv_heads=1, stride_h=1, k_scale=None, v_scale=None):
+    """The byte stream MigrationManager::send_multi_layer_fast sends (src/blitz/migration_manager.h:455-467):
+    for every page in order, for every layer, the stride_page elements at get_page_ptr (:86-92) =
+    base + layer*max_pages*stride_page + page*stride_page.  With an e4m3 wire on a 16-bit pool every
+    element travels as e4m3(x / scale[layer][head])."""
+    pool = _c(pool_bits, storage_np(kv_dtype)).reshape(-1)
+    wire_dtype = kv_dtype if wire_dtype is None else wire_dtype
+    sc = _wire_scales(kv_dtype, wire_dtype, stride_page, stride_h, num_kv_heads, layer_cnt, k_scale, v_scale)
+    out = []
+    for page in np.asarray(page_ids, np.int64):
+        for l in range(layer_cnt):
+            off = ((start_layer + l) * max_pages + int(page)) * stride_page
+            chunk = pool[off:off + stride_page]
+            if wire_dtype != kv_dtype:
+                x = to_f32(chunk, kv_dtype)
+                if sc is not None:
+                    x = (x / sc[l]).astype(np.float32)
+                chunk = from_f32(x, wire_dtype)
+            out.append(chunk)
+    if not out:
+        return np.empty(0, storage_np(wire_dtype))
+    return np.concatenate(out)
+
+
+def kv_pages_unpack(pool_bits, kv_dtype, max_pages, stride_page, page_ids, start_layer, layer_cnt, wire_bits,
+                    wire_dtype=None, num_kv_heads=1, stride_h=1, k_scale=None, v_scale=None):
+    """The receiving side, in place on pool_bits: message (i, l) goes to page page_ids[i] of layer start_layer + l."""
+    pool = pool_bits.reshape(-1)
+    wire_dtype = kv_dtype if wire_dtype is None else wire_dtype
+    wire = _c(wire_bits, storage_np(wire_dtype)).reshape(-1)
+    sc = _wire_scales(kv_dtype, wire_dtype, stride_page, stride_h, num_kv_heads, layer_cnt, k_scale, v_scale)
+    c = 0
+    for page in np.asarray(page_ids, np.int64):
+        for l in range(layer_cnt):
+            chunk = wire[c * stride_page:(c + 1) * stride_page]
+            if wire_dtype != kv_dtype:
+                x = to_f32(chunk, wire_dtype)
+                if sc is not None:
+                    x = (x * sc[l]).astype(np.float32)
+                chunk = from_f32(x, kv_dtype)
+            off = ((start_layer + l) * max_pages + int(page)) * stride_page
+            pool[off:off + stride_page] = chunk
+            c += 1
+    return pool_bits
+
+
 def prefill_reservation(lens, page_size):
     lens = _c(lens, np.int32)
     B = len(lens)
