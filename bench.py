@@ -9,7 +9,8 @@ by the previous step.  plan() runs once per model step in the reference (src/mod
 outside the layer loop, and is timed separately.
 
 --workload C2 | C4 | C5 run the other configurations (C2 adds the RMSNorm and SiLU-gate kernels of the
-layer, C4 is the ragged causal prefill + page store, C5 the e4m3-KV decode).  One GPU only.
+layer, C4 is the ragged causal prefill + page store, C5 the e4m3-KV decode); ENDS and MIGRATE time the
+row gathers / argmax either side of the layer loop and the KV migration pack / unpack.  One GPU only.
 """
 import argparse
 import json
@@ -29,7 +30,7 @@ def parse():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=None)
     ap.add_argument("--warmup", type=int, default=None)
-    ap.add_argument("--workload", default="C3", choices=["C2", "C3", "C4", "C5", "ENDS"])
+    ap.add_argument("--workload", default="C3", choices=["C2", "C3", "C4", "C5", "ENDS", "MIGRATE"])
     ap.add_argument("--layers", type=int, default=None, help="layer planes of the KV pool the steps cycle over")
     ap.add_argument("--seed", type=lambda s: int(s, 0), default=0x5EED)
     ap.add_argument("--sigma", type=float, default=1.0, help="sigma of the log-normal context lengths (C3)")
@@ -415,6 +416,65 @@ def bench_ends(args):
                          "kernel": "bz::batch_find_max_kernel (the largest of the three)"}}
 
 
+def bench_migrate(args):
+    """KV migration payload of a prefilled batch: pack every (page, layer) of 16 prompts of 2048 tokens,
+    Llama-3-8B geometry (32 layers, 8 kv heads, D 128, P 16, bf16: 128 KiB per token), into one buffer
+    and scatter it into other pages of a second pool.  Bytes: payload read + payload written, per pass."""
+    import numpy as np
+    import torch
+
+    from blitz_scale_amd import kernel as K
+    from blitz_scale_amd._lib import BZ_E4M3
+
+    layers, Hkv, P, D, nreq, ntok = 32, 8, 16, 128, 16, 2048
+    sp = 2 * Hkv * P * D
+    n = nreq * ntok // P
+    max_pages = 2 * n
+    rng = np.random.default_rng(args.seed)
+    g = torch.Generator(device="cuda")
+    g.manual_seed(args.seed)
+    src = torch.randn(layers * max_pages * sp, dtype=torch.bfloat16, device="cuda", generator=g)
+    dst = torch.zeros_like(src)
+    spt, dpt = K.PageTable(nreq, P, Hkv, D, src), K.PageTable(nreq, P, Hkv, D, dst)
+    src_ids = torch.from_numpy(rng.permutation(max_pages)[:n].astype(np.int32)).cuda()
+    dst_ids = torch.from_numpy(rng.permutation(max_pages)[:n].astype(np.int32)).cuda()
+    payload = K.kv_wire_bytes(spt, n, layers)
+    wire = torch.empty(payload, dtype=torch.uint8, device="cuda")
+    ks = torch.full((layers, Hkv), 5.0 / 448, dtype=torch.float32, device="cuda")
+    steps = args.steps or 20
+    warmup = args.warmup if args.warmup is not None else 3
+    ops = {
+        "pack": (lambda: K.pack_kv_pages(spt, max_pages, src_ids, 0, layers, wire), 2 * payload),
+        "unpack": (lambda: K.unpack_kv_pages(dpt, max_pages, dst_ids, 0, layers, wire), 2 * payload),
+        "pack_e4m3_wire": (lambda: K.pack_kv_pages(spt, max_pages, src_ids, 0, layers, wire, wire_dtype=BZ_E4M3,
+                                                   k_scale=ks, v_scale=ks), payload + payload // 2),
+    }
+    out = {}
+    for name, (fn, nbytes) in ops.items():
+        ms, ev = timed(lambda i, e: (e[0].record(), fn(), e[1].record()) if e is not None else fn(), steps, warmup)
+        out[name] = {"us": pct(ev)["mean"], "algorithmic_bytes": nbytes,
+                     "GB_per_s": round(nbytes / (float(ev.mean()) * 1e-3) / 1e9, 1)}
+    # parity on the spot: the receiver's pages hold the sender's bits
+    ops["pack"][0]()
+    ops["unpack"][0]()
+    torch.cuda.synchronize()
+    s3 = src.view(torch.int16).view(layers, max_pages, sp)
+    d3 = dst.view(torch.int16).view(layers, max_pages, sp)
+    ok = bool(torch.equal(s3[:, src_ids.long()], d3[:, dst_ids.long()]))
+    ms = (out["pack"]["us"] + out["unpack"]["us"]) * 1e-3
+    dom = out["pack"]
+    return {"metric": "kv_migration_pack_unpack_ms", "value": round(ms, 4), "unit": "ms/step", "n_gpus": 1,
+            "steps": steps, "warmup": warmup, "ms_per_step": round(ms, 6), "higher_is_better": False,
+            "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+            "config": {"workload": "MIGRATE: wire payload of 16 prompts x 2048 tokens, Llama-3-8B KV geometry "
+                                   f"(32 layers, {n} pages, {payload / 2**30:.1f} GiB): pack on the sender + unpack "
+                                   "on the receiver"},
+            "ops": out, "round_trip_bit_exact": ok,
+            "roofline": {"bound": "hbm", "achieved": dom["GB_per_s"], "peak": 8000.0, "unit": "GB/s",
+                         "frac": round(dom["GB_per_s"] / 8000.0, 4), "traffic": None,
+                         "kernel": "bz::wire_kernel (pack), payload read + payload written"}}
+
+
 def main():
     args = parse()
     import torch
@@ -430,6 +490,8 @@ def main():
         del src, dst
     if args.workload == "ENDS":
         res = bench_ends(args)
+    elif args.workload == "MIGRATE":
+        res = bench_migrate(args)
     else:
         res = bench_prefill(args) if args.workload == "C4" else bench_decode(args, args.workload)
     print(json.dumps(res))

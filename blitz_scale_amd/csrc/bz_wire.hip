@@ -15,6 +15,31 @@
 
 namespace bz {
 
+typedef __attribute__((ext_vector_type(4))) uint32_t wire_u32x4;
+typedef __attribute__((ext_vector_type(2))) uint32_t wire_u32x2;
+// Streaming (non-temporal) accesses: every byte is touched once, so nothing is worth keeping in the
+// caches (measured: pack 4.9 -> 5.5 TB/s).
+template <typename T> __device__ __forceinline__ void wire_load(Vec8<T>& v, const void* p) {
+    if constexpr (sizeof(v.raw) == 16) {
+        const wire_u32x4 r = __builtin_nontemporal_load(reinterpret_cast<const wire_u32x4*>(p));
+        v.raw = make_uint4(r.x, r.y, r.z, r.w);
+    } else {
+        const wire_u32x2 r = __builtin_nontemporal_load(reinterpret_cast<const wire_u32x2*>(p));
+        v.raw = make_uint2(r.x, r.y);
+    }
+}
+template <typename T> __device__ __forceinline__ void wire_store(const Vec8<T>& v, void* p) {
+    if constexpr (sizeof(v.raw) == 16) {
+        const wire_u32x4 r = {v.raw.x, v.raw.y, v.raw.z, v.raw.w};
+        __builtin_nontemporal_store(r, reinterpret_cast<wire_u32x4*>(p));
+    } else {
+        const wire_u32x2 r = {v.raw.x, v.raw.y};
+        __builtin_nontemporal_store(r, reinterpret_cast<wire_u32x2*>(p));
+    }
+}
+
+constexpr int kWirePer = 4; // vectors per lane
+
 struct WireArgs {
     char* pool;            // base of the whole pool (layer 0)
     char* wire;
@@ -33,7 +58,7 @@ struct WireArgs {
 // PT: pool element type, WT: wire element type, PACK: pool -> wire (else wire -> pool)
 template <typename PT, typename WT, bool PACK>
 __global__ __launch_bounds__(256) void wire_kernel(WireArgs a) {
-    constexpr int kPer = 4;
+    constexpr int kPer = kWirePer;
     const uint64_t g0 = (uint64_t)blockIdx.x * (256 * kPer) + threadIdx.x;
     using ST = typename std::conditional<PACK, PT, WT>::type; // what is read
     using DT = typename std::conditional<PACK, WT, PT>::type; // what is written
@@ -59,7 +84,7 @@ __global__ __launch_bounds__(256) void wire_kernel(WireArgs a) {
         }
         const ST* src = PACK ? reinterpret_cast<const ST*>(a.pool) + pool_off[u]
                              : reinterpret_cast<const ST*>(a.wire) + g * 8;
-        in[u].load(src);
+        wire_load(in[u], src);
     }
 #pragma unroll
     for (int u = 0; u < kPer; ++u) {
@@ -69,7 +94,7 @@ __global__ __launch_bounds__(256) void wire_kernel(WireArgs a) {
         if constexpr (sizeof(PT) == sizeof(WT)) {
             Vec8<DT> o;
             o.raw = in[u].raw; // bit copy
-            o.store(dst);
+            wire_store(o, dst);
         } else {
             float x[8];
             in[u].to_float(x);
@@ -80,14 +105,14 @@ __global__ __launch_bounds__(256) void wire_kernel(WireArgs a) {
             }
             Vec8<DT> o;
             o.from_float(x);
-            o.store(dst);
+            wire_store(o, dst);
         }
     }
 }
 
 template <typename PT, typename WT, bool PACK>
 static int launch_wire(const WireArgs& a, hipStream_t s) {
-    const uint64_t per_wg = 256 * 4;
+    const uint64_t per_wg = 256 * kWirePer;
     const uint64_t grid = (a.total_vecs + per_wg - 1) / per_wg;
     if (grid == 0) return 0;
     if (grid > 0x7fffffffull) return BZ_ERR_UNSUPPORTED;

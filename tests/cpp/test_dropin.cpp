@@ -12,6 +12,7 @@
 #include <hip/hip_runtime.h>
 
 #include "blitz/cache_manager.h"
+#include "blitz/kv_wire.h"
 #include "kernel/activation.h"
 #include "kernel/add.h"
 #include "kernel/attention.h"
@@ -289,6 +290,46 @@ int main() {
         printf("embedding / gather_last_token / batch_find_max: %s\n", ends_ok ? "bit-exact" : "MISMATCH");
     }
 
+    // ---- migration payload (src/blitz/migration_manager.h:455-467): the batch's pages, all layers, through
+    // one buffer into another pool at other page ids; every (page, layer) unit arrives bit for bit
+    bool wire_ok = true;
+    {
+        blitz::CacheManager<half_t, int32_t> cm2(Hkv, layers, D, P, max_pages, BZ_LAYOUT_HND, true, 64 << 10);
+        blitz::HostBatch<half_t, int32_t> pad(&cm2, std::vector<int32_t>{40}); // so that the receiver's ids differ
+        std::vector<int32_t> lens2;
+        for (int b = 0; b < B; ++b) lens2.push_back(batch.ragged_indptr[b + 1] - batch.ragged_indptr[b]);
+        blitz::HostBatch<half_t, int32_t> batch2(&cm2, lens2);
+        const std::vector<int32_t>& src_ids = pt.indices;
+        const std::vector<int32_t> dst_ids(batch2.page_table.indices.begin(),
+                                           batch2.page_table.indices.begin() + src_ids.size());
+        const uint32_t n = (uint32_t)src_ids.size();
+        blitz::KvWire<half_t, int32_t> tx(cm.get_base_ptr(), max_pages), rx(cm2.get_base_ptr(), max_pages);
+        const size_t nbytes = tx.wire_bytes(pt, n, layers);
+        void* wire_d;
+        int32_t *src_d, *dst_d;
+        HIP_OK(hipMalloc(&wire_d, nbytes));
+        HIP_OK(hipMalloc(&src_d, n * 4));
+        HIP_OK(hipMalloc(&dst_d, n * 4));
+        HIP_OK(hipMemcpy(src_d, src_ids.data(), n * 4, hipMemcpyHostToDevice));
+        HIP_OK(hipMemcpy(dst_d, dst_ids.data(), n * 4, hipMemcpyHostToDevice));
+        tx.pack(pt, src_d, n, 0, layers, wire_d);
+        rx.unpack(batch2.page_table, dst_d, n, 0, layers, wire_d);
+        HIP_OK(hipDeviceSynchronize());
+        bits_t pool2(pool_gpu.size()), wire_h(nbytes / 2);
+        HIP_OK(hipMemcpy(pool2.data(), cm2.get_base_ptr(), pool2.size() * 2, hipMemcpyDeviceToHost));
+        HIP_OK(hipMemcpy(wire_h.data(), wire_d, nbytes, hipMemcpyDeviceToHost));
+        wire_ok = nbytes == (size_t)n * layers * pt.stride_page * 2 && src_ids != dst_ids;
+        for (uint32_t i = 0; i < n; ++i)
+            for (uint32_t l = 0; l < layers; ++l) {
+                const uint16_t* a = pool_gpu.data() + (tx.get_page_ptr(pt, src_ids[i], l) - cm.get_base_ptr());
+                const uint16_t* b = pool2.data() + (rx.get_page_ptr(batch2.page_table, dst_ids[i], l) - cm2.get_base_ptr());
+                const uint16_t* w = wire_h.data() + ((size_t)i * layers + l) * pt.stride_page;
+                wire_ok = wire_ok && memcmp(a, b, pt.stride_page * 2) == 0 && memcmp(a, w, pt.stride_page * 2) == 0;
+            }
+        printf("migration payload of %u pages x %u layers (%zu bytes): %s\n", n, layers, nbytes,
+               wire_ok ? "bit-exact" : "MISMATCH");
+    }
+
     // error convention: std::runtime_error with the reference's message prefix
     bool threw = false;
     try {
@@ -298,7 +339,7 @@ int main() {
         threw = strncmp(e.what(), "batchDecodeAttention error: ", 28) == 0;
     }
     // the activations are O(1); a chain of f16 roundings through four GEMMs stays within a few 1e-3
-    const bool ok = e1 < 2e-2 && e2 < 2e-2 && e3 < 5e-3 && touched0 == 0 && threw && ends_ok;
+    const bool ok = e1 < 2e-2 && e2 < 2e-2 && e3 < 5e-3 && touched0 == 0 && threw && ends_ok && wire_ok;
     printf(ok ? "PASS\n" : "FAIL\n");
     return ok ? 0 : 1;
 }
