@@ -10,7 +10,8 @@ outside the layer loop, and is timed separately.
 
 --workload C2 | C4 | C5 run the other configurations (C2 adds the RMSNorm and SiLU-gate kernels of the
 layer, C4 is the ragged causal prefill + page store, C5 the e4m3-KV decode); ENDS and MIGRATE time the
-row gathers / argmax either side of the layer loop and the KV migration pack / unpack.  One GPU only.
+row gathers / argmax either side of the layer loop and the KV migration pack / unpack, LAYERS a
+small-batch 32-layer decode step launched eagerly and replayed from a HIP graph.  One GPU only.
 """
 import argparse
 import json
@@ -30,7 +31,7 @@ def parse():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=None)
     ap.add_argument("--warmup", type=int, default=None)
-    ap.add_argument("--workload", default="C3", choices=["C2", "C3", "C4", "C5", "ENDS", "MIGRATE"])
+    ap.add_argument("--workload", default="C3", choices=["C2", "C3", "C4", "C5", "ENDS", "MIGRATE", "LAYERS"])
     ap.add_argument("--layers", type=int, default=None, help="layer planes of the KV pool the steps cycle over")
     ap.add_argument("--seed", type=lambda s: int(s, 0), default=0x5EED)
     ap.add_argument("--sigma", type=float, default=1.0, help="sigma of the log-normal context lengths (C3)")
@@ -475,6 +476,88 @@ def bench_migrate(args):
                          "kernel": "bz::wire_kernel (pack), payload read + payload written"}}
 
 
+def bench_layers(args):
+    """Small-batch decode through all 32 layers of a Llama-3-8B-shaped model (attention part of each layer:
+    fused RoPE + KV append, paged decode), launched eagerly and replayed from one HIP graph.  At this
+    size every kernel is shorter than a launch, so the step is bound by the launches, which is what the
+    graph removes.  One plan and one page-table upload per step serve all layers, as in the reference
+    (src/model/llama.h:363-375)."""
+    import numpy as np
+    import torch
+
+    from blitz_scale_amd import kernel as K, workloads as wl
+    from blitz_scale_amd._lib import BZ_LAYOUT_HND, BZ_ROPE_NONE
+
+    layers, B, Hq, Hkv, D, P, ctx = 32, 8, 32, 8, 128, 16, 1024
+    rng = np.random.default_rng(args.seed)
+    lens = np.full(B, ctx, np.int64)
+    max_pages = 2 * B * (ctx // P + 1)
+    indices, indptr, lpl = wl.page_table_for(lens, P, max_pages, rng)
+    stride_page, _, _ = wl.strides(BZ_LAYOUT_HND, Hkv, P, D)
+    g = torch.Generator(device="cuda")
+    g.manual_seed(args.seed)
+    pool = torch.randn(layers * max_pages * stride_page, dtype=torch.bfloat16, device="cuda", generator=g)
+    q = torch.randn((layers, B, Hq, D), dtype=torch.bfloat16, device="cuda", generator=g)
+    k = torch.randn((layers, B, Hkv, D), dtype=torch.bfloat16, device="cuda", generator=g)
+    v = torch.randn((layers, B, Hkv, D), dtype=torch.bfloat16, device="cuda", generator=g)
+    q_raw = q.clone()
+    out = torch.empty_like(q)
+    pts = []
+    for l in range(layers):
+        pt = K.PageTable(B, P, Hkv, D, pool, layout=BZ_LAYOUT_HND)
+        pt.set_layer(l, max_pages)
+        pt.indices, pt.indptr, pt.last_page_len = indices, indptr, lpl
+        pts.append(pt)
+    pts[0].upload()
+    for pt in pts[1:]:
+        pt.indices_d, pt.indptr_d, pt.last_page_len_d = pts[0].indices_d, pts[0].indptr_d, pts[0].last_page_len_d
+    float_ws = torch.empty(128 << 20, dtype=torch.uint8, device="cuda")
+    int_ws = torch.empty(8 << 20, dtype=torch.uint8, device="cuda")
+    handler = K.BlitzBatchDecodeHandler()
+    handler.plan(float_ws, float_ws.numel(), int_ws, int_ws.numel(), indptr, lpl, B, Hq, Hkv, D, P,
+                 split_tokens=args.split_tokens)
+
+    def step_layers(stream=None):
+        for l in range(layers):
+            K.append_decode_kv_cache(pts[l], k[l], v[l], q=q[l], num_qo_heads=Hq, rope=True, rope_theta=5e5,
+                                     stream=stream)
+            K.batch_decode_attention(handler, q[l], pts[l], out[l], Hq, rope_mode=BZ_ROPE_NONE, stream=stream)
+
+    steps = args.steps or 50
+    warmup = args.warmup if args.warmup is not None else 5
+    eager_ms, _ = timed(lambda i, e: step_layers(), steps, warmup, torch_events=False)
+    q.copy_(q_raw)
+    torch.cuda.synchronize()
+    step_layers()
+    torch.cuda.synchronize()
+    want = out.clone()
+    side = torch.cuda.Stream()
+    graph = torch.cuda.CUDAGraph()
+    q.copy_(q_raw)
+    torch.cuda.synchronize()
+    with torch.cuda.graph(graph, stream=side):
+        step_layers(torch.cuda.current_stream().cuda_stream)
+    torch.cuda.synchronize()
+    q.copy_(q_raw)
+    out.zero_()
+    graph.replay()
+    torch.cuda.synchronize()
+    same = bool(torch.equal(out.view(torch.int16), want.view(torch.int16)))
+    graph_ms, _ = timed(lambda i, e: graph.replay(), steps, warmup, torch_events=False)
+    kv_bytes = layers * B * ctx * 2 * Hkv * D * 2
+    return {"metric": "small_batch_decode_32_layers_us", "value": round(graph_ms * 1e3, 2), "unit": "us/step",
+            "n_gpus": 1, "steps": steps, "warmup": warmup, "ms_per_step": round(graph_ms, 6),
+            "higher_is_better": False, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+            "config": {"workload": "LAYERS: attention part (fused RoPE + append, paged decode) of 32 Llama-3-8B "
+                                   f"layers, batch {B}, context {ctx}, one plan per step; value = HIP-graph replay"},
+            "eager_us_per_step": round(eager_ms * 1e3, 2), "graph_us_per_step": round(graph_ms * 1e3, 2),
+            "us_per_layer": {"eager": round(eager_ms * 1e3 / layers, 2), "graph": round(graph_ms * 1e3 / layers, 2)},
+            "graph_replay_bit_exact_vs_eager": same,
+            "roofline": {"bound": "hbm", "achieved": round(kv_bytes / (graph_ms * 1e-3) / 1e9, 1), "peak": 8000.0,
+                         "unit": "GB/s", "frac": round(kv_bytes / (graph_ms * 1e-3) / 1e9 / 8000.0, 4), "traffic": None,
+                         "kernel": "whole replayed step (launch-latency bound at this size, not a kernel figure)"}}
+
+
 def main():
     args = parse()
     import torch
@@ -492,6 +575,8 @@ def main():
         res = bench_ends(args)
     elif args.workload == "MIGRATE":
         res = bench_migrate(args)
+    elif args.workload == "LAYERS":
+        res = bench_layers(args)
     else:
         res = bench_prefill(args) if args.workload == "C4" else bench_decode(args, args.workload)
     print(json.dumps(res))
