@@ -36,6 +36,9 @@ def parse():
     ap.add_argument("--seed", type=lambda s: int(s, 0), default=0x5EED)
     ap.add_argument("--sigma", type=float, default=1.0, help="sigma of the log-normal context lengths (C3)")
     ap.add_argument("--split-tokens", type=int, default=2048)
+    ap.add_argument("--page-size", type=int, default=None,
+                    help="tokens per KV page for the decode workloads (default: the configuration's 16; the "
+                         "reference's production value is 64, src/server/disaggregate.cc:310)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also launch a few plain device copies of 1 GiB (reference point for rocprofv3 --pmc byte counters)")
@@ -97,7 +100,7 @@ def timed(step, steps, warmup, torch_events=True):
 def measured_traffic(name, args):
     """HBM bytes per launch of the dominant kernel, measured offline with rocprofv3 --pmc (profiles/*.md);
     only reported for the exact workload it was measured on."""
-    if args.seed != 0x5EED or args.sigma != 1.0 or args.split_tokens != 2048:
+    if args.seed != 0x5EED or args.sigma != 1.0 or args.split_tokens != 2048 or args.page_size:
         return None
     try:
         with open(os.path.join(ROOT, "blitz_scale_amd", "measured_traffic.json")) as f:
@@ -115,7 +118,7 @@ def bench_decode(args, name):
 
     dev = "cuda"
     cfg = dict(wl.CONFIGS[name])
-    B, Hq, Hkv, D, P = cfg["batch"], cfg["Hq"], cfg["Hkv"], cfg["D"], cfg["P"]
+    B, Hq, Hkv, D, P = cfg["batch"], cfg["Hq"], cfg["Hkv"], cfg["D"], args.page_size or cfg["P"]
     theta = cfg["rope_theta"]
     tdt = torch.float16 if cfg["dtype"] == BZ_F16 else torch.bfloat16
     fp8 = cfg["kv_dtype"] == BZ_E4M3
