@@ -1,6 +1,13 @@
 """ctypes front end of the CPU checker (oracle/bz_oracle.c).  TEST INFRASTRUCTURE ONLY:
 imported by tests/, __graft_entry__.smoke() and bench.py's cpu_baseline leg, never by the
 product.  Arrays are numpy: uint16 bits for f16/bf16, uint8 bits for e4m3, int32 page tables.
+
+Everything numeric goes through the C file; the KV migration wire format (kv_pages_pack /
+kv_pages_unpack) is byte and index work and is stated here in numpy, following
+src/blitz/migration_manager.h:86-92 (page addressing) and :455-467 (message order).  Every function
+is pinned by independent checks in tests/ (closed forms, float64 dense implementations, library
+routines, literal walks of the reference's loops); none is "parity unpinned" except, for all of them,
+agreement with the reference's private FlashInfer fork, whose source is not in the checkout.
 """
 import ctypes as C
 import os
