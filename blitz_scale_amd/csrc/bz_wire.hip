@@ -74,7 +74,9 @@ __global__ __launch_bounds__(256) void wire_kernel(WireArgs a) {
         if (!live[u]) continue;
         const uint32_t c = (uint32_t)(g / a.vecs_per_chunk), e = (uint32_t)(g % a.vecs_per_chunk) * 8;
         const uint32_t i = c / a.layer_cnt, l = c % a.layer_cnt;
-        pool_off[u] = ((uint64_t)(a.start_layer + l) * a.max_pages + (uint64_t)a.page_ids[i]) * a.stride_page + e;
+        const int32_t page = a.page_ids[i];
+        if ((uint64_t)(uint32_t)page >= a.max_pages) { live[u] = false; continue; } // not a page of this pool: skipped
+        pool_off[u] = ((uint64_t)(a.start_layer + l) * a.max_pages + (uint64_t)page) * a.stride_page + e;
         if (sizeof(PT) != sizeof(WT)) {
             const uint32_t half = (uint32_t)(a.stride_page / 2);
             const bool is_v = e >= half;

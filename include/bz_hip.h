@@ -217,7 +217,8 @@ int bz_batch_find_max(uint32_t* output_indices, const void* input, int dtype, ui
  *   wire_dtype: the pool's type (bit copy), or BZ_E4M3 for a 16-bit pool: elements travel as
  *               e4m3(x / scale) and arrive as e4m3 * scale, scale = k_scale / v_scale[l*num_kv_heads +
  *               head] (device arrays [layer_cnt][num_kv_heads]; NULL = 1), half the bytes.
- * Pages listed twice in an unpack race.  Launch only; no allocation, copy or synchronisation.
+ * Page ids outside [0, max_pages) are skipped (their chunk of `wire` is left untouched by pack, ignored
+ * by unpack).  Pages listed twice in an unpack race.  Launch only; no allocation, copy or synchronisation.
  * ------------------------------------------------------------------------------------- */
 uint64_t bz_kv_wire_bytes(uint32_t num_pages, uint32_t layer_cnt, const bz_paged_kv_t* kv, int wire_dtype);
 int bz_kv_pages_pack(const void* pool_base, uint64_t max_pages, const bz_paged_kv_t* kv, const int32_t* page_ids,
