@@ -44,6 +44,16 @@ __device__ __forceinline__ uint16_t f32_to_bf16_bits(float f) {
     return (uint16_t)(u >> 16);
 }
 
+// One rotate-half pair: (x, y) -> (x c - y s, y c + x s).  Every product and sum is rounded on its own
+// (no fused multiply-add), so that all kernels of the library that rotate the same row get the same
+// bits, and so does a scalar restatement compiled without contraction.
+__device__ __forceinline__ void rope_pair(float x, float y, float c, float s, float& xr, float& yr) {
+#pragma clang fp contract(off)
+    const float xc = x * c, ys = y * s, yc = y * c, xs = x * s;
+    xr = xc - ys;
+    yr = yc + xs;
+}
+
 template <typename T> struct StoreCvt;
 template <> struct StoreCvt<f16_t> {
     __device__ static __forceinline__ f16_t from(float f) { return f16_t{f32_to_f16_bits(f)}; }

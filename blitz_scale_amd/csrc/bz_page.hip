@@ -90,7 +90,8 @@ __global__ __launch_bounds__(256) void page_write_kernel(PageWriteArgs a) {
 #pragma unroll
             for (int e = 0; e < 8; ++e) {
                 const float c = s_cos[lane * 8 + e], s = s_sin[lane * 8 + e];
-                const float xr = x[e] * c - y[e] * s, yr = y[e] * c + x[e] * s;
+                float xr, yr;
+                rope_pair(x[e], y[e], c, s, xr, yr);
                 x[e] = xr;
                 y[e] = yr;
             }
@@ -128,7 +129,8 @@ __global__ __launch_bounds__(256) void page_write_kernel(PageWriteArgs a) {
 #pragma unroll
             for (int e = 0; e < 8; ++e) {
                 const float c = s_cos[lane * 8 + e], s = s_sin[lane * 8 + e];
-                const float xr = x[e] * c - y[e] * s, yr = y[e] * c + x[e] * s;
+                float xr, yr;
+                rope_pair(x[e], y[e], c, s, xr, yr);
                 x[e] = xr;
                 y[e] = yr;
             }
