@@ -293,8 +293,8 @@ static void launch_zero(const DecodePlan* p, void* out, uint32_t row_elems, hipS
 
 int decode_fast_path(const DecodePlan* p, const void* q, void* out, float* lse, int q_dtype, int out_dtype,
                      int rope_mode, float sm_scale_log2, const RopeFreqs& freqs, const bz_paged_kv_t* kv,
-                     uint32_t num_qo_heads, const float* k_scale, const float* v_scale, hipStream_t s,
-                     const void* k_new = nullptr, const void* v_new = nullptr, int fused_rope = 0); // bz_decode_mfma.hip
+                     uint32_t num_qo_heads, const float* k_scale, const float* v_scale,
+                     hipStream_t s); // bz_decode_mfma.hip
 
 } // namespace bz
 
@@ -378,44 +378,4 @@ extern "C" int bz_batch_decode(bz_decode_plan_t* plan_, const void* q, int q_dty
         BZ_LAUNCH_CHECK();
     }
     return 0;
-}
-
-extern "C" int bz_append_and_decode(bz_decode_plan_t* plan_, const void* q, int q_dtype, const bz_paged_kv_t* kv,
-                                    const void* k_new, const void* v_new, void* out, int out_dtype,
-                                    uint32_t num_qo_heads, int rope, float rope_theta, float sm_scale, float* lse,
-                                    void* stream) {
-    DecodePlan* p = reinterpret_cast<DecodePlan*>(plan_);
-    if (!p || !kv || !q || !out || !k_new || !v_new) return BZ_ERR_BAD_ARG;
-    if (!p->planned) return BZ_ERR_NOT_PLANNED;
-    if (kv->batch_size != p->batch_size || kv->page_size != p->page_size || kv->num_kv_heads != p->num_kv_heads ||
-        kv->head_dim != p->head_dim || num_qo_heads != p->num_qo_heads)
-        return BZ_ERR_BAD_ARG;
-    if (q_dtype != BZ_F16 && q_dtype != BZ_BF16) return BZ_ERR_UNSUPPORTED;
-    if (out_dtype != q_dtype && out_dtype != BZ_F32) return BZ_ERR_UNSUPPORTED;
-    hipStream_t s = (hipStream_t)stream;
-    if (p->batch_size == 0) return 0;
-    const int D = (int)kv->head_dim;
-    if (kv->kv_dtype == q_dtype && p->num_segments > 0 && !p->force_general) {
-        if (!(sm_scale > 0.f)) sm_scale = 1.0f / sqrtf((float)D);
-        const RopeFreqs freqs = make_rope_freqs(D, rope_theta > 0.f ? rope_theta : 1e4f);
-        const int rc = decode_fast_path(p, q, out, lse, q_dtype, out_dtype, BZ_ROPE_NONE, sm_scale * 1.4426950408889634f,
-                                        freqs, kv, num_qo_heads, nullptr, nullptr, s, k_new, v_new, rope ? 1 : 0);
-        if (rc == 0) {
-            if (p->num_empty > 0) {
-                const uint32_t row = num_qo_heads * D;
-                if (out_dtype == BZ_F32) launch_zero<float>(p, out, row, s);
-                else if (out_dtype == BZ_F16) launch_zero<f16_t>(p, out, row, s);
-                else launch_zero<bf16_t>(p, out, row, s);
-                BZ_LAUNCH_CHECK();
-            }
-            return 0;
-        }
-        if (rc != BZ_ERR_UNSUPPORTED) return rc;
-    }
-    // two launches: the page writer (K rotated on the way in, q left alone), then the decode call, which
-    // rotates q itself
-    int rc = bz_append_decode_kv(kv, k_new, v_new, q_dtype, nullptr, 0, rope, rope_theta, nullptr, nullptr, stream);
-    if (rc) return rc;
-    return bz_batch_decode(plan_, q, q_dtype, kv, out, out_dtype, num_qo_heads, rope ? BZ_ROPE_Q_ONLY : BZ_ROPE_NONE,
-                           rope_theta, sm_scale, nullptr, nullptr, lse, stream);
 }

@@ -47,13 +47,6 @@ struct MfmaDecodeArgs {
     const float* k_scale; // e4m3 pool only: per-kv-head dequantisation factors (nullptr = 1)
     const float* v_scale;
     RopeFreqs freqs;
-    // fused step only: the new token's K and V rows [batch][kv head][128] (not yet in the pool), the number
-    // of wave slots of the schedule (workgroups past them write those rows into the pool) and whether
-    // q and the new K row are rotated (position seq_len-1) on the way
-    const char* k_new;
-    const char* v_new;
-    uint32_t num_slots, batch_size, num_kv_heads;
-    int fused_rope;
 };
 
 template <bool BF16> struct Mma;
@@ -130,47 +123,7 @@ constexpr int kInfoInts = 12; // per-tile description kept in LDS (see fetch_inf
 // on their way to the matrix cores; the per-head scales are folded into the softmax scale and into
 // the final normalisation.  A lane then fetches 16 bytes = 16 elements of a K row, so the contraction
 // index of MFMA step ks, lane group j, element i is d = 64*(ks/2) + 16*j + 8*(ks%2) + i (q follows).
-// Writer half of the fused step: one wave stores the new token of sequence b at position seq_len-1
-// (src/kernel/page.cu:96-115), K rotated like the q rows when the step rotates.  Lane l owns the
-// rotate-half pair (l, l+64) of every row.
-template <bool BF16>
-__device__ __forceinline__ void fused_append_row(const MfmaDecodeArgs& a, int b) {
-    using M = Mma<BF16>;
-    const int lane = threadIdx.x;
-    const int np = a.indptr[b + 1] - a.indptr[b];
-    if (np <= 0) return;
-    const int P = (int)a.page_size;
-    const int pos = (np - 1) * P + a.last_page_len[b] - 1;
-    const size_t page = (size_t)a.indices[a.indptr[b] + pos / P];
-    const int slot = pos % P;
-    float sn = 0.f, cs = 1.f;
-    if (a.fused_rope) sincosf((float)pos * a.freqs.f[lane], &sn, &cs);
-    for (uint32_t h = 0; h < a.num_kv_heads; ++h) {
-        const uint16_t* kr = reinterpret_cast<const uint16_t*>(a.k_new) + ((size_t)b * a.num_kv_heads + h) * 128;
-        const uint16_t* vr = reinterpret_cast<const uint16_t*>(a.v_new) + ((size_t)b * a.num_kv_heads + h) * 128;
-        const size_t off = page * a.stride_page + (size_t)slot * a.stride_n + (size_t)h * a.stride_h;
-        uint16_t* kd = reinterpret_cast<uint16_t*>(const_cast<char*>(a.k_data)) + off;
-        uint16_t* vd = reinterpret_cast<uint16_t*>(const_cast<char*>(a.v_data)) + off;
-        uint16_t k0 = kr[lane], k1 = kr[lane + 64];
-        if (a.fused_rope) {
-            const float x = M::unpack_lo(k0), y = M::unpack_lo(k1);
-            float xr, yr;
-            rope_pair(x, y, cs, sn, xr, yr);
-            k0 = (uint16_t)(M::pack2(xr, 0.f) & 0xffffu);
-            k1 = (uint16_t)(M::pack2(yr, 0.f) & 0xffffu);
-        }
-        kd[lane] = k0;
-        kd[lane + 64] = k1;
-        vd[lane] = vr[lane];
-        vd[lane + 64] = vr[lane + 64];
-    }
-}
-
-// FUSED: the decode step in one launch.  q is rotated in registers (rounded to the storage type, as a
-// separate append would leave it in memory), the new token's K and V rows are taken from the caller's
-// buffers instead of the pool, and the workgroups past the schedule's wave slots write those rows into
-// the pool for the steps to come.
-template <bool BF16, typename OT, bool ROPE_Q, bool KV8, bool FUSED = false>
+template <bool BF16, typename OT, bool ROPE_Q, bool KV8>
 __global__ __launch_bounds__(64, 2) void decode_mfma_kernel(MfmaDecodeArgs a, const char* __restrict__ q_ptr,
                                                             const char* __restrict__ k_data,
                                                             const char* __restrict__ v_data,
@@ -181,18 +134,10 @@ __global__ __launch_bounds__(64, 2) void decode_mfma_kernel(MfmaDecodeArgs a, co
     using M = Mma<BF16>;
     __shared__ __attribute__((aligned(16))) unsigned char v_lds[kTileTok * kVRowBytes];
     __shared__ __attribute__((aligned(16))) int info_lds[2][32][kInfoInts];
-    // fused step: the new token's K row as MFMA operand slices (rotated, rounded), parked from the start
-    // of the piece that ends the sequence until the tile that holds the row
-    __shared__ uint4 k_stash[FUSED ? 4 : 1][64];
+    // cos / sin of position * frequency i for the piece being opened: one sincosf per lane instead of
+    // sixteen (each lane needs the angles of its own 16 contraction indices)
+    __shared__ float rope_cs[ROPE_Q ? 2 : 1][64];
 
-    if constexpr (FUSED) {
-        if (blockIdx.x >= a.num_slots) {
-            fused_append_row<BF16>(a, (int)(blockIdx.x - a.num_slots));
-            return;
-        }
-    }
-    constexpr bool Q_TAIL = ROPE_Q && !FUSED; // q = head + tail of the storage type, both contracted
-    const bool rotate_q = ROPE_Q && (!FUSED || a.fused_rope);
     const int lane = threadIdx.x;
     const int n = lane & 15; // query head (scores) / d column (output) / token row (K operand)
     const int j = lane >> 4; // lane group: which 8-wide slice of the MFMA contraction
@@ -339,58 +284,35 @@ __global__ __launch_bounds__(64, 2) void decode_mfma_kernel(MfmaDecodeArgs a, co
         if (uc.flags & 1) { // ================= first tile of a piece =================
 #pragma unroll
             for (int ks = 0; ks < 4; ++ks) { qhi[ks] = qnext[ks]; qlo[ks] = make_uint4(0, 0, 0, 0); }
-            // fused step: this piece ends the sequence, so it will need the new token's K row
-            const bool has_last = FUSED && tok_end == seq_len; // wave-uniform
-            uint4 kn[4];
-            if constexpr (FUSED) {
-                if (has_last) {
-                    const char* krow = a.k_new + ((size_t)uc.seq * a.num_kv_heads + (size_t)uc.kvh) * 256;
-#pragma unroll
-                    for (int ks = 0; ks < 4; ++ks) kn[ks] = *reinterpret_cast<const uint4*>(krow + d_of(ks) * 2);
-                }
+            if (ROPE_Q) {
+                float sn1, cs1;
+                sincosf((float)(seq_len - 1) * a.freqs.f[lane], &sn1, &cs1);
+                wave_lds_sync(); // the previous piece's reads of the table are done
+                rope_cs[0][lane] = cs1;
+                rope_cs[ROPE_Q ? 1 : 0][lane] = sn1; // (the index keeps the one-row dummy of the other instantiations in bounds)
+                wave_lds_sync();
             }
-            if (rotate_q && (FUSED || n < G)) { // lanes without a q row hold zeros, which rotate to zeros
+            if (ROPE_Q && n < G) {
                 // the rotated q is split into a storage-precision head and tail (q = hi + lo) and both are
-                // contracted, so rotating inside the kernel costs no precision (the fused step keeps the
-                // head only: that is the q a separate append would have left in memory)
-                const float pos = (float)(seq_len - 1);
+                // contracted, so rotating inside the kernel costs no precision
 #pragma unroll
                 for (int ks = 0; ks < 2; ++ks) { // dims d = 32ks+8j+e pair with d+64, held at ks+2
 #pragma unroll
                     for (int w = 0; w < 4; ++w) {
                         float x[2] = {M::unpack_lo(u4(qhi[ks], w)), M::unpack_hi(u4(qhi[ks], w))};
                         float y[2] = {M::unpack_lo(u4(qhi[ks + 2], w)), M::unpack_hi(u4(qhi[ks + 2], w))};
-                        float xr[2], yr[2], sn[2], cs[2];
+                        float xr[2], yr[2];
 #pragma unroll
                         for (int e = 0; e < 2; ++e) {
-                            sincosf(pos * a.freqs.f[d_of(ks) + 2 * w + e], &sn[e], &cs[e]);
-                            rope_pair(x[e], y[e], cs[e], sn[e], xr[e], yr[e]);
+                            const float c = rope_cs[0][d_of(ks) + 2 * w + e], s = rope_cs[ROPE_Q ? 1 : 0][d_of(ks) + 2 * w + e];
+                            rope_pair(x[e], y[e], c, s, xr[e], yr[e]);
                         }
                         const uint32_t xh = M::pack2(xr[0], xr[1]), yh = M::pack2(yr[0], yr[1]);
                         u4(qhi[ks], w) = xh;
                         u4(qhi[ks + 2], w) = yh;
-                        if (Q_TAIL) {
-                            u4(qlo[ks], w) = M::pack2(xr[0] - M::unpack_lo(xh), xr[1] - M::unpack_hi(xh));
-                            u4(qlo[ks + 2], w) = M::pack2(yr[0] - M::unpack_lo(yh), yr[1] - M::unpack_hi(yh));
-                        }
-                        if constexpr (FUSED) {
-                            if (has_last) { // the new K row, same angles
-                                const float kx[2] = {M::unpack_lo(u4(kn[ks], w)), M::unpack_hi(u4(kn[ks], w))};
-                                const float ky[2] = {M::unpack_lo(u4(kn[ks + 2], w)), M::unpack_hi(u4(kn[ks + 2], w))};
-                                float kxr[2], kyr[2];
-                                rope_pair(kx[0], ky[0], cs[0], sn[0], kxr[0], kyr[0]);
-                                rope_pair(kx[1], ky[1], cs[1], sn[1], kxr[1], kyr[1]);
-                                u4(kn[ks], w) = M::pack2(kxr[0], kxr[1]);
-                                u4(kn[ks + 2], w) = M::pack2(kyr[0], kyr[1]);
-                            }
-                        }
+                        u4(qlo[ks], w) = M::pack2(xr[0] - M::unpack_lo(xh), xr[1] - M::unpack_hi(xh));
+                        u4(qlo[ks + 2], w) = M::pack2(yr[0] - M::unpack_lo(yh), yr[1] - M::unpack_hi(yh));
                     }
-                }
-            }
-            if constexpr (FUSED) {
-                if (has_last) {
-#pragma unroll
-                    for (int ks = 0; ks < 4; ++ks) k_stash[ks][lane] = kn[ks];
                 }
             }
             m_run = -INFINITY;
@@ -429,26 +351,6 @@ __global__ __launch_bounds__(64, 2) void decode_mfma_kernel(MfmaDecodeArgs a, co
                 if constexpr (KV8) kcur[u][ks] = fp8x8_to_op<BF16>(kreg[u][ks >> 1], ks & 1);
                 else kcur[u][ks] = kreg[u][ks];
             }
-        if constexpr (FUSED) {
-            // the tile that holds position seq_len-1: that row is not in the pool yet, it comes from the
-            // caller's k / v rows (K rotated and rounded exactly as the writer workgroups store it)
-            const int last = seq_len - 1 - tile_tok0; // wave-uniform
-            if (last >= 0 && last < kTileTok && seq_len <= tok_end) {
-                if (lane < 16) {
-                    const size_t row = ((size_t)uc.seq * a.num_kv_heads + (size_t)uc.kvh) * 256;
-                    const uint4 vn = *reinterpret_cast<const uint4*>(a.v_new + row + lane * 16);
-                    *reinterpret_cast<uint4*>(v_lds + last * kVRowBytes + lane * 16) = vn;
-                }
-                if (n == (last & 15)) {
-#pragma unroll
-                    for (int ks = 0; ks < 4; ++ks) {
-                        const uint4 kn = k_stash[ks][lane];
-                        if (last < 16) kcur[0][ks] = kn;
-                        else kcur[1][ks] = kn;
-                    }
-                }
-            }
-        }
         if (g + 1 < g_end) {
             if (i + 1 == 32) { chunk_base += 32; buf ^= 1; }
             if (un.flags & 1) issue_q(un); // next tile opens a new piece
@@ -461,7 +363,7 @@ __global__ __launch_bounds__(64, 2) void decode_mfma_kernel(MfmaDecodeArgs a, co
             s[u] = f32x4_t{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
             for (int ks = 0; ks < 4; ++ks) s[u] = M::run(kcur[u][ks], qhi[ks], s[u]);
-            if (Q_TAIL) {
+            if (ROPE_Q) {
 #pragma unroll
                 for (int ks = 0; ks < 4; ++ks) s[u] = M::run(kcur[u][ks], qlo[ks], s[u]);
             }
@@ -608,18 +510,11 @@ static void launch_mfma_k(const DecodePlan* p, const MfmaDecodeArgs& a, hipStrea
     hipLaunchKernelGGL((decode_mfma_kernel<BF16, OT, ROPE_Q, KV8>), dim3(p->mfma_slots), dim3(64), 0, s, a,
                        (const char*)a.q, a.k_data, a.v_data, a.indices, a.pieces, a.tiles, a.tile_ptr);
 }
-template <bool BF16, typename OT>
-static void launch_mfma_fused(const DecodePlan* p, const MfmaDecodeArgs& a, hipStream_t s) {
-    hipLaunchKernelGGL((decode_mfma_kernel<BF16, OT, true, false, true>), dim3(p->mfma_slots + a.batch_size), dim3(64), 0,
-                       s, a, (const char*)a.q, a.k_data, a.v_data, a.indices, a.pieces, a.tiles, a.tile_ptr);
-}
 
 template <bool BF16, typename OT>
 static int launch_mfma(const DecodePlan* p, const MfmaDecodeArgs& a, bool kv8, hipStream_t s) {
     if (p->time_start) BZ_CHECK_HIP(hipEventRecord(p->time_start, s));
-    if (a.k_new) {
-        launch_mfma_fused<BF16, OT>(p, a, s);
-    } else if (kv8) {
+    if (kv8) {
         if (a.rope_q) launch_mfma_k<BF16, OT, true, true>(p, a, s);
         else launch_mfma_k<BF16, OT, false, true>(p, a, s);
     } else {
@@ -638,12 +533,9 @@ static int launch_mfma(const DecodePlan* p, const MfmaDecodeArgs& a, bool kv8, h
 
 int decode_fast_path(const DecodePlan* p, const void* q, void* out, float* lse, int q_dtype, int out_dtype,
                      int rope_mode, float sm_scale_log2, const RopeFreqs& freqs, const bz_paged_kv_t* kv,
-                     uint32_t num_qo_heads, const float* k_scale, const float* v_scale, hipStream_t s,
-                     const void* k_new, const void* v_new, int fused_rope) {
+                     uint32_t num_qo_heads, const float* k_scale, const float* v_scale, hipStream_t s) {
     if (!p->mfma_ok || p->mfma_slots == 0) return BZ_ERR_UNSUPPORTED;
     const bool kv8 = kv->kv_dtype == BZ_E4M3;
-    if (k_new && (kv8 || !v_new || rope_mode != BZ_ROPE_NONE || (((uintptr_t)k_new | (uintptr_t)v_new) % 16)))
-        return BZ_ERR_UNSUPPORTED;
     if ((!kv8 && kv->kv_dtype != q_dtype) || rope_mode == BZ_ROPE_FULL) return BZ_ERR_UNSUPPORTED;
     if (!kv8 && (k_scale || v_scale)) return BZ_ERR_UNSUPPORTED;
     const uint64_t es = kv8 ? 1 : 2;
@@ -661,9 +553,6 @@ int decode_fast_path(const DecodePlan* p, const void* q, void* out, float* lse, 
     a.sm_scale_log2 = sm_scale_log2;
     a.k_scale = k_scale; a.v_scale = v_scale;
     a.freqs = freqs;
-    a.k_new = (const char*)k_new; a.v_new = (const char*)v_new;
-    a.num_slots = p->mfma_slots; a.batch_size = p->batch_size; a.num_kv_heads = kv->num_kv_heads;
-    a.fused_rope = fused_rope;
     if (q_dtype == BZ_BF16)
         return out_dtype == BZ_F32 ? launch_mfma<true, float>(p, a, kv8, s) : launch_mfma<true, bf16_t>(p, a, kv8, s);
     return out_dtype == BZ_F32 ? launch_mfma<false, float>(p, a, kv8, s) : launch_mfma<false, f16_t>(p, a, kv8, s);

@@ -180,16 +180,6 @@ def batch_decode_attention(handler, q_input, paged_kv, output, num_qo_heads, *, 
     check(rc, "batchDecodeAttention")
 
 
-def append_and_decode_attention(handler, q_input, paged_kv, k_new, v_new, output, num_qo_heads, *, rope=True,
-                                rope_theta=1e4, sm_scale=0.0, lse=None, stream=None):
-    """append_decode_kv_cache + batch_decode_attention (src/layer/attn.h:196-203) in one call; q is not modified."""
-    s = paged_kv.as_struct()
-    rc = _lib.load().bz_append_and_decode(handler.get(), _ptr(q_input), bz_dtype(q_input), C.byref(s), _ptr(k_new),
-                                          _ptr(v_new), _ptr(output), bz_dtype(output), num_qo_heads, int(rope),
-                                          rope_theta, sm_scale, _ptr(lse), _stream(stream))
-    check(rc, "batchDecodeAttention")
-
-
 def batch_prefill_attention(handler, q_input, qo_indptr, k_input, v_input, kv_indptr, output, batch_size,
                             num_qo_heads, num_kv_heads, head_size, *, causal=True, rope_mode=BZ_ROPE_NONE,
                             rope_theta=1e4, sm_scale=0.0, stream=None):

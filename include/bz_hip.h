@@ -122,21 +122,6 @@ int bz_batch_decode(bz_decode_plan_t* plan, const void* q, int q_dtype, const bz
                     int out_dtype, uint32_t num_qo_heads, int rope_mode, float rope_theta, float sm_scale,
                     const float* k_scale, const float* v_scale, float* lse, void* stream);
 
-/*
- * One decode step of a layer in one call: what bz_append_decode_kv(kv, k_new, v_new, ..., rope) followed
- * by bz_batch_decode(...) compute (src/layer/attn.h:196-203 calls the two back to back), without the
- * launch in between.  The page table must already hold the new token (seq_len counts it, as for
- * bz_append_decode_kv).  rope != 0: q and the new K row are rotated at position seq_len-1 and K is cached
- * rotated; unlike the two-call sequence, q itself is left untouched in memory.  Where the MFMA kernel
- * applies (head_dim 128, page_size % 16 == 0, <= 16 q heads per kv head, pool of q's type) the new rows
- * are read from k_new / v_new by the attention waves and written to the pool by extra workgroups of the
- * same launch; otherwise the two calls are made one after the other.  k_new / v_new: [batch][kv head][dim]
- * of q's type, 16-byte aligned.
- */
-int bz_append_and_decode(bz_decode_plan_t* plan, const void* q, int q_dtype, const bz_paged_kv_t* kv,
-                         const void* k_new, const void* v_new, void* out, int out_dtype, uint32_t num_qo_heads,
-                         int rope, float rope_theta, float sm_scale, float* lse, void* stream);
-
 /* ---------------------------------------------------------------------------------------
  * Prefill plan: replaces BatchPrefillRaggedHandler::plan (flashinfer_types.h:12-41,
  * flashinfer_types.cu:24-49).  Builds the (request, q-tile) work list, longest first.
