@@ -54,6 +54,27 @@ __device__ __forceinline__ void rope_pair(float x, float y, float c, float s, fl
     yr = yc + xs;
 }
 
+// Reductions over the lanes l, l^16 (and l^32) of a wave with the gfx950 lane-swap instructions: the
+// partner's value arrives through the vector ALU instead of an LDS round trip (ds_bpermute).  With the
+// same value in both operands v_permlane16_swap leaves rows {0,0,2,2} in the first result and rows
+// {1,1,3,3} in the second, v_permlane32_swap the lower half twice and the upper half twice.
+__device__ __forceinline__ float lane_max_xor16(float v) {
+    const auto r = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+    return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
+}
+__device__ __forceinline__ float lane_max_xor32(float v) {
+    const auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+    return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
+}
+__device__ __forceinline__ float lane_sum_xor16(float v) {
+    const auto r = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+    return __uint_as_float(r[0]) + __uint_as_float(r[1]);
+}
+__device__ __forceinline__ float lane_sum_xor32(float v) {
+    const auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+    return __uint_as_float(r[0]) + __uint_as_float(r[1]);
+}
+
 template <typename T> struct StoreCvt;
 template <> struct StoreCvt<f16_t> {
     __device__ static __forceinline__ f16_t from(float f) { return f16_t{f32_to_f16_bits(f)}; }

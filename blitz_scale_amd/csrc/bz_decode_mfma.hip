@@ -378,8 +378,7 @@ __global__ __launch_bounds__(64, 2) void decode_mfma_kernel(MfmaDecodeArgs a, co
                 s[u][r] = v;
                 tmax = fmaxf(tmax, v);
             }
-        tmax = fmaxf(tmax, __shfl_xor(tmax, 16, 64));
-        tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
+        tmax = lane_max_xor32(lane_max_xor16(tmax));
         const float m_new = fmaxf(m_run, tmax);   // finite: every tile holds at least one live token
         const float alpha = exp2f(m_run - m_new); // 0 on the first tile (m_run = -inf)
         // The probabilities enter the second contraction as a storage-precision head plus tail
@@ -398,8 +397,7 @@ __global__ __launch_bounds__(64, 2) void decode_mfma_kernel(MfmaDecodeArgs a, co
             u4(pb, 2 * u) = M::pack2(p0 - M::unpack_lo(h01), p1 - M::unpack_hi(h01));
             u4(pb, 2 * u + 1) = M::pack2(p2 - M::unpack_lo(h23), p3 - M::unpack_hi(h23));
         }
-        psum += __shfl_xor(psum, 16, 64);
-        psum += __shfl_xor(psum, 32, 64);
+        psum = lane_sum_xor32(lane_sum_xor16(psum));
         l_run = l_run * alpha + psum;
         m_run = m_new;
 

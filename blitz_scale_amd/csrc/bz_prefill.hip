@@ -271,7 +271,7 @@ __global__ __launch_bounds__(256, 2) void prefill_kernel(PrefillArgs a, const ch
             }
             // the scores stay unscaled in registers: the (positive) softmax scale is applied to the maximum
             // here and to every score inside the fused multiply-add that feeds exp2
-            tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64)) * a.sm_scale_log2;
+            tmax = lane_max_xor32(tmax) * a.sm_scale_log2;
             // The reference maximum only moves when some row's maximum has grown by more than 2^8 since
             // it was last set (wave-uniform decision): until then exp2(s - m_run) is at most 256, which
             // fp32 sums and 16-bit operands hold without loss, and the accumulators need no rescaling.
@@ -302,7 +302,7 @@ __global__ __launch_bounds__(256, 2) void prefill_kernel(PrefillArgs a, const ch
                     if (SPLIT_P) pf_u4(pb[st], w) = M::pack2(p0 - M::lo(hw), p1 - M::hi(hw));
                 }
             }
-            psum += __shfl_xor(psum, 32, 64);
+            psum = lane_sum_xor32(psum);
             l_run += psum;
             __builtin_amdgcn_sched_barrier(0);
             // ---- O^T += V^T P^T: step i takes tokens 16*(i/4) .. +15 and d block i%4
