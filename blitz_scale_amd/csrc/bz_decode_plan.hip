@@ -122,6 +122,8 @@ extern "C" int bz_decode_plan(bz_decode_plan_t* plan_, void* float_buffer, size_
             const int64_t len = (int64_t)(np - 1) * page_size + last_page_len_h[b];
             total_tiles += (uint64_t)((len + 31) / 32) * num_kv_heads;
         }
+        int page_shift = -1; // log2(page_size) when it is a power of two
+        if ((page_size & (page_size - 1)) == 0) { page_shift = 0; while ((1u << page_shift) < page_size) ++page_shift; }
         const uint64_t max_slots = (uint64_t)cus * 8;
         const uint64_t share = std::max<uint64_t>(1, (total_tiles + max_slots - 1) / max_slots);
         const uint32_t cap_tiles = never_split ? 0x7fffffffu : std::max<uint32_t>(1, split_tokens / 32);
@@ -164,10 +166,24 @@ extern "C" int bz_decode_plan(bz_decode_plan_t* plan_, void* float_buffer, size_
                     const int32_t take = never_split ? (int32_t)left
                                                      : (int32_t)std::min<uint64_t>({left, room, (uint64_t)cap_tiles});
                     room -= std::min<uint64_t>(room, (uint64_t)take);
-                    for (int32_t tt = t; tt < t + take; ++tt) {
-                        const int32_t pg0 = std::min<int32_t>((int32_t)(((int64_t)tt * 32) / page_size), np - 1);
-                        const int32_t pg1 = std::min<int32_t>((int32_t)(((int64_t)tt * 32 + 16) / page_size), np - 1);
-                        mt.push_back({indptr_h[b] + pg0, indptr_h[b] + pg1, tt, (int32_t)mp.size()});
+                    // one record per tile; page sizes are powers of two in practice, so the two page
+                    // indices of a tile come from shifts rather than 64-bit divisions
+                    const size_t first_rec = mt.size();
+                    mt.resize(first_rec + (size_t)take);
+                    MfmaTile* rec = mt.data() + first_rec;
+                    const int32_t piece_id = (int32_t)mp.size(), ip0 = indptr_h[b];
+                    if (page_shift >= 0) {
+                        for (int32_t tt = t; tt < t + take; ++tt, ++rec) {
+                            const int32_t pg0 = std::min<int32_t>((int32_t)(((int64_t)tt * 32) >> page_shift), np - 1);
+                            const int32_t pg1 = std::min<int32_t>((int32_t)(((int64_t)tt * 32 + 16) >> page_shift), np - 1);
+                            *rec = {ip0 + pg0, ip0 + pg1, tt, piece_id};
+                        }
+                    } else {
+                        for (int32_t tt = t; tt < t + take; ++tt, ++rec) {
+                            const int32_t pg0 = std::min<int32_t>((int32_t)(((int64_t)tt * 32) / page_size), np - 1);
+                            const int32_t pg1 = std::min<int32_t>((int32_t)(((int64_t)tt * 32 + 16) / page_size), np - 1);
+                            *rec = {ip0 + pg0, ip0 + pg1, tt, piece_id};
+                        }
                     }
                     mp.push_back({(int32_t)b, (int32_t)h, t, t + take, -1, -1, 0, 0, indptr_h[b], np, (int32_t)len,
                                   {0, 0, 0, 0, 0}});
@@ -222,7 +238,7 @@ extern "C" int bz_decode_plan(bz_decode_plan_t* plan_, void* float_buffer, size_
         p->staging_bytes = want;
     }
     char* st = (char*)p->staging;
-    if (total) memset(st, 0, total);
+    // (the padding between the 256-byte aligned sections is never read: no need to clear the buffer)
     if (!segs.empty()) memcpy(st, segs.data(), segs.size() * sizeof(DecodeSegment));
     if (!combos.empty()) memcpy(st + seg_bytes, combos.data(), combos.size() * sizeof(DecodeCombine));
     if (!empty.empty()) memcpy(st + seg_bytes + combo_bytes, empty.data(), empty.size() * sizeof(int32_t));
