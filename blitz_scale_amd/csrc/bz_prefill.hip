@@ -46,6 +46,20 @@ __device__ __forceinline__ void lds_direct_load16(const char* uniform_base, uint
                  : "memory", "m0");
 }
 
+// Four such loads into four consecutive KiB of LDS with one M0 value: the instruction offset moves the
+// LDS address and the global address alike, so lane offset i is passed less i KiB.
+__device__ __forceinline__ void lds_direct_load16x4(const char* uniform_base, uint32_t o0, uint32_t o1, uint32_t o2,
+                                                    uint32_t o3, uint32_t lds_addr) {
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\t"
+                 "global_load_lds_dwordx4 %1, %5\n\t"
+                 "global_load_lds_dwordx4 %2, %5 offset:1024\n\t"
+                 "global_load_lds_dwordx4 %3, %5 offset:2048\n\t"
+                 "global_load_lds_dwordx4 %4, %5 offset:3072"
+                 :
+                 : "s"(lds_addr), "v"(o0), "v"(o1), "v"(o2), "v"(o3), "s"(uniform_base)
+                 : "memory", "m0");
+}
+
 struct PrefillItem { // one workgroup's job, in launch order
     int32_t tok0; // global index of the request's first token
     int32_t len;  // tokens in the request (0: padding entry, nothing to do)
@@ -151,19 +165,17 @@ __global__ __launch_bounds__(256, 2) void prefill_kernel(PrefillArgs a, const ch
     for (int i = 0; i < 4; ++i) kcol[i] = (uint32_t)((p16 ^ ((4 * i + r4) & 15)) * 16);
     const uint32_t vcol = (uint32_t)((p16 ^ (r4 << 1)) * 16);
 #pragma unroll
-    for (int i = 0; i < 4; ++i) { // lane offsets of copy i inside the wave's 16 rows when no row needs clamping
-        kfast[i] = (uint32_t)(4 * i + r4) * row_stride + kcol[i];
-        vfast[i] = (uint32_t)(4 * i + r4) * row_stride + vcol;
+    for (int i = 0; i < 4; ++i) { // lane offsets of copy i inside the wave's 16 rows when no row needs clamping,
+                                  // less the i KiB that the instruction offset of the grouped copy adds back
+        kfast[i] = (uint32_t)(4 * i + r4) * row_stride + kcol[i] - (uint32_t)(i * 1024);
+        vfast[i] = (uint32_t)(4 * i + r4) * row_stride + vcol - (uint32_t)(i * 1024);
     }
     auto issue_tile = [&](int t, int buf) __attribute__((always_inline)) {
         const uint32_t m0k = lds0 + (uint32_t)(buf * kTile + 16 * wv * 256);
         if ((t + 1) * kBN <= L) { // the whole tile lies inside the request: one wave-uniform base for K, one for V
             const size_t base = (((size_t)it.tok0 + (size_t)(t * kBN + 16 * wv)) * Hkv + kvh) * 256;
-#pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                lds_direct_load16(k_ptr + base, kfast[i], m0k + i * 1024);
-                lds_direct_load16(v_ptr + base, vfast[i], m0k + 2 * kTile + i * 1024);
-            }
+            lds_direct_load16x4(k_ptr + base, kfast[0], kfast[1], kfast[2], kfast[3], m0k);
+            lds_direct_load16x4(v_ptr + base, vfast[0], vfast[1], vfast[2], vfast[3], m0k + 2 * kTile);
         } else {
             const size_t base = (((size_t)it.tok0 + (size_t)t * kBN) * Hkv + kvh) * 256;
 #pragma unroll
