@@ -40,6 +40,7 @@ struct DecodeArgs {
     const float* v_scale;
     uint64_t stride_page, stride_n, stride_h;
     uint32_t page_size, num_qo_heads, num_kv_heads;
+    uint32_t group_div; // workgroups per kv head: a group that is no instantiated size is split into equal parts
     int rope_mode;
     float sm_scale_log2; // sm_scale * log2(e)
     RopeFreqs freqs;
@@ -53,7 +54,8 @@ __global__ __launch_bounds__(256) void decode_general_kernel(DecodeArgs a) {
     constexpr int UNROLL = 4;
 
     const DecodeSegment seg = a.segments[blockIdx.x];
-    const int kvh = blockIdx.y;
+    const int unit = blockIdx.y;                   // G consecutive q heads, all of one kv head
+    const int kvh = unit / (int)a.group_div;
     const int b = seg.seq;
     const int tid = threadIdx.x;
     const int lane_in_row = tid % LANES; // which 8-element slice of the row
@@ -69,7 +71,7 @@ __global__ __launch_bounds__(256) void decode_general_kernel(DecodeArgs a) {
     float q[G][8];
 #pragma unroll
     for (int g = 0; g < G; ++g) {
-        const size_t qoff = ((size_t)b * a.num_qo_heads + (size_t)kvh * G + g) * D + lane_in_row * 8;
+        const size_t qoff = ((size_t)b * a.num_qo_heads + (size_t)unit * G + g) * D + lane_in_row * 8;
         Vec8<QT> qv;
         qv.load(reinterpret_cast<const QT*>(a.q) + qoff);
         qv.to_float(q[g]);
@@ -208,7 +210,7 @@ __global__ __launch_bounds__(256) void decode_general_kernel(DecodeArgs a) {
         }
         const float o = (ll > 0.f) ? oo / ll * vscale : 0.f;
         const float lse2 = (ll > 0.f) ? mm + log2f(ll) : -INFINITY; // base-2 log-sum-exp of scaled logits
-        const int hq = kvh * G + g;
+        const int hq = unit * G + g;
         if (seg.partial < 0) {
             reinterpret_cast<OT*>(a.out)[((size_t)b * a.num_qo_heads + hq) * D + d] = StoreCvt<OT>::from(o);
             if (a.lse && d == 0) a.lse[(size_t)b * a.num_qo_heads + hq] = lse2 * 0.6931471805599453f;
@@ -330,6 +332,7 @@ extern "C" int bz_batch_decode(bz_decode_plan_t* plan_, const void* q, int q_dty
     a.k_scale = k_scale; a.v_scale = v_scale;
     a.stride_page = kv->stride_page; a.stride_n = kv->stride_n; a.stride_h = kv->stride_h;
     a.page_size = kv->page_size; a.num_qo_heads = num_qo_heads; a.num_kv_heads = kv->num_kv_heads;
+    a.group_div = 1;
     a.rope_mode = rope_mode;
     if (!(sm_scale > 0.f)) sm_scale = 1.0f / sqrtf((float)D);
     a.sm_scale_log2 = sm_scale * 1.4426950408889634f;
@@ -352,14 +355,19 @@ extern "C" int bz_batch_decode(bz_decode_plan_t* plan_, const void* q, int q_dty
             return 0;
         }
         if (rc == BZ_ERR_UNSUPPORTED) {
-            dim3 grid(p->num_segments, kv->num_kv_heads);
+            // groups of 1, 2, 4 or 8 q heads per workgroup; any other group size is split into equal parts of
+            // the largest of these that divides it (each part reads the K/V of its kv head again)
+            int Gk = 8;
+            while (G % Gk) Gk >>= 1;
+            a.group_div = (uint32_t)(G / Gk);
+            dim3 grid(p->num_segments, kv->num_kv_heads * a.group_div);
             if (p->time_start) BZ_CHECK_HIP(hipEventRecord(p->time_start, s));
             if (q_dtype == BZ_F16)
-                rc = (out_dtype == BZ_F32) ? launch_general_kv<f16_t, float>(a, kv->kv_dtype, q_dtype, D, G, grid, s)
-                                           : launch_general_kv<f16_t, f16_t>(a, kv->kv_dtype, q_dtype, D, G, grid, s);
+                rc = (out_dtype == BZ_F32) ? launch_general_kv<f16_t, float>(a, kv->kv_dtype, q_dtype, D, Gk, grid, s)
+                                           : launch_general_kv<f16_t, f16_t>(a, kv->kv_dtype, q_dtype, D, Gk, grid, s);
             else
-                rc = (out_dtype == BZ_F32) ? launch_general_kv<bf16_t, float>(a, kv->kv_dtype, q_dtype, D, G, grid, s)
-                                           : launch_general_kv<bf16_t, bf16_t>(a, kv->kv_dtype, q_dtype, D, G, grid, s);
+                rc = (out_dtype == BZ_F32) ? launch_general_kv<bf16_t, float>(a, kv->kv_dtype, q_dtype, D, Gk, grid, s)
+                                           : launch_general_kv<bf16_t, bf16_t>(a, kv->kv_dtype, q_dtype, D, Gk, grid, s);
             if (rc == 0 && p->time_stop) BZ_CHECK_HIP(hipEventRecord(p->time_stop, s));
         }
         if (rc) return rc;

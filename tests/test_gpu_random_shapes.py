@@ -1,0 +1,107 @@
+"""Seeded random shapes through the C ABI against the CPU checker: batch sizes, ragged context lengths
+(zero and one included), head groupings, page sizes, layouts, types, split thresholds and RoPE modes
+drawn at random, so that combinations nobody thought of writing down get exercised too.  The draws are
+fixed by the seed; tolerances as in the per-kernel tests (max-abs <= 2e-3 for f16/bf16 with the bf16
+storage-step widening, <= 3e-2 with an e4m3 pool, page placement bit-exact)."""
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from blitz_scale_amd import kernel as K
+from blitz_scale_amd import workloads as wl
+from blitz_scale_amd._lib import (BZ_BF16, BZ_E4M3, BZ_F16, BZ_LAYOUT_HND, BZ_LAYOUT_NHD, BZ_ROPE_FULL, BZ_ROPE_NONE,
+                                  BZ_ROPE_Q_ONLY)
+
+from _gpu import DeviceDecode, to_dev, to_host_bits
+from _util import DecodeProblem, ulp_tol
+from test_gpu_prefill import Prefill
+
+pytestmark = pytest.mark.gpu
+
+
+def draw_lens(rng, B, longest):
+    kind = rng.integers(0, 3)
+    if kind == 0:
+        lens = rng.integers(0, longest + 1, B)
+    elif kind == 1:  # mostly short with a few long ones
+        lens = np.where(rng.random(B) < 0.2, rng.integers(longest // 2, longest + 1, B), rng.integers(0, 70, B))
+    else:            # around tile and page boundaries
+        lens = rng.choice([0, 1, 15, 16, 17, 31, 32, 33, 63, 64, 65, 127, 128, 129, 255, 256, 257], B)
+    return [int(x) for x in lens]
+
+
+@pytest.mark.parametrize("case", range(24))
+def test_decode_random_shapes(case):
+    rng = np.random.default_rng(9000 + case)
+    B = int(rng.integers(1, 33))
+    Hkv = int(rng.choice([1, 2, 4, 8]))
+    G = int(rng.choice([1, 2, 3, 4, 6, 7, 8, 12, 16, 32]))
+    D = int(rng.choice([64, 128, 128, 128]))
+    P = int(rng.choice([8, 16, 16, 32, 64]))
+    dtype = int(rng.choice([BZ_F16, BZ_BF16]))
+    kv_dtype = BZ_E4M3 if rng.random() < 0.25 else dtype
+    layout = int(rng.choice([BZ_LAYOUT_HND, BZ_LAYOUT_NHD]))
+    rope_mode = int(rng.choice([BZ_ROPE_NONE, BZ_ROPE_NONE, BZ_ROPE_Q_ONLY, BZ_ROPE_FULL]))
+    if kv_dtype == BZ_E4M3 and rope_mode == BZ_ROPE_FULL:
+        rope_mode = BZ_ROPE_Q_ONLY  # rotating quantised K on the fly is not a mode of the library
+    split_tokens = int(rng.choice([0, 64, 256, 2048, 0xFFFFFFFF]))
+    ctx = draw_lens(rng, B, 2500)
+    if not any(ctx):
+        ctx[0] = 40
+    p = DecodeProblem(9100 + case, ctx, Hkv * G, Hkv, D, P, dtype, kv_dtype=kv_dtype, layout=layout)
+    theta = float(rng.choice([1e4, 5e5]))
+    ref = oracle.batch_decode(p.q, dtype, p.oracle_kv(), p.Hq, rope_mode=rope_mode, rope_theta=theta,
+                              k_scale=p.k_scale, v_scale=p.v_scale, parallel=True)
+    dev = DeviceDecode(p)
+    dev.plan(split_tokens)
+    got = dev.decode(None, rope_mode, theta)
+    base = 3e-2 if kv_dtype == BZ_E4M3 else 2e-3
+    live = p.ctx > 0
+    err = np.abs(got - ref)
+    assert (err[live] <= ulp_tol(ref, dtype, base)[live]).all(), (case, float(err[live].max()))
+    assert not got[~live].any()
+
+
+@pytest.mark.parametrize("case", range(8))
+def test_prefill_random_shapes(case):
+    rng = np.random.default_rng(9500 + case)
+    B = int(rng.integers(1, 7))
+    Hkv = int(rng.choice([1, 2, 4]))
+    G = int(rng.choice([1, 2, 4]))
+    dtype = int(rng.choice([BZ_F16, BZ_BF16]))
+    causal = bool(rng.random() < 0.75)
+    lens = [max(1, x) for x in draw_lens(rng, B, 700)]
+    pf = Prefill(9600 + case, lens, Hkv * G, Hkv, 128, dtype)
+    rope_mode = BZ_ROPE_FULL if rng.random() < 0.3 else BZ_ROPE_NONE
+    got = pf.run(causal=causal, rope_mode=rope_mode, theta=1e4)
+    ref = oracle.batch_prefill_ragged(pf.q, pf.k, pf.v, dtype, pf.indptr, Hkv * G, Hkv, 128, causal=causal,
+                                      rope=rope_mode == BZ_ROPE_FULL, rope_theta=1e4, parallel=True)
+    assert not np.isnan(got).any()
+    assert (np.abs(got - ref) <= ulp_tol(ref, dtype)).all(), (case, float(np.abs(got - ref).max()))
+
+
+@pytest.mark.parametrize("case", range(6))
+def test_store_and_append_random_shapes(case):
+    """Prefill store followed by a decode append into the same table: page placement bit-exact."""
+    rng = np.random.default_rng(9800 + case)
+    B = int(rng.integers(1, 9))
+    Hkv = int(rng.choice([1, 2, 8]))
+    D = int(rng.choice([64, 128]))
+    P = int(rng.choice([8, 16, 64]))
+    dtype = int(rng.choice([BZ_F16, BZ_BF16]))
+    layout = int(rng.choice([BZ_LAYOUT_HND, BZ_LAYOUT_NHD]))
+    lens = [max(1, x) for x in draw_lens(rng, B, 300)]
+    p = DecodeProblem(9900 + case, [l + 1 for l in lens], Hkv, Hkv, D, P, dtype, layout=layout)  # len+1 slots reserved
+    indptr = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+    N = int(indptr[-1])
+    k, v = wl.randn_bits(rng, (N, Hkv, D), dtype), wl.randn_bits(rng, (N, Hkv, D), dtype)
+    kn, vn = wl.randn_bits(rng, (B, Hkv, D), dtype), wl.randn_bits(rng, (B, Hkv, D), dtype)
+    want = p.pool.copy()
+    oracle.store_prefill_kv(p.oracle_kv(want), k, v, dtype, indptr)
+    oracle.append_decode_kv(p.oracle_kv(want), kn, vn, dtype)
+    dev = DeviceDecode(p)
+    K.store_prefill_kv_cache(dev.pt, to_dev(k, dtype), to_dev(v, dtype), torch.from_numpy(indptr).cuda(), num_tokens=N)
+    K.append_decode_kv_cache(dev.pt, to_dev(kn, dtype), to_dev(vn, dtype))
+    torch.cuda.synchronize()
+    assert np.array_equal(to_host_bits(dev.pool), want), case
