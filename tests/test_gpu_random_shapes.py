@@ -68,7 +68,7 @@ def test_prefill_random_shapes(case):
     rng = np.random.default_rng(9500 + case)
     B = int(rng.integers(1, 7))
     Hkv = int(rng.choice([1, 2, 4]))
-    G = int(rng.choice([1, 2, 4]))
+    G = int(rng.choice([1, 2, 3, 4, 7, 8]))
     dtype = int(rng.choice([BZ_F16, BZ_BF16]))
     causal = bool(rng.random() < 0.75)
     lens = [max(1, x) for x in draw_lens(rng, B, 700)]
@@ -105,3 +105,74 @@ def test_store_and_append_random_shapes(case):
     K.append_decode_kv_cache(dev.pt, to_dev(kn, dtype), to_dev(vn, dtype))
     torch.cuda.synchronize()
     assert np.array_equal(to_host_bits(dev.pool), want), case
+
+
+@pytest.mark.parametrize("case", range(8))
+def test_elementwise_random_shapes(case):
+    """RMSNorm, add+RMSNorm, SiLU-gate and residual add at odd row counts and widths (multiples of 8)."""
+    rng = np.random.default_rng(9950 + case)
+    N = int(rng.integers(1, 90))
+    h = 8 * int(rng.integers(1, 1400))
+    I = 8 * int(rng.integers(1, 2000))
+    dtype = int(rng.choice([BZ_F16, BZ_BF16]))
+    x, r = wl.randn_bits(rng, (N, h), dtype), wl.randn_bits(rng, (N, h), dtype)
+    w = wl.randn_bits(rng, (h,), dtype, mean=1.0, std=0.02)
+    gu = wl.randn_bits(rng, (N, 2 * I), dtype)
+
+    def close(got_bits, ref):
+        got = wl.to_f32(got_bits, dtype)
+        assert (np.abs(got - ref) <= ulp_tol(ref, dtype)).all(), (case, float(np.abs(got - ref).max()))
+
+    xd, rd, wd = to_dev(x, dtype), to_dev(r, dtype), to_dev(w, dtype)
+    out = torch.empty_like(xd)
+    K.rms_norm(xd, wd, out, N, h)
+    torch.cuda.synchronize()
+    close(to_host_bits(out), oracle.rms_norm(x, w, dtype, 1e-5))
+    ref, ref_res = oracle.add_rms_norm(x, r, w, dtype)
+    K.add_rms_norm(xd, rd, wd, N, h)
+    torch.cuda.synchronize()
+    assert np.array_equal(to_host_bits(rd), ref_res)
+    close(to_host_bits(xd), ref)
+    act = torch.empty((N, I), dtype=xd.dtype, device="cuda")
+    K.silu_and_mul(to_dev(gu, dtype), act, N, I)
+    torch.cuda.synchronize()
+    close(to_host_bits(act), oracle.silu_and_mul(gu, dtype))
+    a2, b2 = to_dev(x, dtype), to_dev(r, dtype)
+    K.add_residual(a2, b2, N, h)
+    torch.cuda.synchronize()
+    assert np.array_equal(to_host_bits(b2), oracle.add_residual(x, r, dtype))
+
+
+@pytest.mark.parametrize("case", range(6))
+def test_wire_random_shapes(case):
+    """Migration payload at random geometry: byte-exact pack, and unpack into other pages."""
+    rng = np.random.default_rng(9980 + case)
+    layers, max_pages = int(rng.integers(1, 6)), int(rng.integers(3, 40))
+    Hkv, P, D = int(rng.choice([1, 2, 5, 8])), int(rng.choice([4, 16, 64])), int(rng.choice([64, 128]))
+    dtype = int(rng.choice([BZ_F16, BZ_BF16, BZ_E4M3]))
+    layout = int(rng.choice([BZ_LAYOUT_HND, BZ_LAYOUT_NHD]))
+    sp = 2 * Hkv * P * D
+    if dtype == BZ_E4M3:
+        bits = rng.integers(0, 256, size=layers * max_pages * sp, dtype=np.uint8)
+    else:
+        bits = wl.randn_bits(rng, (layers * max_pages * sp,), dtype)
+    n = int(rng.integers(1, max_pages + 1))
+    ids = rng.permutation(max_pages)[:n].astype(np.int32)
+    start = int(rng.integers(0, layers))
+    cnt = int(rng.integers(1, layers - start + 1))
+    pool = to_dev(bits, dtype)
+    pt = K.PageTable(1, P, Hkv, D, pool, layout=layout)
+    want = oracle.kv_pages_pack(bits, dtype, max_pages, sp, ids, start, cnt)
+    wire = torch.zeros(want.nbytes, dtype=torch.uint8, device="cuda")
+    ids_d = torch.from_numpy(ids).cuda()
+    K.pack_kv_pages(pt, max_pages, ids_d, start, cnt, wire)
+    torch.cuda.synchronize()
+    assert np.array_equal(wire.cpu().numpy(), want.view(np.uint8)), case
+    dst_bits = np.zeros_like(bits)
+    dst = to_dev(dst_bits, dtype)
+    dpt = K.PageTable(1, P, Hkv, D, dst, layout=layout)
+    dst_ids = rng.permutation(max_pages)[:n].astype(np.int32)
+    K.unpack_kv_pages(dpt, max_pages, torch.from_numpy(dst_ids).cuda(), start, cnt, wire)
+    torch.cuda.synchronize()
+    oracle.kv_pages_unpack(dst_bits, dtype, max_pages, sp, dst_ids, start, cnt, want)
+    assert np.array_equal(to_host_bits(dst), dst_bits), case
