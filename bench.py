@@ -549,6 +549,52 @@ def bench_layers(args):
     torch.cuda.synchronize()
     same = bool(torch.equal(out.view(torch.int16), want.view(torch.int16)))
     graph_ms, _ = timed(lambda i, e: graph.replay(), steps, warmup, torch_events=False)
+
+    # The same replay with the reference's per-step host work in front of it (page-table upload and
+    # plan(), src/model/llama.h:363-375, src/blitz/stub.h:1288-1313) ...
+    def host_then_replay(i, e):
+        pts[0].upload()
+        handler.plan(float_ws, float_ws.numel(), int_ws, int_ws.numel(), indptr, lpl, B, Hq, Hkv, D, P,
+                     split_tokens=args.split_tokens)
+        graph.replay()
+    host_ms, _ = timed(host_then_replay, steps, warmup, torch_events=False)
+    t0 = time.perf_counter()
+    for _ in range(200):
+        handler.plan(float_ws, float_ws.numel(), int_ws, int_ws.numel(), indptr, lpl, B, Hq, Hkv, D, P,
+                     split_tokens=args.split_tokens)
+    plan_us = (time.perf_counter() - t0) / 200 * 1e6
+    torch.cuda.synchronize()
+    # ... and with the table taken as running `horizon` steps ahead of the present (same table and plan:
+    # the measured lengths are the state at the end of the horizon): one upload and one plan serve
+    # `horizon` steps, a device counter says how far the present lags, and the replayed graph ends by
+    # counting it down.  Nothing but graph.replay() happens on the host inside the horizon.
+    horizon = 32
+    ahead = torch.tensor([horizon - 1], dtype=torch.int32, device="cuda")
+    for pt in pts:
+        pt.steps_ahead_d = ahead
+
+    def step_ahead(stream=None):
+        step_layers(stream)
+        K.steps_ahead_advance(ahead, stream=stream)
+
+    torch.cuda.synchronize()
+    graph2 = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph2, stream=side):
+        step_ahead(torch.cuda.current_stream().cuda_stream)
+    torch.cuda.synchronize()
+
+    def replay_ahead(i, e):
+        if i % horizon == 0:  # the host's turn, once per horizon: grow the table, upload, plan, reset the counter
+            pts[0].upload()
+            for pt in pts:
+                pt.indices_d, pt.indptr_d, pt.last_page_len_d = (pts[0].indices_d, pts[0].indptr_d,
+                                                                 pts[0].last_page_len_d)
+            handler.plan(float_ws, float_ws.numel(), int_ws, int_ws.numel(), indptr, lpl, B, Hq, Hkv, D, P,
+                         split_tokens=args.split_tokens)
+            ahead.fill_(horizon - 1)
+        graph2.replay()
+    ahead_ms, _ = timed(replay_ahead, max(steps, 2 * horizon), warmup, torch_events=False)
+    ahead_only_ms, _ = timed(lambda i, e: graph2.replay(), steps, warmup, torch_events=False)
     kv_bytes = layers * B * ctx * 2 * Hkv * D * 2
     return {"metric": "small_batch_decode_32_layers_us", "value": round(graph_ms * 1e3, 2), "unit": "us/step",
             "n_gpus": 1, "steps": steps, "warmup": warmup, "ms_per_step": round(graph_ms, 6),
@@ -558,6 +604,10 @@ def bench_layers(args):
             "eager_us_per_step": round(eager_ms * 1e3, 2), "graph_us_per_step": round(graph_ms * 1e3, 2),
             "us_per_layer": {"eager": round(eager_ms * 1e3 / layers, 2), "graph": round(graph_ms * 1e3 / layers, 2)},
             "graph_replay_bit_exact_vs_eager": same,
+            "with_host_work_us_per_step": {"upload_and_plan_every_step": round(host_ms * 1e3, 2),
+                                           f"table_{horizon}_steps_ahead": round(ahead_ms * 1e3, 2),
+                                           "replay_alone_with_counter": round(ahead_only_ms * 1e3, 2),
+                                           "plan_call_host_us": round(plan_us, 2)},
             "roofline": {"bound": "hbm", "achieved": round(kv_bytes / (graph_ms * 1e-3) / 1e9, 1), "peak": 8000.0,
                          "unit": "GB/s", "frac": round(kv_bytes / (graph_ms * 1e-3) / 1e9 / 8000.0, 4), "traffic": None,
                          "kernel": "whole replayed step (launch-latency bound at this size, not a kernel figure)"}}

@@ -34,6 +34,7 @@ class BzPagedKV(C.Structure):
         ("stride_h", C.c_uint64),
         ("kv_dtype", C.c_int32),
         ("reserved", C.c_int32),
+        ("steps_ahead", C.c_void_p),
     ]
 
 
@@ -59,6 +60,7 @@ SIGNATURES = {
                                        _f32, _f32, _vp]),
     "bz_store_prefill_kv": (_i32, [_kvp, _vp, _vp, _i32, _vp, _u32, _vp, _u32, _i32, _f32, _vp, _vp, _vp]),
     "bz_append_decode_kv": (_i32, [_kvp, _vp, _vp, _i32, _vp, _u32, _i32, _f32, _vp, _vp, _vp]),
+    "bz_steps_ahead_advance": (_i32, [_vp, _vp]),
     "bz_rms_norm": (_i32, [_vp, _vp, _vp, _i32, _u32, _u32, _f32, _vp]),
     "bz_add_rms_norm": (_i32, [_vp, _vp, _vp, _i32, _u32, _u32, _f32, _vp]),
     "bz_silu_and_mul": (_i32, [_vp, _vp, _i32, _u32, _u32, _vp]),

@@ -42,6 +42,9 @@ struct PageTable {
     IdType* indices_d = nullptr;
     IdType* indptr_d = nullptr;
     IdType* last_page_len_d = nullptr;
+    // optional device counter: the table describes the batch this many decode steps ahead of the present
+    // (pages of the tokens to come already listed); nullptr = the table is the present
+    IdType* steps_ahead_d = nullptr;
 
     PageTable(uint32_t batch_size_, uint32_t page_size_, uint32_t num_heads_, uint32_t head_size_, DType* base_ptr,
               int layout_ = BZ_LAYOUT_HND) :
@@ -66,6 +69,7 @@ struct PageTable {
         kv.batch_size = batch_size; kv.page_size = page_size; kv.num_kv_heads = num_heads; kv.head_dim = head_size;
         kv.stride_page = stride_page; kv.stride_n = stride_n; kv.stride_h = stride_h;
         kv.kv_dtype = bz_dtype<DType>::value; kv.reserved = 0;
+        kv.steps_ahead = reinterpret_cast<const int32_t*>(steps_ahead_d);
         return kv;
     }
 };

@@ -33,6 +33,7 @@ struct DecodeArgs {
     const int32_t* indices;
     const int32_t* indptr;
     const int32_t* last_page_len;
+    const int32_t* steps_ahead; // optional: the table is this many decode steps ahead of the present
     const DecodeSegment* segments;
     float* part_o;   // [num_partials][Hq][D]
     float* part_lse; // [num_partials][Hq]
@@ -61,9 +62,10 @@ __global__ __launch_bounds__(256) void decode_general_kernel(DecodeArgs a) {
     const int lane_in_row = tid % LANES; // which 8-element slice of the row
     const int slot = tid / LANES;        // token slot 0..TOK-1
 
+    const int ahead = a.steps_ahead ? *a.steps_ahead : 0;
     const int ip0 = a.indptr[b];
     const int npages = a.indptr[b + 1] - ip0;
-    const int seq_len = (npages - 1) * (int)a.page_size + a.last_page_len[b];
+    const int seq_len = max((npages - 1) * (int)a.page_size + a.last_page_len[b] - max(ahead, 0), 0);
     const int tok_begin = seg.page_begin * (int)a.page_size;
     const int tok_end = min(seg.page_end * (int)a.page_size, seq_len);
 
@@ -327,6 +329,7 @@ extern "C" int bz_batch_decode(bz_decode_plan_t* plan_, const void* q, int q_dty
     a.q = q; a.out = out; a.lse = lse;
     a.k_data = (const char*)kv->k_data; a.v_data = (const char*)kv->v_data;
     a.indices = kv->indices; a.indptr = kv->indptr; a.last_page_len = kv->last_page_len;
+    a.steps_ahead = kv->steps_ahead;
     a.segments = p->segments_d;
     a.part_o = p->part_o; a.part_lse = p->part_lse;
     a.k_scale = k_scale; a.v_scale = v_scale;

@@ -35,6 +35,7 @@ struct MfmaDecodeArgs {
     const int32_t* indices;
     const int32_t* indptr;
     const int32_t* last_page_len;
+    const int32_t* steps_ahead; // optional: the table (and the plan made from it) is this many steps ahead
     const MfmaPiece* pieces;
     const MfmaTile* tiles;
     const int32_t* tile_ptr;
@@ -147,8 +148,14 @@ __global__ __launch_bounds__(64, 2) void decode_mfma_kernel(MfmaDecodeArgs a, co
     auto d_of = [&](int ks) { return KV8 ? 64 * (ks >> 1) + 16 * j + 8 * (ks & 1) : 32 * ks + 8 * j; };
     const int G = (int)a.group;
 
+    // A plan made from a table that runs ahead lists tiles up to the future lengths; at present every
+    // sequence is `ahead` tokens shorter.  Tiles past the present end are masked as a whole (their pages
+    // exist), so a piece can come out empty: zero weight in the split-K combine.  (Read together with
+    // the slot boundaries: one round trip, not two.)
+    const int ahead_raw = a.steps_ahead ? *a.steps_ahead : 0;
     const int g_begin = tile_ptr[blockIdx.x], g_end = tile_ptr[blockIdx.x + 1];
     if (g_begin >= g_end) return;
+    const int ahead = max(ahead_raw, 0);
 
     // ---- descriptions of 32 tiles at a time: lane l < 32 fetches the record of tile base+l, the two
     // page ids it points at and the piece it belongs to, and leaves 12 ints in LDS:
@@ -169,8 +176,8 @@ __global__ __launch_bounds__(64, 2) void decode_mfma_kernel(MfmaDecodeArgs a, co
         d.v[4] = m0.y;                                             // kvh
         d.v[5] = (rec.t == m0.z ? 1 : 0) | (rec.t + 1 == m0.w ? 2 : 0);
         d.v[6] = m1.x;                                             // partial slot or -1
-        d.v[7] = min(m0.w * kTileTok, m2.z);                       // tok_end of the piece
-        d.v[8] = m2.z;                                             // seq_len
+        d.v[8] = max(m2.z - ahead, 0);                             // seq_len at present
+        d.v[7] = min(m0.w * kTileTok, d.v[8]);                     // tok_end of the piece
         return d;
     };
     auto stash_info = [&](const Desc& d, int buf) {
@@ -379,7 +386,9 @@ __global__ __launch_bounds__(64, 2) void decode_mfma_kernel(MfmaDecodeArgs a, co
                 tmax = fmaxf(tmax, v);
             }
         tmax = lane_max_xor32(lane_max_xor16(tmax));
-        const float m_new = fmaxf(m_run, tmax);   // finite: every tile holds at least one live token
+        // finite also for a tile without live tokens (one past the present end under a table that runs
+        // ahead): its probabilities and alpha come out 0 instead of NaN
+        const float m_new = fmaxf(fmaxf(m_run, tmax), -1e30f);
         const float alpha = exp2f(m_run - m_new); // 0 on the first tile (m_run = -inf)
         // The probabilities enter the second contraction as a storage-precision head plus tail
         // (p = hi + lo, two MFMAs per block): the matrix cores cost nothing here and the result
@@ -543,6 +552,7 @@ int decode_fast_path(const DecodePlan* p, const void* q, void* out, float* lse, 
     a.q = q; a.out = out; a.lse = lse;
     a.k_data = (const char*)kv->k_data; a.v_data = (const char*)kv->v_data;
     a.indices = kv->indices; a.indptr = kv->indptr; a.last_page_len = kv->last_page_len;
+    a.steps_ahead = kv->steps_ahead;
     a.pieces = p->mfma_pieces_d; a.tiles = p->mfma_tiles_d; a.tile_ptr = p->mfma_tile_ptr_d;
     a.part_o = p->mfma_part_o; a.part_lse = p->mfma_part_lse;
     a.stride_page = kv->stride_page; a.stride_n = kv->stride_n; a.stride_h = kv->stride_h;

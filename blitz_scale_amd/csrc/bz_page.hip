@@ -15,6 +15,7 @@ struct PageWriteArgs {
     const int32_t* indices;
     const int32_t* indptr;
     const int32_t* last_page_len;
+    const int32_t* steps_ahead; // optional: the table is this many decode steps ahead of the present
     const void* k_src;
     const void* v_src;
     void* q_inout;
@@ -56,9 +57,11 @@ __global__ __launch_bounds__(256) void page_write_kernel(PageWriteArgs a) {
         if (n >= a.ragged_indptr[a.batch_size]) return;
     } else {
         b = blockIdx.x;
+        const int ahead = a.steps_ahead ? *a.steps_ahead : 0; // fetched together with the table entries
         const int np = a.indptr[b + 1] - a.indptr[b];
         if (np <= 0) return;
-        pos = (np - 1) * (int)a.page_size + a.last_page_len[b] - 1;
+        pos = (np - 1) * (int)a.page_size + a.last_page_len[b] - 1 - max(ahead, 0);
+        if (pos < 0) return; // the sequence has no token yet at the present step
         src_tok = (size_t)b;
     }
     const int64_t page = a.indices[a.indptr[b] + pos / (int)a.page_size];
@@ -184,6 +187,7 @@ static int fill_args(PageWriteArgs& a, const bz_paged_kv_t* kv, const void* k, c
     if (kv->stride_n % 8 || kv->stride_h % 8 || kv->stride_page % 8) return BZ_ERR_BAD_ARG;
     a.k_data = (char*)kv->k_data; a.v_data = (char*)kv->v_data;
     a.indices = kv->indices; a.indptr = kv->indptr; a.last_page_len = kv->last_page_len;
+    a.steps_ahead = kv->steps_ahead;
     a.k_src = k; a.v_src = v; a.q_inout = q_inout; a.ragged_indptr = nullptr;
     a.k_scale = k_scale; a.v_scale = v_scale;
     a.stride_page = kv->stride_page; a.stride_n = kv->stride_n; a.stride_h = kv->stride_h;
@@ -194,9 +198,21 @@ static int fill_args(PageWriteArgs& a, const bz_paged_kv_t* kv, const void* k, c
     return 0;
 }
 
+__global__ void steps_ahead_advance_kernel(int32_t* steps_ahead) {
+    const int32_t v = *steps_ahead;
+    if (v > 0) *steps_ahead = v - 1;
+}
+
 } // namespace bz
 
 using namespace bz;
+
+extern "C" int bz_steps_ahead_advance(int32_t* steps_ahead, void* stream) {
+    if (!steps_ahead) return BZ_ERR_BAD_ARG;
+    hipLaunchKernelGGL(steps_ahead_advance_kernel, dim3(1), dim3(1), 0, (hipStream_t)stream, steps_ahead);
+    BZ_LAUNCH_CHECK();
+    return 0;
+}
 
 extern "C" int bz_store_prefill_kv(const bz_paged_kv_t* kv, void* k, const void* v, int src_dtype,
                                    const int32_t* ragged_indptr, uint32_t num_tokens, void* q_inout,

@@ -67,6 +67,7 @@ class PageTable:
         self.k_data = base.data_ptr()
         self.v_data = self.k_data + (self.stride_page // 2) * self.elem_bytes
         self.indices_d = self.indptr_d = self.last_page_len_d = None
+        self.steps_ahead_d = None  # optional device int32: the table is this many decode steps ahead of the present
 
     def set_layer(self, layer, max_num_pages):
         """The per-layer pointer bump of src/model/llama.h:378-381, as an absolute view."""
@@ -76,7 +77,12 @@ class PageTable:
     def upload(self, device="cuda"):
         """One blob [indices | indptr | last_page_len] like Stub::forward (src/blitz/stub.h:1288-1313)."""
         blob = np.concatenate([_host_i32(self.indices), _host_i32(self.indptr), _host_i32(self.last_page_len)])
-        self._blob_d = torch.from_numpy(blob).to(device)
+        host = torch.from_numpy(blob)
+        prev = getattr(self, "_blob_d", None)
+        if prev is not None and prev.numel() == host.numel() and prev.device.type == torch.device(device).type:
+            prev.copy_(host)  # same device buffer: addresses recorded into a HIP graph stay valid
+        else:
+            self._blob_d = host.to(device)
         n0, n1 = len(self.indices), len(self.indptr)
         self.indices_d = self._blob_d[:n0]
         self.indptr_d = self._blob_d[n0:n0 + n1]
@@ -98,6 +104,7 @@ class PageTable:
         s.num_kv_heads, s.head_dim = self.num_heads, self.head_size
         s.stride_page, s.stride_n, s.stride_h = self.stride_page, self.stride_n, self.stride_h
         s.kv_dtype = self.kv_dtype
+        s.steps_ahead = self.steps_ahead_d.data_ptr() if self.steps_ahead_d is not None else None
         return s
 
 
@@ -211,6 +218,11 @@ def append_decode_kv_cache(page_table, k_data, v_data, *, q=None, num_qo_heads=0
                                          num_qo_heads, int(rope), rope_theta, _ptr(k_scale), _ptr(v_scale),
                                          _stream(stream))
     check(rc, "AppendPagedKVCacheDecode")
+
+
+def steps_ahead_advance(steps_ahead, *, stream=None):
+    """End of a decode step under a page table that runs ahead of the present: counter -= 1, not below 0."""
+    check(_lib.load().bz_steps_ahead_advance(_ptr(steps_ahead), _stream(stream)), "stepsAheadAdvance")
 
 
 def rms_norm(input, weight, output, num_tokens, hidden_size, eps=1e-5, *, stream=None):

@@ -52,6 +52,17 @@ extern "C" {
  * image of blitz::kernel::PageTable (src/kernel/page.h:12-64).  Element address relative
  * to k_data / v_data:  page*stride_page + slot*stride_n + head*stride_h + d   (elements).
  * seq_len_b = (indptr[b+1]-indptr[b]-1)*page_size + last_page_len[b]   (page.cu:38-40).
+ *
+ * steps_ahead (optional, no counterpart in the reference): a device int32.  When non-NULL the table
+ * describes the batch steps_ahead[0] decode steps in the FUTURE: every sequence is at present that many
+ * tokens shorter than indptr / last_page_len say, and the pages of the tokens to come are already in
+ * `indices`.  bz_append_decode_kv and bz_batch_decode then work at the present length
+ * (seq_len_b - steps_ahead[0]; a sequence this leaves without tokens is skipped / yields a zero row).
+ * A host that grows the table H steps ahead uploads it and plans ONCE, sets the counter to H-1, and runs
+ * H decode steps (bz_steps_ahead_advance after each) without touching table, plan or counter from the
+ * host again: the per-step plan() and table upload of src/model/llama.h:363-375 and
+ * src/blitz/stub.h:1288-1313 leave the step, and a whole step can be replayed from one HIP graph.
+ * The prefill store ignores it.
  */
 typedef struct bz_paged_kv {
     void* k_data;
@@ -68,6 +79,7 @@ typedef struct bz_paged_kv {
     uint64_t stride_h;
     int32_t kv_dtype;             /* BZ_F16 | BZ_BF16 | BZ_E4M3 */
     int32_t reserved;
+    const int32_t* steps_ahead;   /* optional device scalar, see above; NULL = the table is the present */
 } bz_paged_kv_t;
 
 /* Fill the stride fields for a layout (stride_page = 2*H*P*D for both; page.h:59-61). */
@@ -167,6 +179,10 @@ int bz_store_prefill_kv(const bz_paged_kv_t* kv, void* k, const void* v, int src
 int bz_append_decode_kv(const bz_paged_kv_t* kv, const void* k, const void* v, int src_dtype, void* q_inout,
                         uint32_t num_qo_heads, int rope, float rope_theta, const float* k_scale,
                         const float* v_scale, void* stream);
+
+/* End of a decode step under a table that runs ahead (bz_paged_kv_t.steps_ahead): the counter goes down
+ * by one, not below zero.  One tiny launch on `stream`, recordable into a HIP graph. */
+int bz_steps_ahead_advance(int32_t* steps_ahead, void* stream);
 
 /* ---------------------------------------------------------------------------------------
  * element-wise kernels of src/layer's call sites
