@@ -471,7 +471,9 @@ __global__ __launch_bounds__(64, 2) void decode_mfma_kernel(MfmaDecodeArgs a, co
 // Combine the partials of one split (sequence, kv head): o = sum_i o_i 2^(lse_i - M) / sum_i 2^(lse_i - M).
 // One workgroup of 128 lanes per (split, q head of the group).  The partials are fetched eight at a
 // time with all loads issued before any is used, and merged with a running maximum, so a split with up
-// to eight partials costs two dependent memory round trips (schedule entry, then data).
+// to eight partials costs two dependent memory round trips (schedule entry, then data).  (Batches of 32
+// for the 32-piece splits of small batches were measured: 0.3 us less per launch there, 1.4 us more on
+// the large-batch workload, where most splits have two to four partials.)
 template <typename OT>
 __global__ __launch_bounds__(128) void decode_mfma_combine_kernel(const MfmaCombine* __restrict__ combos,
                                                                   const float* __restrict__ part_o,

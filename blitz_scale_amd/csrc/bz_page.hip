@@ -161,12 +161,131 @@ __global__ __launch_bounds__(256) void page_write_kernel(PageWriteArgs a) {
     }
 }
 
+// Decode append: one workgroup per sequence, one new row per (q | k | v) head.  At decode batch sizes the
+// kernel is nothing but its chain of dependent memory round trips, so everything that does not depend
+// on the page table (the counter, the table entries themselves, the caller's q / k / v rows) is
+// requested up front; the page id is the one dependent fetch and overlaps with the angles.
+template <typename ST, typename PT, int D>
+__global__ __launch_bounds__(256) void append_kernel(PageWriteArgs a) {
+    constexpr int LANES = D / 16;
+    constexpr int ROWS = 256 / LANES;
+    constexpr int MAXR = 4; // rows per lane group held in registers; more rows take the loop at the end
+    __shared__ float s_cos[D / 2], s_sin[D / 2];
+
+    const int b = blockIdx.x;
+    const int ahead = a.steps_ahead ? *a.steps_ahead : 0;
+    const int ip0 = a.indptr[b], ip1 = a.indptr[b + 1];
+    const int lpl = a.last_page_len[b];
+    const int lane = threadIdx.x % LANES, r0 = threadIdx.x / LANES;
+    const int Hq = (a.rope && a.q_inout) ? (int)a.num_qo_heads : 0;
+    const int Hkv = (int)a.num_kv_heads;
+    const int total_rows = Hq + 2 * Hkv;
+    auto row_src = [&](int r) -> const ST* { // rows 0..Hq-1: q heads, then the k heads, then the v heads
+        if (r < Hq) return reinterpret_cast<const ST*>(a.q_inout) + ((size_t)b * a.num_qo_heads + r) * D;
+        const bool is_k = r < Hq + Hkv;
+        return reinterpret_cast<const ST*>(is_k ? a.k_src : a.v_src) + ((size_t)b * Hkv + (is_k ? r - Hq : r - Hq - Hkv)) * D;
+    };
+    Vec8<ST> lo[MAXR], hi[MAXR];
+#pragma unroll
+    for (int i = 0; i < MAXR; ++i) {
+        const int r = r0 + i * ROWS;
+        if (r < total_rows) {
+            const ST* src = row_src(r);
+            lo[i].load(src + lane * 8);
+            hi[i].load(src + D / 2 + lane * 8);
+        }
+    }
+    const int np = ip1 - ip0;
+    if (np <= 0) return;
+    const int pos = (np - 1) * (int)a.page_size + lpl - 1 - max(ahead, 0);
+    if (pos < 0) return; // the sequence has no token yet at the present step
+    const int64_t page = a.indices[ip0 + pos / (int)a.page_size];
+    const int slot = pos % (int)a.page_size;
+    if (a.rope) {
+        for (int i = threadIdx.x; i < D / 2; i += 256) {
+            float s, c;
+            sincosf((float)pos * a.freqs.f[i], &s, &c);
+            s_cos[i] = c;
+            s_sin[i] = s;
+        }
+        __syncthreads();
+    }
+    auto finish_row = [&](int r, Vec8<ST>& l, Vec8<ST>& h) {
+        const bool is_q = r < Hq, is_k = !is_q && r < Hq + Hkv;
+        const bool rotate = (is_q || is_k) && a.rope;
+        float x[8], y[8];
+        if (is_q || rotate || (is_k ? a.k_scale : a.v_scale) || sizeof(ST) != sizeof(PT)) {
+            l.to_float(x);
+            h.to_float(y);
+        }
+        if (rotate) {
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                const float c = s_cos[lane * 8 + e], sn = s_sin[lane * 8 + e];
+                float xr, yr;
+                rope_pair(x[e], y[e], c, sn, xr, yr);
+                x[e] = xr;
+                y[e] = yr;
+            }
+        }
+        if (is_q) { // rotated in place
+            ST* row = const_cast<ST*>(row_src(r));
+            l.from_float(x);
+            h.from_float(y);
+            l.store(row + lane * 8);
+            h.store(row + D / 2 + lane * 8);
+            return;
+        }
+        const int hd = is_k ? r - Hq : r - Hq - Hkv;
+        PT* dst = reinterpret_cast<PT*>(is_k ? a.k_data : a.v_data) +
+                  ((size_t)page * a.stride_page + (size_t)slot * a.stride_n + (size_t)hd * a.stride_h);
+        const float* scale = is_k ? a.k_scale : a.v_scale;
+        Vec8<PT> l2, h2;
+        if constexpr (sizeof(ST) == sizeof(PT)) {
+            if (!rotate && !scale) { // bit-exact copy
+                l2.raw = l.raw;
+                h2.raw = h.raw;
+                l2.store(dst + lane * 8);
+                h2.store(dst + D / 2 + lane * 8);
+                return;
+            }
+        }
+        if (scale) {
+            const float sc = scale[hd];
+#pragma unroll
+            for (int e = 0; e < 8; ++e) { x[e] = x[e] / sc; y[e] = y[e] / sc; }
+        }
+        l2.from_float(x);
+        h2.from_float(y);
+        l2.store(dst + lane * 8);
+        h2.store(dst + D / 2 + lane * 8);
+    };
+#pragma unroll
+    for (int i = 0; i < MAXR; ++i) {
+        const int r = r0 + i * ROWS;
+        if (r < total_rows) finish_row(r, lo[i], hi[i]);
+    }
+    for (int r = r0 + MAXR * ROWS; r < total_rows; r += ROWS) {
+        Vec8<ST> l, h;
+        const ST* src = row_src(r);
+        l.load(src + lane * 8);
+        h.load(src + D / 2 + lane * 8);
+        finish_row(r, l, h);
+    }
+}
+
 template <typename ST, typename PT, bool PREFILL>
 static int launch_page_write_d(const PageWriteArgs& a, int D, uint32_t grid, hipStream_t s) {
     if (grid == 0) return 0;
-    if (D == 128) hipLaunchKernelGGL((page_write_kernel<ST, PT, 128, PREFILL>), dim3(grid), dim3(256), 0, s, a);
-    else if (D == 64) hipLaunchKernelGGL((page_write_kernel<ST, PT, 64, PREFILL>), dim3(grid), dim3(256), 0, s, a);
-    else return BZ_ERR_UNSUPPORTED;
+    if constexpr (PREFILL) {
+        if (D == 128) hipLaunchKernelGGL((page_write_kernel<ST, PT, 128, true>), dim3(grid), dim3(256), 0, s, a);
+        else if (D == 64) hipLaunchKernelGGL((page_write_kernel<ST, PT, 64, true>), dim3(grid), dim3(256), 0, s, a);
+        else return BZ_ERR_UNSUPPORTED;
+    } else {
+        if (D == 128) hipLaunchKernelGGL((append_kernel<ST, PT, 128>), dim3(grid), dim3(256), 0, s, a);
+        else if (D == 64) hipLaunchKernelGGL((append_kernel<ST, PT, 64>), dim3(grid), dim3(256), 0, s, a);
+        else return BZ_ERR_UNSUPPORTED;
+    }
     BZ_LAUNCH_CHECK();
     return 0;
 }
