@@ -38,7 +38,7 @@ struct MfmaDecodeArgs {
     const int32_t* steps_ahead; // optional: the table (and the plan made from it) is this many steps ahead
     const MfmaPiece* pieces;
     const MfmaTile* tiles;
-    const int32_t* tile_ptr;
+    const MfmaSlotHead* heads;
     float* part_o;   // [num_partials][16][128]
     float* part_lse; // [num_partials][16]
     uint64_t stride_page, stride_n, stride_h; // elements
@@ -118,7 +118,7 @@ __device__ __forceinline__ void wave_lds_sync() {
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 }
 
-constexpr int kInfoInts = 12; // per-tile description kept in LDS (see fetch_info)
+constexpr int kInfoInts = 12; // per-tile description kept in LDS (see fetch_info): 9 ints, padded
 
 // KV8: the pool holds e4m3 bytes.  K and V are widened to the 16-bit type of q in registers (exactly)
 // on their way to the matrix cores; the per-head scales are folded into the softmax scale and into
@@ -131,7 +131,7 @@ __global__ __launch_bounds__(64, 2) void decode_mfma_kernel(MfmaDecodeArgs a, co
                                                             const int32_t* __restrict__ indices,
                                                             const MfmaPiece* __restrict__ pieces,
                                                             const MfmaTile* __restrict__ tiles,
-                                                            const int32_t* __restrict__ tile_ptr) {
+                                                            const MfmaSlotHead* __restrict__ heads) {
     using M = Mma<BF16>;
     __shared__ __attribute__((aligned(16))) unsigned char v_lds[kTileTok * kVRowBytes];
     __shared__ __attribute__((aligned(16))) int info_lds[2][32][kInfoInts];
@@ -150,15 +150,19 @@ __global__ __launch_bounds__(64, 2) void decode_mfma_kernel(MfmaDecodeArgs a, co
 
     // A plan made from a table that runs ahead lists tiles up to the future lengths; at present every
     // sequence is `ahead` tokens shorter.  Tiles past the present end are masked as a whole (their pages
-    // exist), so a piece can come out empty: zero weight in the split-K combine.  (Read together with
-    // the slot boundaries: one round trip, not two.)
+    // exist), so a piece can come out empty: zero weight in the split-K combine.
+    // The slot's head holds its range of tile records and the description of the first tile: after one
+    // round trip (head and counter together) only the two page ids stand between the wave and its first
+    // K/V loads.
     const int ahead_raw = a.steps_ahead ? *a.steps_ahead : 0;
-    const int g_begin = tile_ptr[blockIdx.x], g_end = tile_ptr[blockIdx.x + 1];
+    const MfmaSlotHead* __restrict__ head = heads + blockIdx.x;
+    const int g_begin = head->begin, g_end = head->end;
+    const MfmaSlotHead first = *head;
     if (g_begin >= g_end) return;
     const int ahead = max(ahead_raw, 0);
 
     // ---- descriptions of 32 tiles at a time: lane l < 32 fetches the record of tile base+l, the two
-    // page ids it points at and the piece it belongs to, and leaves 12 ints in LDS:
+    // page ids it points at and the piece it belongs to, and leaves 9 ints in LDS:
     //   [pid0, pid1, t, seq | kvh, flags (1: first tile of its piece, 2: last), partial, tok_end | seq_len]
     struct Desc { int v[9]; };
     auto fetch_info = [&](int base) -> Desc {
@@ -253,17 +257,21 @@ __global__ __launch_bounds__(64, 2) void decode_mfma_kernel(MfmaDecodeArgs a, co
         }
     };
 
-    {
-        const Desc d0 = fetch_info(g_begin);
-        stash_info(d0, 0);
-        wave_lds_sync();
-    }
-    int chunk_base = g_begin, buf = 0;
-    Desc dnext;
-    TileUni un = read_info(0, 0); // description of the tile whose loads are issued next
+    // The records of the first 32 tiles are requested first and the first tile's q, K and V right behind
+    // them (its description came with the slot head), so parking the records in LDS waits for them only.
+    const Desc d0 = fetch_info(g_begin);
+    TileUni un; // description of the tile whose loads are issued next
+    un.pid0 = indices[first.idx0];
+    un.pid1 = indices[first.idx1];
+    un.t = first.t; un.seq = first.seq; un.kvh = first.kvh; un.flags = first.flags; un.partial = first.partial;
+    un.seq_len = max(first.seq_len - ahead, 0);
+    un.tok_end = min(first.tile_end * kTileTok, un.seq_len);
     issue_q(un);
     issue_loads(tile_base(un));
-
+    stash_info(d0, 0);
+    wave_lds_sync();
+    int chunk_base = g_begin, buf = 0;
+    Desc dnext;
 
     uint4 qhi[4], qlo[4];
     float m_run = -INFINITY, l_run = 0.f;
@@ -517,7 +525,7 @@ struct DecodeArgs; // general-kernel argument block (bz_decode.hip); only its sc
 template <bool BF16, typename OT, bool ROPE_Q, bool KV8>
 static void launch_mfma_k(const DecodePlan* p, const MfmaDecodeArgs& a, hipStream_t s) {
     hipLaunchKernelGGL((decode_mfma_kernel<BF16, OT, ROPE_Q, KV8>), dim3(p->mfma_slots), dim3(64), 0, s, a,
-                       (const char*)a.q, a.k_data, a.v_data, a.indices, a.pieces, a.tiles, a.tile_ptr);
+                       (const char*)a.q, a.k_data, a.v_data, a.indices, a.pieces, a.tiles, a.heads);
 }
 
 template <bool BF16, typename OT>
@@ -555,7 +563,7 @@ int decode_fast_path(const DecodePlan* p, const void* q, void* out, float* lse, 
     a.k_data = (const char*)kv->k_data; a.v_data = (const char*)kv->v_data;
     a.indices = kv->indices; a.indptr = kv->indptr; a.last_page_len = kv->last_page_len;
     a.steps_ahead = kv->steps_ahead;
-    a.pieces = p->mfma_pieces_d; a.tiles = p->mfma_tiles_d; a.tile_ptr = p->mfma_tile_ptr_d;
+    a.pieces = p->mfma_pieces_d; a.tiles = p->mfma_tiles_d; a.heads = p->mfma_heads_d;
     a.part_o = p->mfma_part_o; a.part_lse = p->mfma_part_lse;
     a.stride_page = kv->stride_page; a.stride_n = kv->stride_n; a.stride_h = kv->stride_h;
     a.page_size = kv->page_size; a.num_qo_heads = num_qo_heads; a.group = num_qo_heads / kv->num_kv_heads;

@@ -109,7 +109,7 @@ extern "C" int bz_decode_plan(bz_decode_plan_t* plan_, void* float_buffer, size_
     // gets a 16-byte record so that the kernel never has to chase the piece list tile by tile.
     std::vector<MfmaPiece> mp;
     std::vector<MfmaTile> mt;
-    std::vector<int32_t> mptr; // tiles of slot s: [mptr[s], mptr[s+1])
+    std::vector<int32_t> mptr; // tiles of slot s: [mptr[s], mptr[s+1]); uploaded as one MfmaSlotHead per slot
     std::vector<MfmaCombine> mc;
     uint32_t mfma_partials = 0;
     const uint32_t group = num_qo_heads / num_kv_heads;
@@ -217,7 +217,8 @@ extern "C" int bz_decode_plan(bz_decode_plan_t* plan_, void* float_buffer, size_
     if (part_o_bytes + part_lse_bytes > float_buffer_bytes) return BZ_ERR_WORKSPACE;
     // the MFMA schedule is optional: without room for it the general kernel runs
     const size_t mp_bytes = align_up(mp.size() * sizeof(MfmaPiece), 256);
-    const size_t mptr_bytes = align_up(mptr.size() * sizeof(int32_t), 256);
+    const size_t nheads = mptr.empty() ? 0 : mptr.size() - 1;
+    const size_t mptr_bytes = align_up(nheads * sizeof(MfmaSlotHead), 256); // slot heads
     const size_t mc_bytes = align_up(mc.size() * sizeof(MfmaCombine), 256);
     const size_t cnt_bytes = align_up(mt.size() * sizeof(MfmaTile), 256); // tile records
     const size_t mpart_o_bytes = align_up((size_t)mfma_partials * 16 * 128 * sizeof(float), 256);
@@ -244,7 +245,20 @@ extern "C" int bz_decode_plan(bz_decode_plan_t* plan_, void* float_buffer, size_
     if (!empty.empty()) memcpy(st + seg_bytes + combo_bytes, empty.data(), empty.size() * sizeof(int32_t));
     if (mfma_ok) {
         memcpy(st + base_total, mp.data(), mp.size() * sizeof(MfmaPiece));
-        memcpy(st + base_total + mp_bytes, mptr.data(), mptr.size() * sizeof(int32_t));
+        MfmaSlotHead* heads = reinterpret_cast<MfmaSlotHead*>(st + base_total + mp_bytes);
+        for (size_t sl = 0; sl < nheads; ++sl) {
+            const int32_t b0 = mptr[sl], e0 = mptr[sl + 1];
+            MfmaSlotHead hd = {b0, e0, 0, 0, 0, 0, 0, 0, -1, 0, 0, 0};
+            if (b0 < e0) {
+                const MfmaTile& r = mt[(size_t)b0];
+                const MfmaPiece& pc = mp[(size_t)r.piece];
+                hd.idx0 = r.idx0; hd.idx1 = r.idx1; hd.t = r.t;
+                hd.seq = pc.seq; hd.kvh = pc.kvh;
+                hd.flags = (r.t == pc.tile_begin ? 1 : 0) | (r.t + 1 == pc.tile_end ? 2 : 0);
+                hd.partial = pc.partial; hd.tile_end = pc.tile_end; hd.seq_len = pc.seq_len;
+            }
+            heads[sl] = hd;
+        }
         if (!mc.empty()) memcpy(st + base_total + mp_bytes + mptr_bytes, mc.data(), mc.size() * sizeof(MfmaCombine));
         memcpy(st + base_total + mp_bytes + mptr_bytes + mc_bytes, mt.data(), mt.size() * sizeof(MfmaTile));
     }
@@ -264,10 +278,9 @@ extern "C" int bz_decode_plan(bz_decode_plan_t* plan_, void* float_buffer, size_
     p->mfma_ok = mfma_ok;
     if (mfma_ok) {
         p->mfma_pieces_d = (const MfmaPiece*)((char*)int_buffer + base_total);
-        p->mfma_piece_ptr_d = (const int32_t*)((char*)int_buffer + base_total + mp_bytes);
+        p->mfma_heads_d = (const MfmaSlotHead*)((char*)int_buffer + base_total + mp_bytes);
         p->mfma_combos_d = (const MfmaCombine*)((char*)int_buffer + base_total + mp_bytes + mptr_bytes);
         p->mfma_tiles_d = (const MfmaTile*)((char*)int_buffer + base_total + mp_bytes + mptr_bytes + mc_bytes);
-        p->mfma_tile_ptr_d = p->mfma_piece_ptr_d;
         p->mfma_part_o = (float*)float_buffer; // the two paths never run in the same call: same workspace
         p->mfma_part_lse = (float*)((char*)float_buffer + mpart_o_bytes);
         p->mfma_slots = (uint32_t)mptr.size() - 1;

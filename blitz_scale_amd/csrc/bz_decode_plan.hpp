@@ -37,6 +37,19 @@ struct MfmaTile {
     int32_t piece;      // index into the piece array
 };
 
+// What a wave slot reads first: its range of tile records and the full description of the first of
+// them (record and piece joined), so that the loads of the first tile go out after one round trip.
+struct MfmaSlotHead {
+    int32_t begin, end;   // tile records [begin, end)
+    int32_t idx0, idx1, t; // the first record
+    int32_t seq, kvh;
+    int32_t flags;        // 1: first tile of its piece, 2: last tile of its piece
+    int32_t partial;      // -1 or partial slot
+    int32_t tile_end;     // one past the last tile of the piece
+    int32_t seq_len;
+    int32_t pad;
+};
+
 // One split (sequence, kv head): partial slots [first, first+count).
 struct MfmaCombine {
     int32_t seq, kvh, first, count;
@@ -58,10 +71,9 @@ struct DecodePlan {
     bool force_general = false; // tests: run the general kernel even where the MFMA path applies
     uint32_t mfma_slots = 0, mfma_combos = 0, mfma_partials = 0, mfma_pieces = 0, mfma_split_seqs = 0;
     const MfmaPiece* mfma_pieces_d = nullptr;
-    const int32_t* mfma_piece_ptr_d = nullptr;
     const MfmaCombine* mfma_combos_d = nullptr;
     const MfmaTile* mfma_tiles_d = nullptr;
-    const int32_t* mfma_tile_ptr_d = nullptr; // tiles of slot s: [tile_ptr[s], tile_ptr[s+1])
+    const MfmaSlotHead* mfma_heads_d = nullptr; // one per wave slot
     float* mfma_part_o = nullptr;
     float* mfma_part_lse = nullptr;
     // pinned staging for the schedule upload and the event that guards its reuse
