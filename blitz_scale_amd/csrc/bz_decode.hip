@@ -311,6 +311,8 @@ extern "C" int bz_batch_decode(bz_decode_plan_t* plan_, const void* q, int q_dty
     DecodePlan* p = reinterpret_cast<DecodePlan*>(plan_);
     if (!p || !kv || !q || !out) return BZ_ERR_BAD_ARG;
     if (!p->planned) return BZ_ERR_NOT_PLANNED;
+    // a table whose device pointers were cleared after the previous step (src/blitz/stub.h:1361-1363)
+    if (!kv->k_data || !kv->v_data || !kv->indices || !kv->indptr || !kv->last_page_len) return BZ_ERR_BAD_ARG;
     if (kv->batch_size != p->batch_size || kv->page_size != p->page_size || kv->num_kv_heads != p->num_kv_heads ||
         kv->head_dim != p->head_dim || num_qo_heads != p->num_qo_heads)
         return BZ_ERR_BAD_ARG;

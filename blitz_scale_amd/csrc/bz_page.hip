@@ -301,8 +301,10 @@ static int launch_page_write(const PageWriteArgs& a, int src_dtype, int pool_dty
 }
 
 static int fill_args(PageWriteArgs& a, const bz_paged_kv_t* kv, const void* k, const void* v, void* q_inout,
-                     uint32_t num_qo_heads, int rope, float rope_theta, const float* k_scale, const float* v_scale) {
+                     uint32_t num_qo_heads, int rope, float rope_theta, const float* k_scale, const float* v_scale,
+                     bool prefill) {
     if (!kv || !k || !v || !kv->k_data || !kv->v_data) return BZ_ERR_BAD_ARG;
+    if (!kv->indices || !kv->indptr || (!prefill && !kv->last_page_len)) return BZ_ERR_BAD_ARG;
     if (kv->stride_n % 8 || kv->stride_h % 8 || kv->stride_page % 8) return BZ_ERR_BAD_ARG;
     a.k_data = (char*)kv->k_data; a.v_data = (char*)kv->v_data;
     a.indices = kv->indices; a.indptr = kv->indptr; a.last_page_len = kv->last_page_len;
@@ -338,7 +340,7 @@ extern "C" int bz_store_prefill_kv(const bz_paged_kv_t* kv, void* k, const void*
                                    uint32_t num_qo_heads, int rope, float rope_theta, const float* k_scale,
                                    const float* v_scale, void* stream) {
     PageWriteArgs a;
-    int rc = fill_args(a, kv, k, v, q_inout, num_qo_heads, rope, rope_theta, k_scale, v_scale);
+    int rc = fill_args(a, kv, k, v, q_inout, num_qo_heads, rope, rope_theta, k_scale, v_scale, true);
     if (rc) return rc;
     if (!ragged_indptr) return BZ_ERR_BAD_ARG;
     a.ragged_indptr = ragged_indptr;
@@ -351,7 +353,7 @@ extern "C" int bz_append_decode_kv(const bz_paged_kv_t* kv, const void* k, const
                                    void* q_inout, uint32_t num_qo_heads, int rope, float rope_theta,
                                    const float* k_scale, const float* v_scale, void* stream) {
     PageWriteArgs a;
-    int rc = fill_args(a, kv, k, v, q_inout, num_qo_heads, rope, rope_theta, k_scale, v_scale);
+    int rc = fill_args(a, kv, k, v, q_inout, num_qo_heads, rope, rope_theta, k_scale, v_scale, false);
     if (rc) return rc;
     return launch_page_write<false>(a, src_dtype, kv->kv_dtype, (int)kv->head_dim, kv->batch_size,
                                     (hipStream_t)stream);

@@ -47,3 +47,38 @@ def test_layout_strides_and_pool_size():
     lib.bz_kv_layer_view(kv, 1 << 40, 3, 1000)  # layer stride = max_pages * stride_page (llama.h:378-381)
     assert kv.k_data == (1 << 40) + 3 * 1000 * kv.stride_page * 2
     assert kv.v_data == kv.k_data + kv.stride_page  # v = k + H*P*D elements (page.h:42-43)
+
+
+def test_argument_errors_are_reported_before_anything_touches_a_gpu():
+    """Bad arguments come back as BZ_ERR_* codes from the host-side checks (no kernel is launched on a
+    null table, an unplanned handle or an unsupported type), so this runs without a GPU."""
+    import ctypes as C
+    lib = _lib.load()
+    kv = _lib.BzPagedKV()
+    kv.num_kv_heads, kv.page_size, kv.head_dim, kv.kv_dtype, kv.batch_size = 8, 16, 128, _lib.BZ_BF16, 4
+    lib.bz_paged_kv_set_layout(kv, _lib.BZ_LAYOUT_HND)
+    fake = C.c_void_p(1 << 20)  # never dereferenced on the host
+    assert lib.bz_batch_decode(None, fake, _lib.BZ_BF16, C.byref(kv), fake, _lib.BZ_BF16, 32, 0, 1e4, 0.0, None,
+                               None, None, None) == _lib.BZ_ERR_BAD_ARG
+    plan = lib.bz_decode_plan_create()
+    try:
+        assert lib.bz_batch_decode(plan, fake, _lib.BZ_BF16, C.byref(kv), fake, _lib.BZ_BF16, 32, 0, 1e4, 0.0, None,
+                                   None, None, None) == _lib.BZ_ERR_NOT_PLANNED
+        assert lib.bz_decode_plan(plan, fake, 1 << 20, fake, 1 << 20, None, None, 4, 32, 8, 128, 16, 0,
+                                  None) == _lib.BZ_ERR_BAD_ARG
+        assert lib.bz_decode_plan_info(plan, None, None, None) == _lib.BZ_ERR_NOT_PLANNED
+    finally:
+        lib.bz_decode_plan_destroy(plan)
+    # page writers: pool pointers set, table pointers cleared (what Stub::forward leaves behind after a step)
+    kv.k_data, kv.v_data = 1 << 30, (1 << 30) + 4096
+    assert lib.bz_append_decode_kv(C.byref(kv), fake, fake, _lib.BZ_BF16, None, 0, 0, 1e4, None, None,
+                                   None) == _lib.BZ_ERR_BAD_ARG
+    assert lib.bz_store_prefill_kv(C.byref(kv), fake, fake, _lib.BZ_BF16, None, 16, None, 0, 0, 1e4, None, None,
+                                   None) == _lib.BZ_ERR_BAD_ARG
+    assert lib.bz_steps_ahead_advance(None, None) == _lib.BZ_ERR_BAD_ARG
+    # migration payload: an e4m3 pool cannot travel as bf16
+    kv.kv_dtype = _lib.BZ_E4M3
+    assert lib.bz_kv_pages_pack(fake, 100, C.byref(kv), fake, 4, 0, 2, fake, _lib.BZ_BF16, None, None,
+                                None) == _lib.BZ_ERR_UNSUPPORTED
+    assert lib.bz_kv_pages_pack(fake, 100, None, fake, 4, 0, 2, fake, _lib.BZ_E4M3, None, None,
+                                None) == _lib.BZ_ERR_BAD_ARG
