@@ -140,3 +140,34 @@ def test_decode_steps_from_one_plan(dtype, kv_dtype, Hq, Hkv, D, P, layout, ctx0
 
     # past the horizon the counter stays at zero and the table is the present
     assert int(ahead.item()) == 0
+
+
+@pytest.mark.parametrize("Hq,Hkv,D", [(32, 8, 128), (4, 4, 64)])
+def test_counter_larger_than_a_sequence(Hq, Hkv, D):
+    """A counter that leaves a sequence without tokens: the append skips it, its output row is zero, the
+    other sequences are unaffected (MFMA kernel and general kernel)."""
+    dtype, P = BZ_F16, 16
+    ctx = np.asarray([3, 40, 5, 200])
+    ahead_n = 5
+    p = DecodeProblem(0xB0B, ctx, Hq, Hkv, D, P, dtype)
+    dev = DeviceDecode(p)
+    dev.plan(split_tokens=64)
+    dev.pt.steps_ahead_d = torch.tensor([ahead_n], dtype=torch.int32, device="cuda")
+    lens = np.maximum(ctx - ahead_n, 0)  # [0, 35, 0, 195]
+    rng = np.random.default_rng(5)
+    k_bits, v_bits = wl.randn_bits(rng, (p.B, Hkv, D), dtype), wl.randn_bits(rng, (p.B, Hkv, D), dtype)
+    K.append_decode_kv_cache(dev.pt, to_dev(k_bits, dtype), to_dev(v_bits, dtype))
+    torch.cuda.synchronize()
+    want = p.pool.copy()
+    live = [b for b in range(p.B) if lens[b] > 0]
+    for b in live:  # raw copy: bit-exact
+        idx = row_elements(p, b, int(lens[b]) - 1)
+        half = idx.size // 2
+        want[idx[:half]] = k_bits[b].reshape(-1)
+        want[idx[half:]] = v_bits[b].reshape(-1)
+    pool_got = to_host_bits(dev.pool)
+    assert np.array_equal(pool_got, want)
+    got = dev.decode(None, BZ_ROPE_NONE)
+    ref = oracle.batch_decode(p.q, dtype, truncated_kv(p, pool_got, lens), Hq, rope_mode=BZ_ROPE_NONE)
+    assert not got[lens == 0].any()
+    assert (np.abs(got[lens > 0] - ref[lens > 0]) <= 2e-3).all()
