@@ -74,9 +74,10 @@ extern "C" int bz_decode_plan(bz_decode_plan_t* plan_, void* float_buffer, size_
     while (!never_split && piece > min_pages && count_items(piece) < (uint64_t)cus * 4)
         piece = std::max(min_pages, piece / 2);
 
-    std::vector<DecodeSegment> segs;
-    std::vector<DecodeCombine> combos;
-    std::vector<int32_t> empty;
+    std::vector<DecodeSegment>& segs = p->h_segs;
+    std::vector<DecodeCombine>& combos = p->h_combos;
+    std::vector<int32_t>& empty = p->h_empty;
+    segs.clear(); combos.clear(); empty.clear();
     uint32_t partials = 0;
     for (uint32_t b = 0; b < batch_size; ++b) {
         const int32_t np = indptr_h[b + 1] - indptr_h[b];
@@ -107,10 +108,11 @@ extern "C" int bz_decode_plan(bz_decode_plan_t* plan_, void* float_buffer, size_
     // head) boundary becomes several pieces; a (sequence, kv head) that ends up in more than one
     // piece, or is longer than split_tokens, is folded from partial results.  Every tile of a share
     // gets a 16-byte record so that the kernel never has to chase the piece list tile by tile.
-    std::vector<MfmaPiece> mp;
-    std::vector<MfmaTile> mt;
-    std::vector<int32_t> mptr; // tiles of slot s: [mptr[s], mptr[s+1]); uploaded as one MfmaSlotHead per slot
-    std::vector<MfmaCombine> mc;
+    std::vector<MfmaPiece>& mp = p->h_pieces;
+    std::vector<MfmaTile>& mt = p->h_tiles;
+    std::vector<int32_t>& mptr = p->h_slot_ptr; // tiles of slot s: [mptr[s], mptr[s+1]); uploaded as one MfmaSlotHead per slot
+    std::vector<MfmaCombine>& mc = p->h_mcombos;
+    mp.clear(); mt.clear(); mptr.clear(); mc.clear();
     uint32_t mfma_partials = 0;
     const uint32_t group = num_qo_heads / num_kv_heads;
     const bool mfma_shape = head_dim == 128 && page_size % 16 == 0 && group <= 16;
@@ -145,7 +147,8 @@ extern "C" int bz_decode_plan(bz_decode_plan_t* plan_, void* float_buffer, size_
             return std::max<uint64_t>(1, hi > lo ? hi - lo : 1);
         };
         uint64_t room = slot_share(); // tiles the current slot can still take
-        mt.reserve(total_tiles);
+        mt.resize(total_tiles); // sized once (records are written in place below)
+        size_t n_rec = 0;
         mptr.push_back(0);
         for (uint32_t b = 0; b < batch_size; ++b) {
             const int32_t np = indptr_h[b + 1] - indptr_h[b];
@@ -157,7 +160,7 @@ extern "C" int bz_decode_plan(bz_decode_plan_t* plan_, void* float_buffer, size_
                 int32_t t = 0;
                 while (t < tiles) {
                     if (room == 0) {
-                        mptr.push_back((int32_t)mt.size());
+                        mptr.push_back((int32_t)n_rec);
                         ++slot;
                         wacc += slot_weight(slot);
                         room = slot_share();
@@ -168,9 +171,8 @@ extern "C" int bz_decode_plan(bz_decode_plan_t* plan_, void* float_buffer, size_
                     room -= std::min<uint64_t>(room, (uint64_t)take);
                     // one record per tile; page sizes are powers of two in practice, so the two page
                     // indices of a tile come from shifts rather than 64-bit divisions
-                    const size_t first_rec = mt.size();
-                    mt.resize(first_rec + (size_t)take);
-                    MfmaTile* rec = mt.data() + first_rec;
+                    MfmaTile* rec = mt.data() + n_rec;
+                    n_rec += (size_t)take;
                     const int32_t piece_id = (int32_t)mp.size(), ip0 = indptr_h[b];
                     if (page_shift >= 0) {
                         for (int32_t tt = t; tt < t + take; ++tt, ++rec) {
@@ -203,7 +205,7 @@ extern "C" int bz_decode_plan(bz_decode_plan_t* plan_, void* float_buffer, size_
                 }
             }
         }
-        mptr.push_back((int32_t)mt.size());
+        mptr.push_back((int32_t)n_rec);
     }
 
     // ---- workspaces -------------------------------------------------------------------------

@@ -76,6 +76,14 @@ struct DecodePlan {
     const MfmaSlotHead* mfma_heads_d = nullptr; // one per wave slot
     float* mfma_part_o = nullptr;
     float* mfma_part_lse = nullptr;
+    // host scratch of plan(), kept between calls so that a step's plan neither allocates nor faults in
+    // fresh pages (the schedule of a large batch is around a megabyte)
+    std::vector<DecodeSegment> h_segs;
+    std::vector<DecodeCombine> h_combos;
+    std::vector<int32_t> h_empty, h_slot_ptr;
+    std::vector<MfmaPiece> h_pieces;
+    std::vector<MfmaTile> h_tiles;
+    std::vector<MfmaCombine> h_mcombos;
     // pinned staging for the schedule upload and the event that guards its reuse
     void* staging = nullptr;
     size_t staging_bytes = 0;
