@@ -330,6 +330,48 @@ int main() {
                wire_ok ? "bit-exact" : "MISMATCH");
     }
 
+    // ---- three more decode steps from ONE table upload and ONE plan: the table is grown three steps
+    // ahead and a device counter says how far the present lags behind it (PageTable::steps_ahead_d)
+    bool ahead_ok = true;
+    {
+        const int H = 3;
+        std::vector<std::vector<int32_t>> ind(H), ptr(H), lpl(H); // the table as it is at each step, for the checker
+        for (int i = 0; i < H; ++i) {
+            batch.grow();
+            ind[i] = pt.indices; ptr[i] = pt.indptr; lpl[i] = pt.last_page_len;
+        }
+        cm.set_layer(pt, 1);
+        upload_table();
+        decode_h.plan(float_ws, 8 << 20, int_ws, 1 << 20, pt.indptr_h, pt.last_page_len_h, B, Hq, Hkv, D, P);
+        int32_t* counter_d;
+        const int32_t c0 = H - 1;
+        HIP_OK(hipMalloc(&counter_d, 4));
+        HIP_OK(hipMemcpy(counter_d, &c0, 4, hipMemcpyHostToDevice));
+        pt.steps_ahead_d = counter_d;
+        // the checker continues from what the device's pool holds
+        HIP_OK(hipMemcpy(pool_cpu.data(), cm.get_base_ptr(), pool_cpu.size() * 2, hipMemcpyDeviceToHost));
+        for (int i = 0; i < H; ++i) {
+            bits_t xs = rand_bits((size_t)B * hidden, 1.0f);
+            HIP_OK(hipMemcpy(ws_d, xs.data(), xs.size() * 2, hipMemcpyHostToDevice));
+            attn.forward(B, nullptr, pt);
+            glu.forward(B);
+            ahead_ok = ahead_ok && bz_steps_ahead_advance(counter_d, nullptr) == 0;
+            HIP_OK(hipDeviceSynchronize());
+            bits_t got((size_t)B * hidden);
+            HIP_OK(hipMemcpy(got.data(), ws_d, got.size() * 2, hipMemcpyDeviceToHost));
+            okv.indices = ind[i].data(); okv.indptr = ptr[i].data(); okv.last_page_len = lpl[i].data();
+            bits_t want = xs;
+            layer_cpu(want, B, false);
+            const double e = max_abs_diff(got.data(), want.data(), want.size());
+            printf("decode step %d of %d from one plan: max |gpu - cpu| = %.3e\n", i + 1, H, e);
+            ahead_ok = ahead_ok && e < 2e-2;
+        }
+        int32_t c_end = -1;
+        HIP_OK(hipMemcpy(&c_end, counter_d, 4, hipMemcpyDeviceToHost));
+        ahead_ok = ahead_ok && c_end == 0;
+        pt.steps_ahead_d = nullptr;
+    }
+
     // error convention: std::runtime_error with the reference's message prefix
     bool threw = false;
     try {
@@ -339,7 +381,7 @@ int main() {
         threw = strncmp(e.what(), "batchDecodeAttention error: ", 28) == 0;
     }
     // the activations are O(1); a chain of f16 roundings through four GEMMs stays within a few 1e-3
-    const bool ok = e1 < 2e-2 && e2 < 2e-2 && e3 < 5e-3 && touched0 == 0 && threw && ends_ok && wire_ok;
+    const bool ok = e1 < 2e-2 && e2 < 2e-2 && e3 < 5e-3 && touched0 == 0 && threw && ends_ok && wire_ok && ahead_ok;
     printf(ok ? "PASS\n" : "FAIL\n");
     return ok ? 0 : 1;
 }
