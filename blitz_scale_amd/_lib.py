@@ -50,6 +50,9 @@ SIGNATURES = {
     "bz_decode_plan_create": (_vp, []),
     "bz_decode_plan_destroy": (None, [_vp]),
     "bz_decode_plan": (_i32, [_vp, _vp, _sz, _vp, _sz, _vp, _vp, _u32, _u32, _u32, _u32, _u32, _u32, _vp]),
+    "bz_decode_plan_workspace": (_i32, [_vp, _vp, _vp, _u32, _u32, _u32, _u32, _u32, _u32, _u32, C.POINTER(_sz),
+                                        C.POINTER(_sz)]),
+    "bz_decode_plan_host_schedule": (_i32, [_vp, _i32, C.POINTER(_vp), C.POINTER(_sz), C.POINTER(_u32)]),
     "bz_decode_plan_info": (_i32, [_vp, C.POINTER(_u32), C.POINTER(_u32), C.POINTER(_u32)]),
     "bz_decode_plan_set_timing_events": (_i32, [_vp, _vp, _vp]),
     "bz_batch_decode": (_i32, [_vp, _vp, _i32, _kvp, _vp, _i32, _u32, _i32, _f32, _f32, _vp, _vp, _vp, _vp]),

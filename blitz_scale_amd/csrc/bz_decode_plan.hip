@@ -43,21 +43,27 @@ extern "C" void bz_decode_plan_destroy(bz_decode_plan_t* plan_) {
     delete p;
 }
 
-extern "C" int bz_decode_plan(bz_decode_plan_t* plan_, void* float_buffer, size_t float_buffer_bytes,
-                              void* int_buffer, size_t int_buffer_bytes, const int32_t* indptr_h,
-                              const int32_t* last_page_len_h, uint32_t batch_size, uint32_t num_qo_heads,
-                              uint32_t num_kv_heads, uint32_t head_dim, uint32_t page_size, uint32_t split_tokens,
-                              void* stream) {
-    DecodePlan* p = reinterpret_cast<DecodePlan*>(plan_);
-    if (!p || !indptr_h || !last_page_len_h || !float_buffer || !int_buffer) return BZ_ERR_BAD_ARG;
-    if (page_size == 0 || num_kv_heads == 0 || num_qo_heads % num_kv_heads) return BZ_ERR_BAD_ARG;
-    p->planned = false;
-    if (split_tokens == 0) split_tokens = 2048;
+namespace bz {
 
+struct ScheduleCounts {
+    uint32_t partials = 0, mfma_partials = 0;
+    bool mfma_shape = false;
+};
+
+// Section sizes of the schedule inside the two workspaces (each section 256-byte aligned).
+struct ScheduleLayout {
+    size_t seg_bytes, combo_bytes, empty_bytes, base_total, part_o_bytes, part_lse_bytes;
+    size_t mp_bytes, nheads, mptr_bytes, mc_bytes, cnt_bytes, mpart_o_bytes, mpart_lse_bytes;
+};
+
+// Pure host work: fills the plan's host scratch (h_*) from the host copies of the page table.
+static int build_schedule(DecodePlan* p, const int32_t* indptr_h, const int32_t* last_page_len_h, uint32_t batch_size,
+                          uint32_t num_qo_heads, uint32_t num_kv_heads, uint32_t head_dim, uint32_t page_size,
+                          uint32_t split_tokens, int cus, ScheduleCounts* counts) {
+    if (split_tokens == 0) split_tokens = 2048;
     // ---- choose the piece length (in pages) -------------------------------------------------
     // Pieces never exceed split_tokens (contexts longer than that are always split); they are
     // shortened further, down to 256 tokens, until the launch holds about four workgroups per CU.
-    const int cus = device_cu_count();
     const uint32_t max_pages_cap = std::max<uint32_t>(1, split_tokens / page_size);
     const uint32_t min_pages = std::min<uint32_t>(max_pages_cap, std::max<uint32_t>(1, 256 / page_size));
     uint32_t piece = max_pages_cap;
@@ -208,23 +214,65 @@ extern "C" int bz_decode_plan(bz_decode_plan_t* plan_, void* float_buffer, size_
         mptr.push_back((int32_t)n_rec);
     }
 
+    counts->partials = partials;
+    counts->mfma_partials = mfma_partials;
+    counts->mfma_shape = mfma_shape;
+    return 0;
+}
+
+static ScheduleLayout schedule_layout(const DecodePlan* p, const ScheduleCounts& c, uint32_t num_qo_heads,
+                                      uint32_t head_dim) {
+    ScheduleLayout L;
+    L.seg_bytes = align_up(p->h_segs.size() * sizeof(DecodeSegment), 256);
+    L.combo_bytes = align_up(p->h_combos.size() * sizeof(DecodeCombine), 256);
+    L.empty_bytes = align_up(p->h_empty.size() * sizeof(int32_t), 256);
+    L.base_total = L.seg_bytes + L.combo_bytes + L.empty_bytes;
+    L.part_o_bytes = align_up((size_t)c.partials * num_qo_heads * head_dim * sizeof(float), 256);
+    L.part_lse_bytes = align_up((size_t)c.partials * num_qo_heads * sizeof(float), 256);
+    L.mp_bytes = align_up(p->h_pieces.size() * sizeof(MfmaPiece), 256);
+    L.nheads = p->h_slot_ptr.empty() ? 0 : p->h_slot_ptr.size() - 1;
+    L.mptr_bytes = align_up(L.nheads * sizeof(MfmaSlotHead), 256); // slot heads
+    L.mc_bytes = align_up(p->h_mcombos.size() * sizeof(MfmaCombine), 256);
+    L.cnt_bytes = align_up(p->h_tiles.size() * sizeof(MfmaTile), 256); // tile records
+    L.mpart_o_bytes = align_up((size_t)c.mfma_partials * 16 * 128 * sizeof(float), 256);
+    L.mpart_lse_bytes = align_up((size_t)c.mfma_partials * 16 * sizeof(float), 256);
+    return L;
+}
+
+} // namespace bz
+
+extern "C" int bz_decode_plan(bz_decode_plan_t* plan_, void* float_buffer, size_t float_buffer_bytes,
+                              void* int_buffer, size_t int_buffer_bytes, const int32_t* indptr_h,
+                              const int32_t* last_page_len_h, uint32_t batch_size, uint32_t num_qo_heads,
+                              uint32_t num_kv_heads, uint32_t head_dim, uint32_t page_size, uint32_t split_tokens,
+                              void* stream) {
+    DecodePlan* p = reinterpret_cast<DecodePlan*>(plan_);
+    if (!p || !indptr_h || !last_page_len_h || !float_buffer || !int_buffer) return BZ_ERR_BAD_ARG;
+    if (page_size == 0 || num_kv_heads == 0 || num_qo_heads % num_kv_heads) return BZ_ERR_BAD_ARG;
+    p->planned = false;
+    ScheduleCounts counts;
+    const int rc = build_schedule(p, indptr_h, last_page_len_h, batch_size, num_qo_heads, num_kv_heads, head_dim,
+                                  page_size, split_tokens, device_cu_count(), &counts);
+    if (rc) return rc;
+    const std::vector<DecodeSegment>& segs = p->h_segs;
+    const std::vector<DecodeCombine>& combos = p->h_combos;
+    const std::vector<int32_t>& empty = p->h_empty;
+    const std::vector<MfmaPiece>& mp = p->h_pieces;
+    const std::vector<MfmaTile>& mt = p->h_tiles;
+    const std::vector<int32_t>& mptr = p->h_slot_ptr;
+    const std::vector<MfmaCombine>& mc = p->h_mcombos;
+    const uint32_t partials = counts.partials, mfma_partials = counts.mfma_partials;
+    const bool mfma_shape = counts.mfma_shape;
+
     // ---- workspaces -------------------------------------------------------------------------
-    const size_t seg_bytes = align_up(segs.size() * sizeof(DecodeSegment), 256);
-    const size_t combo_bytes = align_up(combos.size() * sizeof(DecodeCombine), 256);
-    const size_t empty_bytes = align_up(empty.size() * sizeof(int32_t), 256);
-    const size_t base_total = seg_bytes + combo_bytes + empty_bytes;
+    const ScheduleLayout L = schedule_layout(p, counts, num_qo_heads, head_dim);
+    const size_t seg_bytes = L.seg_bytes, combo_bytes = L.combo_bytes, base_total = L.base_total;
+    const size_t part_o_bytes = L.part_o_bytes, part_lse_bytes = L.part_lse_bytes;
+    const size_t mp_bytes = L.mp_bytes, nheads = L.nheads, mptr_bytes = L.mptr_bytes, mc_bytes = L.mc_bytes;
+    const size_t cnt_bytes = L.cnt_bytes, mpart_o_bytes = L.mpart_o_bytes, mpart_lse_bytes = L.mpart_lse_bytes;
     if (base_total > int_buffer_bytes) return BZ_ERR_WORKSPACE;
-    const size_t part_o_bytes = align_up((size_t)partials * num_qo_heads * head_dim * sizeof(float), 256);
-    const size_t part_lse_bytes = align_up((size_t)partials * num_qo_heads * sizeof(float), 256);
     if (part_o_bytes + part_lse_bytes > float_buffer_bytes) return BZ_ERR_WORKSPACE;
     // the MFMA schedule is optional: without room for it the general kernel runs
-    const size_t mp_bytes = align_up(mp.size() * sizeof(MfmaPiece), 256);
-    const size_t nheads = mptr.empty() ? 0 : mptr.size() - 1;
-    const size_t mptr_bytes = align_up(nheads * sizeof(MfmaSlotHead), 256); // slot heads
-    const size_t mc_bytes = align_up(mc.size() * sizeof(MfmaCombine), 256);
-    const size_t cnt_bytes = align_up(mt.size() * sizeof(MfmaTile), 256); // tile records
-    const size_t mpart_o_bytes = align_up((size_t)mfma_partials * 16 * 128 * sizeof(float), 256);
-    const size_t mpart_lse_bytes = align_up((size_t)mfma_partials * 16 * sizeof(float), 256);
     const bool mfma_ok = mfma_shape && !mp.empty() && base_total + mp_bytes + mptr_bytes + mc_bytes + cnt_bytes <= int_buffer_bytes &&
                          mpart_o_bytes + mpart_lse_bytes <= float_buffer_bytes;
     const size_t total = mfma_ok ? base_total + mp_bytes + mptr_bytes + mc_bytes + cnt_bytes : base_total;
@@ -300,6 +348,46 @@ extern "C" int bz_decode_plan(bz_decode_plan_t* plan_, void* float_buffer, size_
     p->force_general = path && !strcmp(path, "general");
 
     p->planned = true;
+    return 0;
+}
+
+extern "C" int bz_decode_plan_workspace(bz_decode_plan_t* plan_, const int32_t* indptr_h, const int32_t* last_page_len_h,
+                                        uint32_t batch_size, uint32_t num_qo_heads, uint32_t num_kv_heads,
+                                        uint32_t head_dim, uint32_t page_size, uint32_t split_tokens,
+                                        uint32_t num_compute_units, size_t* float_buffer_bytes,
+                                        size_t* int_buffer_bytes) {
+    DecodePlan* p = reinterpret_cast<DecodePlan*>(plan_);
+    if (!p || !indptr_h || !last_page_len_h) return BZ_ERR_BAD_ARG;
+    if (page_size == 0 || num_kv_heads == 0 || num_qo_heads % num_kv_heads) return BZ_ERR_BAD_ARG;
+    p->planned = false; // the host scratch no longer matches what the device holds
+    ScheduleCounts counts;
+    const int cus = num_compute_units ? (int)num_compute_units : device_cu_count();
+    const int rc = build_schedule(p, indptr_h, last_page_len_h, batch_size, num_qo_heads, num_kv_heads, head_dim,
+                                  page_size, split_tokens, cus, &counts);
+    if (rc) return rc;
+    const ScheduleLayout L = schedule_layout(p, counts, num_qo_heads, head_dim);
+    const bool mfma = counts.mfma_shape && !p->h_pieces.empty();
+    if (float_buffer_bytes)
+        *float_buffer_bytes = std::max(L.part_o_bytes + L.part_lse_bytes, mfma ? L.mpart_o_bytes + L.mpart_lse_bytes : 0);
+    if (int_buffer_bytes)
+        *int_buffer_bytes = L.base_total + (mfma ? L.mp_bytes + L.mptr_bytes + L.mc_bytes + L.cnt_bytes : 0);
+    return 0;
+}
+
+extern "C" int bz_decode_plan_host_schedule(const bz_decode_plan_t* plan_, int which, const int32_t** data,
+                                            size_t* num_records, uint32_t* ints_per_record) {
+    const DecodePlan* p = reinterpret_cast<const DecodePlan*>(plan_);
+    if (!p || !data || !num_records || !ints_per_record) return BZ_ERR_BAD_ARG;
+    switch (which) {
+    case 0: *data = (const int32_t*)p->h_segs.data(); *num_records = p->h_segs.size(); *ints_per_record = sizeof(DecodeSegment) / 4; break;
+    case 1: *data = (const int32_t*)p->h_combos.data(); *num_records = p->h_combos.size(); *ints_per_record = sizeof(DecodeCombine) / 4; break;
+    case 2: *data = p->h_empty.data(); *num_records = p->h_empty.size(); *ints_per_record = 1; break;
+    case 3: *data = (const int32_t*)p->h_tiles.data(); *num_records = p->h_tiles.size(); *ints_per_record = sizeof(MfmaTile) / 4; break;
+    case 4: *data = p->h_slot_ptr.data(); *num_records = p->h_slot_ptr.size(); *ints_per_record = 1; break;
+    case 5: *data = (const int32_t*)p->h_pieces.data(); *num_records = p->h_pieces.size(); *ints_per_record = sizeof(MfmaPiece) / 4; break;
+    case 6: *data = (const int32_t*)p->h_mcombos.data(); *num_records = p->h_mcombos.size(); *ints_per_record = sizeof(MfmaCombine) / 4; break;
+    default: return BZ_ERR_BAD_ARG;
+    }
     return 0;
 }
 

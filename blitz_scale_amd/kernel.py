@@ -130,6 +130,28 @@ class BlitzBatchDecodeHandler:
         check(rc, "Handler plan")
         self._keep = (float_buffer, int_buffer)
 
+    def workspace(self, indptr_h, last_page_len_h, batch_size, num_qo_heads, num_kv_heads, head_dim, page_size, *,
+                  split_tokens=0, num_compute_units=0):
+        """(float_buffer_bytes, int_buffer_bytes) plan() would use for this batch; no GPU needed when
+        num_compute_units is given."""
+        ip, lp = _host_i32(indptr_h), _host_i32(last_page_len_h)
+        fb, ib = C.c_size_t(), C.c_size_t()
+        check(_lib.load().bz_decode_plan_workspace(self._h, ip.ctypes.data_as(C.c_void_p), lp.ctypes.data_as(C.c_void_p),
+                                                   batch_size, num_qo_heads, num_kv_heads, head_dim, page_size,
+                                                   split_tokens, num_compute_units, C.byref(fb), C.byref(ib)),
+              "Handler workspace")
+        return fb.value, ib.value
+
+    def host_schedule(self, which):
+        """numpy copy [records, ints] of one table of the last schedule (see bz_decode_plan_host_schedule)."""
+        data, n, k = C.c_void_p(), C.c_size_t(), C.c_uint32()
+        check(_lib.load().bz_decode_plan_host_schedule(self._h, which, C.byref(data), C.byref(n), C.byref(k)),
+              "Handler schedule")
+        if n.value == 0:
+            return np.zeros((0, max(k.value, 1)), np.int32)
+        buf = (C.c_int32 * (n.value * k.value)).from_address(data.value)
+        return np.frombuffer(buf, np.int32).reshape(n.value, k.value).copy()
+
     def set_timing_events(self, start=None, stop=None):
         """hipEvent_t handles recorded right before / after the decode kernel launch (None: off)."""
         check(_lib.load().bz_decode_plan_set_timing_events(self._h, start, stop), "Handler timing events")

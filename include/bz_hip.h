@@ -113,6 +113,25 @@ int bz_decode_plan(bz_decode_plan_t* plan, void* float_buffer, size_t float_buff
                    size_t int_buffer_bytes, const int32_t* indptr_h, const int32_t* last_page_len_h,
                    uint32_t batch_size, uint32_t num_qo_heads, uint32_t num_kv_heads, uint32_t head_dim,
                    uint32_t page_size, uint32_t split_tokens, void* stream);
+/* Workspace sizing (no counterpart in the reference, which fixes 128 MiB + 8 MiB, src/model/llama.h:111-112):
+ * runs the same host-side scheduling and reports how many bytes of the two workspaces bz_decode_plan would
+ * use for this batch with the matrix-core kernel where the shape allows it.  Touches no GPU when
+ * num_compute_units is given (0 = ask the current device).  The handle must be planned again before the
+ * next bz_batch_decode. */
+int bz_decode_plan_workspace(bz_decode_plan_t* plan, const int32_t* indptr_h, const int32_t* last_page_len_h,
+                             uint32_t batch_size, uint32_t num_qo_heads, uint32_t num_kv_heads, uint32_t head_dim,
+                             uint32_t page_size, uint32_t split_tokens, uint32_t num_compute_units,
+                             size_t* float_buffer_bytes, size_t* int_buffer_bytes);
+/* The host copy of the last schedule built by bz_decode_plan / bz_decode_plan_workspace, for tests and
+ * tools: records of ints_per_record int32 each, valid until the handle plans again.  which = 0: page-aligned
+ * segments of the general kernel {seq, page_begin, page_end, partial | -1}; 1: its split sequences {seq,
+ * first partial, count, 0}; 2: sequences without pages {seq}; 3: one record per 32-token tile of the
+ * matrix-core kernel, in processing order {position in indices[] of the page of tokens 32t.., of tokens
+ * 32t+16.., t, piece}; 4: wave-slot boundaries into those records; 5: pieces {seq, kv head, tile_begin,
+ * tile_end, partial | -1, combine index | -1, partials of its (seq, kv head), first of them, indptr[seq],
+ * pages, tokens, ...}; 6: split (seq, kv head)s {seq, kv head, first partial, count}. */
+int bz_decode_plan_host_schedule(const bz_decode_plan_t* plan, int which, const int32_t** data, size_t* num_records,
+                                 uint32_t* ints_per_record);
 /* introspection for tests and the bench: number of segments / of sequences that were split */
 int bz_decode_plan_info(const bz_decode_plan_t* plan, uint32_t* num_segments, uint32_t* num_split_seqs,
                         uint32_t* num_workgroups);

@@ -1,0 +1,160 @@
+"""CPU tests of the decode planner (the replacement of BlitzBatchDecodeHandler::plan,
+src/kernel/flashinfer_types.cu:52-80): the schedule is pure integer work on the host copies of indptr /
+last_page_len, so its invariants are checked here without a GPU through bz_decode_plan_workspace (which
+builds the same schedule for a stated number of compute units) and bz_decode_plan_host_schedule.
+
+What must hold for the kernels to be right: every 32-token tile of every (sequence, kv head) appears in
+exactly one record, in order inside its piece; the records point at the pages that hold the tile; the
+wave slots cover the records without gaps and evenly; a (sequence, kv head) cut into several pieces, or
+longer than split_tokens, gets distinct partial slots and one combine entry; the general kernel's
+segments tile every sequence's pages exactly once."""
+import numpy as np
+import pytest
+
+from blitz_scale_amd import kernel as K
+from blitz_scale_amd import workloads as wl
+
+CUS = 256
+
+
+def schedule(lens, Hq, Hkv, D, P, split_tokens=0, cus=CUS):
+    rng = np.random.default_rng(1)
+    lens = np.asarray(lens, np.int64)
+    need = int(((lens + P - 1) // P).sum())
+    indices, indptr, lpl = wl.page_table_for(lens, P, max(1, 2 * need), rng)
+    h = K.BlitzBatchDecodeHandler()
+    fb, ib = h.workspace(indptr, lpl, len(lens), Hq, Hkv, D, P, split_tokens=split_tokens, num_compute_units=cus)
+    names = ["segments", "combos", "empty", "tiles", "slot_ptr", "pieces", "mcombos"]
+    s = {n: h.host_schedule(i) for i, n in enumerate(names)}
+    s.update(indptr=np.asarray(indptr), lens=lens, float_bytes=fb, int_bytes=ib)
+    return s
+
+
+def check_mfma_schedule(s, Hkv, P, split_tokens):
+    lens, indptr = s["lens"], s["indptr"]
+    tiles, pieces, slot_ptr, mc = s["tiles"], s["pieces"], s["slot_ptr"][:, 0], s["mcombos"]
+    cap = 0x7FFFFFFF if split_tokens == 0xFFFFFFFF else max(1, (split_tokens or 2048) // 32)
+    # every tile exactly once, pointing at its pages
+    seen = set()
+    for idx0, idx1, t, pc in tiles:
+        seq, kvh, t0, t1 = pieces[pc][:4]
+        assert t0 <= t < t1
+        key = (seq, kvh, t)
+        assert key not in seen
+        seen.add(key)
+        npg = indptr[seq + 1] - indptr[seq]
+        assert idx0 == indptr[seq] + min((32 * t) // P, npg - 1)
+        assert idx1 == indptr[seq] + min((32 * t + 16) // P, npg - 1)
+    want = {(b, h, t) for b in range(len(lens)) for h in range(Hkv) for t in range((int(lens[b]) + 31) // 32)}
+    assert seen == want
+    # records of a piece are consecutive and ascending; pieces are in record order
+    pos = 0
+    for i, pc in enumerate(pieces):
+        seq, kvh, t0, t1, partial, combo, count, first, ip0, npg, seq_len = pc[:11]
+        assert t1 - t0 <= cap and t1 > t0
+        assert (ip0, npg, seq_len) == (indptr[seq], indptr[seq + 1] - indptr[seq], lens[seq])
+        block = tiles[pos:pos + (t1 - t0)]
+        assert (block[:, 3] == i).all() and (block[:, 2] == np.arange(t0, t1)).all()
+        pos += t1 - t0
+    assert pos == len(tiles)
+    # wave slots: monotone cover, no more than 8 per compute unit, even shares (within the odd/even skew + 1)
+    assert slot_ptr[0] == 0 and slot_ptr[-1] == len(tiles) and (np.diff(slot_ptr) >= 0).all()
+    shares = np.diff(slot_ptr)
+    assert len(shares) <= CUS * 8
+    if split_tokens != 0xFFFFFFFF and len(tiles) >= CUS * 8:
+        assert shares.min() >= 1 and shares.max() <= np.ceil(shares.mean() * 1.06) + 1
+    # partial slots and combine entries
+    by_unit = {}
+    for i, pc in enumerate(pieces):
+        by_unit.setdefault((pc[0], pc[1]), []).append(pc)
+    used = []
+    for (seq, kvh), pcs in by_unit.items():
+        assert [p[2] for p in pcs] == sorted(p[2] for p in pcs) and pcs[0][2] == 0
+        assert all(a[3] == b[2] for a, b in zip(pcs, pcs[1:])) and pcs[-1][3] == (int(lens[seq]) + 31) // 32
+        if len(pcs) == 1:
+            assert pcs[0][4] == -1
+        else:
+            first = pcs[0][7]
+            assert [p[4] for p in pcs] == list(range(first, first + len(pcs)))
+            assert all(p[6] == len(pcs) and p[7] == first for p in pcs)
+            c = mc[pcs[0][5]]
+            assert tuple(c) == (seq, kvh, first, len(pcs))
+            used.extend(p[4] for p in pcs)
+    assert sorted(used) == list(range(len(used))) and len(mc) == sum(len(v) > 1 for v in by_unit.values())
+
+
+def check_general_schedule(s, P):
+    lens, indptr = s["lens"], s["indptr"]
+    segs, combos, empty = s["segments"], s["combos"], s["empty"][:, 0]
+    assert sorted(empty) == [b for b in range(len(lens)) if lens[b] == 0]
+    cover = {}
+    for seq, lo, hi, partial in segs:
+        assert 0 <= lo < hi <= indptr[seq + 1] - indptr[seq]
+        cover.setdefault(seq, []).append((lo, hi, partial))
+    sizes = (segs[:, 2] - segs[:, 1])
+    assert (np.diff(sizes) <= 0).all()  # longest first
+    n_partials = 0
+    for seq, lst in cover.items():
+        lst.sort()
+        assert lst[0][0] == 0 and lst[-1][1] == indptr[seq + 1] - indptr[seq]
+        assert all(a[1] == b[0] for a, b in zip(lst, lst[1:]))
+        if len(lst) == 1:
+            assert lst[0][2] == -1
+        else:
+            c = [c for c in combos if c[0] == seq]
+            assert len(c) == 1 and c[0][2] == len(lst)
+            assert [x[2] for x in lst] == list(range(c[0][1], c[0][1] + len(lst)))
+            n_partials += len(lst)
+    assert set(cover) == {b for b in range(len(lens)) if lens[b] > 0}
+    assert len(combos) == sum(len(v) > 1 for v in cover.values())
+    return n_partials
+
+
+@pytest.mark.parametrize("name,lens,Hq,Hkv,P,split", [
+    ("headline", None, 32, 8, 16, 2048),                       # config 3: lognormal contexts, batch 128
+    ("page64", None, 32, 8, 64, 2048),
+    ("small_batch", [1024] * 8, 32, 8, 16, 2048),              # fewer tiles than wave slots
+    ("ragged", [0, 1, 31, 32, 33, 4097, 0, 700, 16, 17], 16, 2, 16, 256),
+    ("never_split", [5000, 40, 900], 8, 8, 16, 0xFFFFFFFF),
+    ("one_token", [1], 8, 1, 16, 0),
+    ("page48", [100, 1000, 47, 48, 49], 32, 8, 48, 512),      # page size not a power of two
+])
+def test_matrix_core_schedule_invariants(name, lens, Hq, Hkv, P, split):
+    if lens is None:
+        lens = wl.lognormal_ctx(np.random.default_rng(0x5EED), 128, 1024, 1.0, 64, 8192)
+    s = schedule(lens, Hq, Hkv, 128, P, split)
+    assert len(s["tiles"]) == sum((int(l) + 31) // 32 for l in lens) * Hkv
+    check_mfma_schedule(s, Hkv, P, split)
+    n_partials = check_general_schedule(s, P)
+    # reported workspace: the sections the kernels read, 256-byte aligned
+    al = lambda x: (x + 255) // 256 * 256
+    n_mp = int(s["mcombos"][:, 3].sum()) if len(s["mcombos"]) else 0  # partial slots of the matrix-core path
+    assert s["int_bytes"] == (al(len(s["segments"]) * 16) + al(len(s["combos"]) * 16) + al(len(s["empty"]) * 4) +
+                              al(len(s["pieces"]) * 64) + al((len(s["slot_ptr"]) - 1) * 48) +
+                              al(len(s["mcombos"]) * 16) + al(len(s["tiles"]) * 16))
+    assert s["float_bytes"] == max(al(n_partials * Hq * 128 * 4) + al(n_partials * Hq * 4),
+                                   al(n_mp * 16 * 128 * 4) + al(n_mp * 16 * 4))
+
+
+def test_shapes_outside_the_matrix_core_kernel_get_segments_only():
+    # config 1 of the baseline (head_dim 64): hand-checked segments; 4 sequences of 2, 4, 9, 16 pages
+    s = schedule([17, 64, 130, 255], 4, 4, 64, 16, split_tokens=0)
+    assert len(s["tiles"]) == 0 and len(s["pieces"]) == 0
+    check_general_schedule(s, 16)
+    # 31 pages over 4 sequences is far fewer items than 4 per compute unit: pieces shrink to 256 tokens = 16 pages,
+    # so nothing is cut here
+    assert sorted(map(tuple, s["segments"][:, :3])) == [(0, 0, 2), (1, 0, 4), (2, 0, 9), (3, 0, 16)]
+    assert (s["segments"][:, 3] == -1).all() and s["float_bytes"] == 0
+    # a long sequence at the same shape is cut into equal page-aligned pieces with one combine entry
+    s = schedule([4096], 4, 4, 64, 16, split_tokens=1024)
+    segs = s["segments"]
+    assert len(segs) == 16 and (segs[:, 2] - segs[:, 1] == 16).all() and sorted(segs[:, 3]) == list(range(16))
+    assert [tuple(c) for c in s["combos"]] == [(0, 0, 16, 0)]
+
+
+def test_fewer_compute_units_mean_fewer_longer_shares():
+    lens = [2048] * 64
+    a = schedule(lens, 32, 8, 128, 16, 2048, cus=256)
+    b = schedule(lens, 32, 8, 128, 16, 2048, cus=64)
+    assert len(a["slot_ptr"]) - 1 == 2048 and len(b["slot_ptr"]) - 1 == 512
+    assert np.diff(b["slot_ptr"][:, 0]).mean() == pytest.approx(4 * np.diff(a["slot_ptr"][:, 0]).mean())

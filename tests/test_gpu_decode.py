@@ -161,3 +161,24 @@ def test_error_codes():
     with pytest.raises(K.BzError, match="Handler plan"):
         dev.handler.plan(dev.float_ws, dev.float_ws.numel(), dev.int_ws, 16, p.indptr, p.last_page_len, p.B, p.Hq,
                          p.Hkv, p.D, p.P)  # int workspace too small
+
+
+def test_plan_fits_the_workspace_it_reports():
+    """bz_decode_plan_workspace names the bytes plan() needs for the matrix-core kernel: buffers of exactly
+    that size are enough, one section less and the plan falls back to the general kernel (same results)."""
+    from blitz_scale_amd import kernel as K
+    p = DecodeProblem(77, [3000, 40, 900, 2100, 64, 1], 32, 8, 128, 16, BZ_BF16)
+    ref = oracle.batch_decode(p.q, p.dtype, p.oracle_kv(), p.Hq)
+    h = K.BlitzBatchDecodeHandler()
+    fb, ib = h.workspace(p.indptr, p.last_page_len, p.B, p.Hq, p.Hkv, p.D, p.P, split_tokens=1024)
+    slots = len(h.host_schedule(4)) - 1
+    assert fb > 0 and ib > 0 and slots > 0
+    infos = []
+    for int_bytes in (ib, ib - 256):
+        dev = DeviceDecode(p, float_ws_bytes=fb, int_ws_bytes=int_bytes)
+        info = dev.plan(1024)
+        got = dev.decode(None, BZ_ROPE_NONE)
+        assert (np.abs(got - ref) <= ulp_tol(ref, p.dtype)).all()
+        infos.append(info)
+    assert infos[0]["workgroups"] == slots          # the matrix-core schedule was taken
+    assert infos[1]["workgroups"] != slots          # no room for it: page-aligned segments x kv heads
