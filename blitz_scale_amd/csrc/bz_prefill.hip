@@ -11,6 +11,7 @@
 // rescaling of O and the P operand of the second contraction are all lane-local (one shuffle per
 // tile joins the two half-waves).
 #include <algorithm>
+#include <atomic>
 #include <cmath>
 #include <cstdio>
 #include <cstdlib>
@@ -72,6 +73,7 @@ struct PrefillPlan {
     uint32_t batch_size = 0, num_qo_heads = 0, num_kv_heads = 0, head_dim = 0, num_items = 0;
     uint32_t total_tokens = 0;
     const PrefillItem* items_d = nullptr;
+    std::vector<PrefillItem> h_items; // host copy of the last job list (kept between calls)
     void* staging = nullptr;
     size_t staging_bytes = 0;
     hipEvent_t upload_done = nullptr;
@@ -445,13 +447,10 @@ extern "C" void bz_prefill_plan_destroy(bz_prefill_plan_t* plan_) {
     delete p;
 }
 
-extern "C" int bz_prefill_plan(bz_prefill_plan_t* plan_, void* float_buffer, size_t float_buffer_bytes,
-                               void* int_buffer, size_t int_buffer_bytes, const int32_t* qo_indptr_h,
-                               const int32_t* kv_indptr_h, uint32_t batch_size, uint32_t num_qo_heads,
-                               uint32_t num_kv_heads, uint32_t head_dim, uint32_t page_size, void* stream) {
-    (void)float_buffer; (void)float_buffer_bytes; (void)page_size;
-    PrefillPlan* p = reinterpret_cast<PrefillPlan*>(plan_);
-    if (!p || !qo_indptr_h || !kv_indptr_h || !int_buffer) return BZ_ERR_BAD_ARG;
+// Pure host work: the job list of a ragged batch into p->h_items.
+static int build_prefill_items(PrefillPlan* p, const int32_t* qo_indptr_h, const int32_t* kv_indptr_h,
+                               uint32_t batch_size, uint32_t num_qo_heads, uint32_t num_kv_heads, uint32_t head_dim) {
+    if (!p || !qo_indptr_h || !kv_indptr_h) return BZ_ERR_BAD_ARG;
     if (num_kv_heads == 0 || num_qo_heads % num_kv_heads) return BZ_ERR_BAD_ARG;
     p->planned = false;
     if (head_dim != 128) return BZ_ERR_UNSUPPORTED;
@@ -484,9 +483,44 @@ extern "C" int bz_prefill_plan(bz_prefill_plan_t* plan_, void* float_buffer, siz
     }
     size_t longest = 0;
     for (auto& v : per_xcd) longest = std::max(longest, v.size());
-    std::vector<PrefillItem> items(longest * kXcd, PrefillItem{0, 0, 0, 0});
+    std::vector<PrefillItem>& items = p->h_items;
+    items.assign(longest * kXcd, PrefillItem{0, 0, 0, 0});
     for (int x = 0; x < kXcd; ++x)
         for (size_t k = 0; k < per_xcd[x].size(); ++k) items[k * kXcd + x] = per_xcd[x][k];
+    return 0;
+}
+
+extern "C" int bz_prefill_plan_workspace(bz_prefill_plan_t* plan_, const int32_t* qo_indptr_h, const int32_t* kv_indptr_h,
+                                         uint32_t batch_size, uint32_t num_qo_heads, uint32_t num_kv_heads,
+                                         uint32_t head_dim, size_t* float_buffer_bytes, size_t* int_buffer_bytes) {
+    PrefillPlan* p = reinterpret_cast<PrefillPlan*>(plan_);
+    const int rc = build_prefill_items(p, qo_indptr_h, kv_indptr_h, batch_size, num_qo_heads, num_kv_heads, head_dim);
+    if (rc) return rc;
+    if (float_buffer_bytes) *float_buffer_bytes = 0;
+    if (int_buffer_bytes) *int_buffer_bytes = pf_align_up(p->h_items.size() * sizeof(PrefillItem), 256);
+    return 0;
+}
+
+extern "C" int bz_prefill_plan_host_schedule(const bz_prefill_plan_t* plan_, const int32_t** data, size_t* num_records,
+                                             uint32_t* ints_per_record) {
+    const PrefillPlan* p = reinterpret_cast<const PrefillPlan*>(plan_);
+    if (!p || !data || !num_records || !ints_per_record) return BZ_ERR_BAD_ARG;
+    *data = (const int32_t*)p->h_items.data();
+    *num_records = p->h_items.size();
+    *ints_per_record = sizeof(PrefillItem) / 4;
+    return 0;
+}
+
+extern "C" int bz_prefill_plan(bz_prefill_plan_t* plan_, void* float_buffer, size_t float_buffer_bytes,
+                               void* int_buffer, size_t int_buffer_bytes, const int32_t* qo_indptr_h,
+                               const int32_t* kv_indptr_h, uint32_t batch_size, uint32_t num_qo_heads,
+                               uint32_t num_kv_heads, uint32_t head_dim, uint32_t page_size, void* stream) {
+    (void)float_buffer; (void)float_buffer_bytes; (void)page_size;
+    PrefillPlan* p = reinterpret_cast<PrefillPlan*>(plan_);
+    if (!p || !int_buffer) return BZ_ERR_BAD_ARG;
+    const int rc0 = build_prefill_items(p, qo_indptr_h, kv_indptr_h, batch_size, num_qo_heads, num_kv_heads, head_dim);
+    if (rc0) return rc0;
+    const std::vector<PrefillItem>& items = p->h_items;
     const size_t bytes = pf_align_up(items.size() * sizeof(PrefillItem), 256);
     if (bytes > int_buffer_bytes) return BZ_ERR_WORKSPACE;
     hipStream_t s = (hipStream_t)stream;
@@ -520,10 +554,14 @@ static int launch_prefill(const PrefillPlan* p, const PrefillArgs& a, const void
                           hipStream_t s) {
     const size_t smem = 4 * (size_t)kTile;
     auto kern = prefill_kernel<BF16, SPLIT_P>;
-    static bool attr_done = false; // raising the dynamic LDS limit is idempotent; a repeated call is harmless
-    if (!attr_done) {
+    // raising the dynamic LDS limit: once per device (idempotent, so a race between two host threads is harmless)
+    static std::atomic<uint64_t> attr_done{0};
+    int dev = 0;
+    BZ_CHECK_HIP(hipGetDevice(&dev));
+    const uint64_t bit = 1ull << (dev & 63);
+    if (!(attr_done.load(std::memory_order_relaxed) & bit)) {
         BZ_CHECK_HIP(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
-        attr_done = true;
+        attr_done.fetch_or(bit, std::memory_order_relaxed);
     }
     hipLaunchKernelGGL(kern, dim3(p->num_items), dim3(256), smem, s, a, (const char*)q, (const char*)k,
                        (const char*)v);

@@ -191,6 +191,26 @@ class BatchPrefillRaggedHandler:
         check(rc, "Handler plan")
         self._keep = (float_buffer, int_buffer)
 
+    def workspace(self, qo_indptr_h, kv_indptr_h, batch_size, num_qo_heads, num_kv_heads, head_dim):
+        """(float_buffer_bytes, int_buffer_bytes) plan() would use; host only."""
+        qo, kv = _host_i32(qo_indptr_h), _host_i32(kv_indptr_h)
+        fb, ib = C.c_size_t(), C.c_size_t()
+        check(_lib.load().bz_prefill_plan_workspace(self._h, qo.ctypes.data_as(C.c_void_p),
+                                                    kv.ctypes.data_as(C.c_void_p), batch_size, num_qo_heads,
+                                                    num_kv_heads, head_dim, C.byref(fb), C.byref(ib)),
+              "Handler workspace")
+        return fb.value, ib.value
+
+    def host_schedule(self):
+        """numpy copy [workgroups, 4] of the last job list: tok0, len (0 = padding), q0, head."""
+        data, n, k = C.c_void_p(), C.c_size_t(), C.c_uint32()
+        check(_lib.load().bz_prefill_plan_host_schedule(self._h, C.byref(data), C.byref(n), C.byref(k)),
+              "Handler schedule")
+        if n.value == 0:
+            return np.zeros((0, 4), np.int32)
+        buf = (C.c_int32 * (n.value * k.value)).from_address(data.value)
+        return np.frombuffer(buf, np.int32).reshape(n.value, k.value).copy()
+
     def __del__(self):
         try:
             if self._h:

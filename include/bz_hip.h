@@ -166,6 +166,16 @@ int bz_prefill_plan(bz_prefill_plan_t* plan, void* float_buffer, size_t float_bu
                     uint32_t batch_size, uint32_t num_qo_heads, uint32_t num_kv_heads, uint32_t head_dim,
                     uint32_t page_size, void* stream);
 
+/* Host-only counterparts of bz_decode_plan_workspace / bz_decode_plan_host_schedule for the prefill plan:
+ * the bytes of int_buffer the job list of this batch takes (the float workspace is not used), and the
+ * host copy of the list, one record per workgroup in launch order {first token of the request, tokens of
+ * the request (0 = padding entry), first q row of the tile inside the request, q head}.  No GPU call. */
+int bz_prefill_plan_workspace(bz_prefill_plan_t* plan, const int32_t* qo_indptr_h, const int32_t* kv_indptr_h,
+                              uint32_t batch_size, uint32_t num_qo_heads, uint32_t num_kv_heads, uint32_t head_dim,
+                              size_t* float_buffer_bytes, size_t* int_buffer_bytes);
+int bz_prefill_plan_host_schedule(const bz_prefill_plan_t* plan, const int32_t** data, size_t* num_records,
+                                  uint32_t* ints_per_record);
+
 /*
  * batch_prefill_attention (src/kernel/attention.h:9-22, attention_prefill.cu:11-46): ragged
  * self-attention, q [N,Hq,D], k,v [N,Hkv,D], out [N,Hq,D], qo_indptr == kv_indptr (the only

@@ -158,3 +158,54 @@ def test_fewer_compute_units_mean_fewer_longer_shares():
     b = schedule(lens, 32, 8, 128, 16, 2048, cus=64)
     assert len(a["slot_ptr"]) - 1 == 2048 and len(b["slot_ptr"]) - 1 == 512
     assert np.diff(b["slot_ptr"][:, 0]).mean() == pytest.approx(4 * np.diff(a["slot_ptr"][:, 0]).mean())
+
+
+@pytest.mark.parametrize("lens,Hq,Hkv", [
+    ([20, 37], 4, 2),
+    ([128, 129, 1, 4096, 0, 640], 8, 8),
+    (None, 40, 40),  # config 4: 16 prompts U[128, 4096], 40 heads
+])
+def test_prefill_job_list_invariants(lens, Hq, Hkv):
+    """The prefill plan (replacement of BatchPrefillRaggedHandler::plan, src/kernel/flashinfer_types.cu:24-49):
+    one job per (request, q head, 128-row q tile), each exactly once; the jobs of a (request, head) pair sit
+    in one column of the 8-wide launch order (one XCD, consecutive there), last tile first; longer requests
+    come first; padding entries have length 0."""
+    if lens is None:
+        lens = np.random.default_rng(0x5EED).integers(128, 4097, 16)
+    lens = np.asarray(lens, np.int64)
+    indptr = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+    h = K.BatchPrefillRaggedHandler()
+    fb, ib = h.workspace(indptr, indptr, len(lens), Hq, Hkv, 128)
+    items = h.host_schedule()
+    assert fb == 0 and ib == (len(items) * 16 + 255) // 256 * 256 and len(items) % 8 == 0
+    tok0_to_req = {int(indptr[b]): b for b in range(len(lens)) if lens[b] > 0}
+    seen, column, last_q0 = set(), {}, {}
+    first_seen_len = []
+    for i, (tok0, ln, q0, head) in enumerate(items):
+        if ln == 0:
+            continue
+        b = tok0_to_req[int(tok0)]
+        assert ln == lens[b] and q0 % 128 == 0 and 0 <= q0 < ln and 0 <= head < Hq
+        key = (b, int(head), int(q0))
+        assert key not in seen
+        seen.add(key)
+        pair = (b, int(head))
+        assert column.setdefault(pair, i % 8) == i % 8
+        if pair in last_q0:
+            assert q0 == last_q0[pair] - 128  # consecutive in its column, most keys first
+        else:
+            first_seen_len.append(int(ln))
+        last_q0[pair] = int(q0)
+    want = {(b, hd, q0) for b in range(len(lens)) for hd in range(Hq) for q0 in range(0, int(lens[b]), 128)}
+    assert seen == want
+    assert all(v == 0 for v in last_q0.values())
+    # pairs are dealt to the columns in turn, longest requests first: within one column lengths never grow
+    for c in range(8):
+        col = [int(ln) for (tok0, ln, q0, head) in items[c::8] if ln > 0]
+        assert all(a >= b for a, b in zip(col, col[1:]))
+    # no column holds more than its share of pairs + 1
+    per_col = np.bincount(list(column.values()), minlength=8)
+    assert per_col.max() - per_col.min() <= 1
+    # a head size the kernel does not cover is refused on the host
+    with pytest.raises(K.BzError):
+        h.workspace(indptr, indptr, len(lens), Hq, Hkv, 64)
