@@ -115,7 +115,7 @@ static int build_schedule(DecodePlan* p, const int32_t* indptr_h, const int32_t*
     // piece, or is longer than split_tokens, is folded from partial results.  Every tile of a share
     // gets a 16-byte record so that the kernel never has to chase the piece list tile by tile.
     std::vector<MfmaPiece>& mp = p->h_pieces;
-    std::vector<MfmaTile>& mt = p->h_tiles;
+    RawArray<MfmaTile>& mt = p->h_tiles;
     std::vector<int32_t>& mptr = p->h_slot_ptr; // tiles of slot s: [mptr[s], mptr[s+1]); uploaded as one MfmaSlotHead per slot
     std::vector<MfmaCombine>& mc = p->h_mcombos;
     mp.clear(); mt.clear(); mptr.clear(); mc.clear();
@@ -145,15 +145,17 @@ static int build_schedule(DecodePlan* p, const int32_t* indptr_h, const int32_t*
         auto slot_weight = [&](uint64_t s) { return (s & 1) ? 1.0 - skew / 2 : 1.0 + skew / 2; };
         double wsum = 0.0;
         for (uint64_t s2 = 0; s2 < nslots; ++s2) wsum += slot_weight(s2);
-        uint64_t slot = 0;
+        const double tiles_per_weight = wsum > 0.0 ? (double)total_tiles / wsum : 0.0;
+        uint64_t slot = 0, bound_lo = 0; // bound_lo: rounded running boundary where the current slot starts
         double wacc = slot_weight(0);
         auto slot_share = [&](void) { // tiles of the current slot: difference of rounded running boundaries
-            const uint64_t hi = (slot + 1 >= nslots) ? total_tiles : (uint64_t)((double)total_tiles * wacc / wsum + 0.5);
-            const uint64_t lo = (uint64_t)((double)total_tiles * (wacc - slot_weight(slot)) / wsum + 0.5);
+            const uint64_t hi = (slot + 1 >= nslots) ? total_tiles : (uint64_t)(wacc * tiles_per_weight + 0.5);
+            const uint64_t lo = bound_lo;
+            bound_lo = hi;
             return std::max<uint64_t>(1, hi > lo ? hi - lo : 1);
         };
         uint64_t room = slot_share(); // tiles the current slot can still take
-        mt.resize(total_tiles); // sized once (records are written in place below)
+        mt.resize_uninitialized(total_tiles); // sized once; every record is written below
         size_t n_rec = 0;
         mptr.push_back(0);
         for (uint32_t b = 0; b < batch_size; ++b) {
@@ -181,7 +183,16 @@ static int build_schedule(DecodePlan* p, const int32_t* indptr_h, const int32_t*
                     n_rec += (size_t)take;
                     const int32_t piece_id = (int32_t)mp.size(), ip0 = indptr_h[b];
                     if (page_shift >= 0) {
-                        for (int32_t tt = t; tt < t + take; ++tt, ++rec) {
+                        // tiles whose second half still lies inside the table need no clamping: plain
+                        // 32-bit shifts the compiler can vectorise; the (at most one) tile after them is clamped
+                        const int64_t cap_tok = ((int64_t)np << page_shift) - 17;
+                        const int32_t fast_end = cap_tok < 0 ? t : (int32_t)std::min<int64_t>(t + take, cap_tok / 32 + 1);
+                        int32_t tt = t;
+                        if ((int64_t)(t + take) * 32 + 16 < 0x7fffffffLL) {
+                            for (; tt < fast_end; ++tt, ++rec)
+                                *rec = {ip0 + ((tt << 5) >> page_shift), ip0 + (((tt << 5) + 16) >> page_shift), tt, piece_id};
+                        }
+                        for (; tt < t + take; ++tt, ++rec) {
                             const int32_t pg0 = std::min<int32_t>((int32_t)(((int64_t)tt * 32) >> page_shift), np - 1);
                             const int32_t pg1 = std::min<int32_t>((int32_t)(((int64_t)tt * 32 + 16) >> page_shift), np - 1);
                             *rec = {ip0 + pg0, ip0 + pg1, tt, piece_id};
@@ -258,7 +269,7 @@ extern "C" int bz_decode_plan(bz_decode_plan_t* plan_, void* float_buffer, size_
     const std::vector<DecodeCombine>& combos = p->h_combos;
     const std::vector<int32_t>& empty = p->h_empty;
     const std::vector<MfmaPiece>& mp = p->h_pieces;
-    const std::vector<MfmaTile>& mt = p->h_tiles;
+    const RawArray<MfmaTile>& mt = p->h_tiles;
     const std::vector<int32_t>& mptr = p->h_slot_ptr;
     const std::vector<MfmaCombine>& mc = p->h_mcombos;
     const uint32_t partials = counts.partials, mfma_partials = counts.mfma_partials;

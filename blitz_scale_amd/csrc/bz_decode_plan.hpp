@@ -2,6 +2,7 @@
 #pragma once
 #include <hip/hip_runtime.h>
 #include <stdint.h>
+#include <new>
 #include <vector>
 
 namespace bz {
@@ -50,6 +51,32 @@ struct MfmaSlotHead {
     int32_t pad;
 };
 
+// Growable array of plain records that does not clear what it hands out (the planner overwrites every
+// record it counts).
+template <typename T> struct RawArray {
+    T* ptr = nullptr;
+    size_t n = 0, cap = 0;
+    RawArray() = default;
+    RawArray(const RawArray&) = delete;
+    RawArray& operator=(const RawArray&) = delete;
+    ~RawArray() { ::operator delete(ptr); }
+    void resize_uninitialized(size_t count) {
+        if (count > cap) {
+            ::operator delete(ptr);
+            cap = count + count / 2 + 64;
+            ptr = static_cast<T*>(::operator new(cap * sizeof(T)));
+        }
+        n = count;
+    }
+    void clear() { n = 0; }
+    size_t size() const { return n; }
+    bool empty() const { return n == 0; }
+    T* data() { return ptr; }
+    const T* data() const { return ptr; }
+    T& operator[](size_t i) { return ptr[i]; }
+    const T& operator[](size_t i) const { return ptr[i]; }
+};
+
 // One split (sequence, kv head): partial slots [first, first+count).
 struct MfmaCombine {
     int32_t seq, kvh, first, count;
@@ -82,7 +109,7 @@ struct DecodePlan {
     std::vector<DecodeCombine> h_combos;
     std::vector<int32_t> h_empty, h_slot_ptr;
     std::vector<MfmaPiece> h_pieces;
-    std::vector<MfmaTile> h_tiles;
+    RawArray<MfmaTile> h_tiles;
     std::vector<MfmaCombine> h_mcombos;
     // pinned staging for the schedule upload and the event that guards its reuse
     void* staging = nullptr;
