@@ -37,12 +37,15 @@ __device__ __forceinline__ float to_f32(bf16_t v) { return __uint_as_float((uint
 __device__ __forceinline__ float to_f32(float v) { return v; }
 
 __device__ __forceinline__ uint16_t f32_to_f16_bits(float f) { return __half_as_ushort(__float2half_rn(f)); }
-__device__ __forceinline__ uint16_t f32_to_bf16_bits(float f) {
-    uint32_t u = __float_as_uint(f);
-    if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x40u);
-    u += 0x7fffu + ((u >> 16) & 1u);
-    return (uint16_t)(u >> 16);
+// fp32 -> bf16, round to nearest even, on the conversion unit of gfx950 (v_cvt_pk_bf16_f32: two values per
+// instruction; the bit-twiddled form costs six vector instructions per value)
+typedef __attribute__((ext_vector_type(2))) __bf16 bz_bf16x2_t;
+typedef __attribute__((ext_vector_type(2))) float bz_f32x2_t;
+__device__ __forceinline__ uint32_t f32x2_to_bf16x2_bits(float lo, float hi) {
+    const bz_f32x2_t v = {lo, hi};
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bz_bf16x2_t));
 }
+__device__ __forceinline__ uint16_t f32_to_bf16_bits(float f) { return (uint16_t)(f32x2_to_bf16x2_bits(f, 0.f) & 0xffffu); }
 
 // One rotate-half pair: (x, y) -> (x c - y s, y c + x s).  Every product and sum is rounded on its own
 // (no fused multiply-add), so that all kernels of the library that rotate the same row get the same
@@ -140,7 +143,7 @@ template <> struct Vec8<bf16_t> {
         uint32_t w[4];
 #pragma unroll
         for (int i = 0; i < 4; ++i)
-            w[i] = (uint32_t)f32_to_bf16_bits(f[2 * i]) | ((uint32_t)f32_to_bf16_bits(f[2 * i + 1]) << 16);
+            w[i] = f32x2_to_bf16x2_bits(f[2 * i], f[2 * i + 1]);
         raw = make_uint4(w[0], w[1], w[2], w[3]);
     }
 };

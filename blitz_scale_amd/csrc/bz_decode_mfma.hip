@@ -58,7 +58,7 @@ template <> struct Mma<true> {
                                                        c, 0, 0, 0);
     }
     __device__ static __forceinline__ uint32_t pack2(float lo, float hi) {
-        return (uint32_t)f32_to_bf16_bits(lo) | ((uint32_t)f32_to_bf16_bits(hi) << 16);
+        return f32x2_to_bf16x2_bits(lo, hi);
     }
     __device__ static __forceinline__ float unpack_lo(uint32_t w) { return __uint_as_float(w << 16); }
     __device__ static __forceinline__ float unpack_hi(uint32_t w) { return __uint_as_float(w & 0xffff0000u); }
