@@ -294,7 +294,8 @@ __global__ __launch_bounds__(64, 2) void decode_mfma_kernel(MfmaDecodeArgs a, co
         if (i == 8 && chunk_base + 32 < g_end) dnext = fetch_info(chunk_base + 32);
         if (i == 24 && chunk_base + 32 < g_end) { stash_info(dnext, buf ^ 1); wave_lds_sync(); }
         const int t = uc.t, tok_end = uc.tok_end, seq_len = uc.seq_len;
-        const float score_scale = a.sm_scale_log2 * ((KV8 && a.k_scale) ? a.k_scale[uc.kvh] : 1.0f);
+        // (positive; the floor keeps masked scores at -inf instead of NaN should a head's K scale be zero)
+        const float score_scale = fmaxf(a.sm_scale_log2 * ((KV8 && a.k_scale) ? a.k_scale[uc.kvh] : 1.0f), 1e-30f);
 
         if (uc.flags & 1) { // ================= first tile of a piece =================
 #pragma unroll
@@ -340,22 +341,40 @@ __global__ __launch_bounds__(64, 2) void decode_mfma_kernel(MfmaDecodeArgs a, co
         const int tile_tok0 = t * kTileTok;
         const bool ragged = tile_tok0 + kTileTok > tok_end; // wave-uniform
         wave_lds_sync(); // transposed reads of the previous tile come before V is overwritten
+        // (the masked variant sits behind a wave-uniform branch: written as one predicated sequence it costs
+        // eight register moves and an exec-mask round trip per row on every tile, between the arrival of a
+        // tile and the next loads)
         if constexpr (KV8) {
+            if (!ragged) {
 #pragma unroll
-            for (int w = 0; w < 4; ++w) { // 16 e4m3 bytes -> 16 operand-type values -> 32 B of the LDS row
-                uint4 v = vreg[w];
-                const int row = 8 * w + (lane >> 3);
-                if (ragged && tile_tok0 + row >= tok_end) v = make_uint4(0, 0, 0, 0); // 0 * garbage must be 0
-                unsigned char* dst = v_lds + row * kVRowBytes + (lane & 7) * 32;
-                *reinterpret_cast<uint4*>(dst) = fp8x8_to_op<BF16>(v, 0);
-                *reinterpret_cast<uint4*>(dst + 16) = fp8x8_to_op<BF16>(v, 1);
+                for (int w = 0; w < 4; ++w) { // 16 e4m3 bytes -> 16 operand-type values -> 32 B of the LDS row
+                    unsigned char* dst = v_lds + (8 * w + (lane >> 3)) * kVRowBytes + (lane & 7) * 32;
+                    *reinterpret_cast<uint4*>(dst) = fp8x8_to_op<BF16>(vreg[w], 0);
+                    *reinterpret_cast<uint4*>(dst + 16) = fp8x8_to_op<BF16>(vreg[w], 1);
+                }
+            } else {
+#pragma unroll
+                for (int w = 0; w < 4; ++w) {
+                    uint4 v = vreg[w];
+                    const int row = 8 * w + (lane >> 3);
+                    if (tile_tok0 + row >= tok_end) v = make_uint4(0, 0, 0, 0); // 0 * garbage must be 0
+                    unsigned char* dst = v_lds + row * kVRowBytes + (lane & 7) * 32;
+                    *reinterpret_cast<uint4*>(dst) = fp8x8_to_op<BF16>(v, 0);
+                    *reinterpret_cast<uint4*>(dst + 16) = fp8x8_to_op<BF16>(v, 1);
+                }
             }
         } else {
+            if (!ragged) {
 #pragma unroll
-            for (int w = 0; w < 8; ++w) {
-                uint4 v = vreg[w];
-                if (ragged && tile_tok0 + 4 * w + j >= tok_end) v = make_uint4(0, 0, 0, 0); // 0 * garbage must be 0
-                *reinterpret_cast<uint4*>(v_lds + (4 * w + j) * kVRowBytes + n * 16) = v;
+                for (int w = 0; w < 8; ++w)
+                    *reinterpret_cast<uint4*>(v_lds + (4 * w + j) * kVRowBytes + n * 16) = vreg[w];
+            } else {
+#pragma unroll
+                for (int w = 0; w < 8; ++w) {
+                    uint4 v = vreg[w];
+                    if (tile_tok0 + 4 * w + j >= tok_end) v = make_uint4(0, 0, 0, 0); // 0 * garbage must be 0
+                    *reinterpret_cast<uint4*>(v_lds + (4 * w + j) * kVRowBytes + n * 16) = v;
+                }
             }
         }
         uint4 kcur[2][4];
@@ -383,21 +402,22 @@ __global__ __launch_bounds__(64, 2) void decode_mfma_kernel(MfmaDecodeArgs a, co
                 for (int ks = 0; ks < 4; ++ks) s[u] = M::run(kcur[u][ks], qlo[ks], s[u]);
             }
         }
-        float tmax = -INFINITY;
+        if (ragged) { // wave-uniform
 #pragma unroll
-        for (int u = 0; u < 2; ++u)
+            for (int u = 0; u < 2; ++u)
 #pragma unroll
-            for (int r = 0; r < 4; ++r) {
-                float v = s[u][r] * score_scale;
-                if (ragged && tile_tok0 + 16 * u + 4 * j + r >= tok_end) v = -INFINITY;
-                s[u][r] = v;
-                tmax = fmaxf(tmax, v);
-            }
-        tmax = lane_max_xor32(lane_max_xor16(tmax));
+                for (int r = 0; r < 4; ++r)
+                    if (tile_tok0 + 16 * u + 4 * j + r >= tok_end) s[u][r] = -INFINITY;
+        }
+        float tmax = fmaxf(fmaxf(fmaxf(s[0][0], s[0][1]), fmaxf(s[0][2], s[0][3])),
+                           fmaxf(fmaxf(s[1][0], s[1][1]), fmaxf(s[1][2], s[1][3])));
+        // the scores stay unscaled in registers: the scale is applied to the maximum here and to every
+        // score inside the fused multiply-add that feeds exp2
+        tmax = lane_max_xor32(lane_max_xor16(tmax)) * score_scale;
         // finite also for a tile without live tokens (one past the present end under a table that runs
         // ahead): its probabilities and alpha come out 0 instead of NaN
         const float m_new = fmaxf(fmaxf(m_run, tmax), -1e30f);
-        const float alpha = exp2f(m_run - m_new); // 0 on the first tile (m_run = -inf)
+        const float alpha = __builtin_amdgcn_exp2f(m_run - m_new); // 0 on the first tile (m_run = -inf)
         // The probabilities enter the second contraction as a storage-precision head plus tail
         // (p = hi + lo, two MFMAs per block): the matrix cores cost nothing here and the result
         // keeps fp32-level accuracy instead of the 8 to 11 bits of a single rounded operand.
@@ -405,8 +425,10 @@ __global__ __launch_bounds__(64, 2) void decode_mfma_kernel(MfmaDecodeArgs a, co
         uint4 pa, pb;
 #pragma unroll
         for (int u = 0; u < 2; ++u) {
-            const float p0 = exp2f(s[u][0] - m_new), p1 = exp2f(s[u][1] - m_new);
-            const float p2 = exp2f(s[u][2] - m_new), p3 = exp2f(s[u][3] - m_new);
+            const float p0 = __builtin_amdgcn_exp2f(fmaf(s[u][0], score_scale, -m_new));
+            const float p1 = __builtin_amdgcn_exp2f(fmaf(s[u][1], score_scale, -m_new));
+            const float p2 = __builtin_amdgcn_exp2f(fmaf(s[u][2], score_scale, -m_new));
+            const float p3 = __builtin_amdgcn_exp2f(fmaf(s[u][3], score_scale, -m_new));
             psum += (p0 + p1) + (p2 + p3);
             const uint32_t h01 = M::pack2(p0, p1), h23 = M::pack2(p2, p3);
             u4(pa, 2 * u) = h01;
