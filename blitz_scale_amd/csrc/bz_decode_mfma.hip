@@ -377,18 +377,24 @@ __global__ __launch_bounds__(64, 2) void decode_mfma_kernel(MfmaDecodeArgs a, co
                 }
             }
         }
-        uint4 kcur[2][4];
-#pragma unroll
-        for (int u = 0; u < 2; ++u)
-#pragma unroll
-            for (int ks = 0; ks < 4; ++ks) {
-                if constexpr (KV8) kcur[u][ks] = fp8x8_to_op<BF16>(kreg[u][ks >> 1], ks & 1);
-                else kcur[u][ks] = kreg[u][ks];
+        // 16-bit pools: the K rows are contracted straight out of their landing registers and the next
+        // tile's loads go out right behind the eight score instructions (which have read their operands
+        // by then); e4m3 pools: the rows are widened into operand registers first, which frees the landing
+        // registers, so the loads go out before the contraction.
+        auto issue_next = [&]() {
+            if (g + 1 < g_end) {
+                if (i + 1 == 32) { chunk_base += 32; buf ^= 1; }
+                if (un.flags & 1) issue_q(un); // next tile opens a new piece
+                issue_loads(nb);
             }
-        if (g + 1 < g_end) {
-            if (i + 1 == 32) { chunk_base += 32; buf ^= 1; }
-            if (un.flags & 1) issue_q(un); // next tile opens a new piece
-            issue_loads(nb);
+        };
+        uint4 kcur[2][4];
+        if constexpr (KV8) {
+#pragma unroll
+            for (int u = 0; u < 2; ++u)
+#pragma unroll
+                for (int ks = 0; ks < 4; ++ks) kcur[u][ks] = fp8x8_to_op<BF16>(kreg[u][ks >> 1], ks & 1);
+            issue_next();
         }
         // ---- scores: S^T[token][head], lane (head n, group j) gets tokens 16u + 4j + r
         f32x4_t s[2];
@@ -396,11 +402,15 @@ __global__ __launch_bounds__(64, 2) void decode_mfma_kernel(MfmaDecodeArgs a, co
         for (int u = 0; u < 2; ++u) {
             s[u] = f32x4_t{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-            for (int ks = 0; ks < 4; ++ks) s[u] = M::run(kcur[u][ks], qhi[ks], s[u]);
+            for (int ks = 0; ks < 4; ++ks) s[u] = M::run(KV8 ? kcur[u][ks] : kreg[u][ks], qhi[ks], s[u]);
             if (ROPE_Q) {
 #pragma unroll
-                for (int ks = 0; ks < 4; ++ks) s[u] = M::run(kcur[u][ks], qlo[ks], s[u]);
+                for (int ks = 0; ks < 4; ++ks) s[u] = M::run(KV8 ? kcur[u][ks] : kreg[u][ks], qlo[ks], s[u]);
             }
+        }
+        if constexpr (!KV8) {
+            __builtin_amdgcn_sched_barrier(0); // the loads below overwrite the operands of the instructions above
+            issue_next();
         }
         if (ragged) { // wave-uniform
 #pragma unroll
