@@ -83,15 +83,20 @@ template <> struct Mma<false> {
 __device__ __forceinline__ uint32_t& u4(uint4& v, int i) { return reinterpret_cast<uint32_t*>(&v)[i]; }
 
 // Four OCP e4m3 bytes -> four values of the 16-bit MFMA operand type.  Every e4m3 value is exactly
-// representable in f16 and in bf16, so the conversion through fp32 loses nothing.
+// representable in f16 and in bf16; gfx950 converts a pair of bytes straight to a pair of 16-bit values
+// (v_cvt_scalef32_pk_{bf16,f16}_fp8 with a unit scale), half the instructions of the way through fp32.
+typedef __attribute__((ext_vector_type(2))) __bf16 mfma_bf16x2_t;
+typedef __attribute__((ext_vector_type(2))) _Float16 mfma_f16x2_t;
 template <bool BF16> __device__ __forceinline__ uint2 fp8x4_to_op(uint32_t w) {
-    const auto lo = __builtin_amdgcn_cvt_pk_f32_fp8(w, false);
-    const auto hi = __builtin_amdgcn_cvt_pk_f32_fp8(w, true);
-    if (BF16) { // the upper halves of the two fp32 values, side by side
-        return make_uint2(__builtin_amdgcn_perm(__float_as_uint(lo[1]), __float_as_uint(lo[0]), 0x07060302u),
-                          __builtin_amdgcn_perm(__float_as_uint(hi[1]), __float_as_uint(hi[0]), 0x07060302u));
+    if constexpr (BF16) {
+        const mfma_bf16x2_t lo = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(w, 1.0f, false);
+        const mfma_bf16x2_t hi = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(w, 1.0f, true);
+        return make_uint2(__builtin_bit_cast(uint32_t, lo), __builtin_bit_cast(uint32_t, hi));
+    } else {
+        const mfma_f16x2_t lo = __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(w, 1.0f, false);
+        const mfma_f16x2_t hi = __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(w, 1.0f, true);
+        return make_uint2(__builtin_bit_cast(uint32_t, lo), __builtin_bit_cast(uint32_t, hi));
     }
-    return make_uint2(Mma<false>::pack2(lo[0], lo[1]), Mma<false>::pack2(hi[0], hi[1]));
 }
 // bytes 8e .. 8e+7 of a 16-byte register -> one 8-element MFMA operand
 template <bool BF16> __device__ __forceinline__ uint4 fp8x8_to_op(const uint4& r, int e) {
