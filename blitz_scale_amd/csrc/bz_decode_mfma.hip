@@ -424,8 +424,11 @@ __global__ __launch_bounds__(64, 2) void decode_mfma_kernel(MfmaDecodeArgs a, co
                 for (int r = 0; r < 4; ++r)
                     if (tile_tok0 + 16 * u + 4 * j + r >= tok_end) s[u][r] = -INFINITY;
         }
-        float tmax = fmaxf(fmaxf(fmaxf(s[0][0], s[0][1]), fmaxf(s[0][2], s[0][3])),
-                           fmaxf(fmaxf(s[1][0], s[1][1]), fmaxf(s[1][2], s[1][3])));
+        float tmax = -INFINITY; // (a running maximum compiles to v_max3 pairs; a tree of fmaxf does not)
+#pragma unroll
+        for (int u = 0; u < 2; ++u)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) tmax = fmaxf(tmax, s[u][r]);
         // the scores stay unscaled in registers: the scale is applied to the maximum here and to every
         // score inside the fused multiply-add that feeds exp2
         tmax = lane_max_xor32(lane_max_xor16(tmax)) * score_scale;

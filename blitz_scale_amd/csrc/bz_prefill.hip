@@ -212,12 +212,17 @@ __global__ __launch_bounds__(256, 2) void prefill_kernel(PrefillArgs a, const ch
     {
         const int y = h ^ (qn & 15);
 #pragma unroll
-        for (int ks = 0; ks < 8; ++ks) koff[ks] = (uint32_t)(qn * 256 + (((2 * ks) ^ y) * 16));
+        for (int ks = 0; ks < 8; ++ks) {
+            koff[ks] = lds0 + (uint32_t)(qn * 256 + (((2 * ks) ^ y) * 16));
+            asm volatile("" : "+v"(koff[ks])); // keep the sum: the compiler would re-add the base on every tile
+        }
         const int srow = (lane & 15) >> 2;
         const int zl = ((((lane >> 4) & 1) << 1) | ((lane & 3) >> 1)) ^ (srow << 1);
 #pragma unroll
-        for (int db = 0; db < 4; ++db)
-            voff[db] = (uint32_t)((4 * h + srow) * 256 + ((((db << 2)) ^ zl) * 16) + (lane & 1) * 8);
+        for (int db = 0; db < 4; ++db) {
+            voff[db] = lds0 + (uint32_t)((4 * h + srow) * 256 + ((((db << 2)) ^ zl) * 16) + (lane & 1) * 8);
+            asm volatile("" : "+v"(voff[db]));
+        }
     }
 
     // the arithmetic of tile t (K/V in LDS buffer BUF = t % 2, a compile-time constant so that the buffer
@@ -232,10 +237,16 @@ __global__ __launch_bounds__(256, 2) void prefill_kernel(PrefillArgs a, const ch
             constexpr int kDK = 4, kDV = 4;
             uint4 ka[kDK], va[kDV];
             auto k_read = [&](int i) __attribute__((always_inline)) { // operand of score step i: block i/8, d step i%8
-                return *reinterpret_cast<const uint4*>(smem + BUF * kTile + (i >> 3) * 32 * 256 + koff[i & 7]);
+                // (koff / voff hold complete LDS addresses, so the rest is the instruction's immediate offset)
+                const unsigned char __attribute__((address_space(3)))* kb =
+                    (const unsigned char __attribute__((address_space(3)))*)(uintptr_t)koff[i & 7];
+                typedef uint32_t __attribute__((ext_vector_type(4))) pf_u32x4;
+                const pf_u32x4 r = *reinterpret_cast<const pf_u32x4 __attribute__((address_space(3)))*>(
+                    kb + (BUF * kTile + (i >> 3) * 32 * 256));
+                return make_uint4(r.x, r.y, r.z, r.w);
             };
             auto v_read = [&](int i) __attribute__((always_inline)) { // operand of step i: tokens 16*(i/4).., d block i%4
-                const unsigned char* vb = smem + (2 + BUF) * kTile + (i >> 2) * 16 * 256 + voff[i & 3];
+                const uint32_t vb = voff[i & 3] + (uint32_t)((2 + BUF) * kTile + (i >> 2) * 16 * 256);
                 const pf_s16x4 t0 =
                     __builtin_amdgcn_ds_read_tr16_b64_v4i16((pf_s16x4 __attribute__((address_space(3)))*)(vb));
                 const pf_s16x4 t1 = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
