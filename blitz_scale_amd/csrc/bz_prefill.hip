@@ -248,9 +248,9 @@ __global__ __launch_bounds__(256, 2) void prefill_kernel(PrefillArgs a, const ch
             auto v_read = [&](int i) __attribute__((always_inline)) { // operand of step i: tokens 16*(i/4).., d block i%4
                 const uint32_t vb = voff[i & 3] + (uint32_t)((2 + BUF) * kTile + (i >> 2) * 16 * 256);
                 const pf_s16x4 t0 =
-                    __builtin_amdgcn_ds_read_tr16_b64_v4i16((pf_s16x4 __attribute__((address_space(3)))*)(vb));
+                    __builtin_amdgcn_ds_read_tr16_b64_v4i16((pf_s16x4 __attribute__((address_space(3)))*)(uintptr_t)(vb));
                 const pf_s16x4 t1 = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-                    (pf_s16x4 __attribute__((address_space(3)))*)(vb + 8 * 256));
+                    (pf_s16x4 __attribute__((address_space(3)))*)(uintptr_t)(vb + 8 * 256));
                 const uint2 w0 = __builtin_bit_cast(uint2, t0), w1 = __builtin_bit_cast(uint2, t1);
                 return make_uint4(w0.x, w0.y, w1.x, w1.y);
             };
