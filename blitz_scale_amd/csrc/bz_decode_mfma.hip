@@ -517,20 +517,23 @@ __global__ __launch_bounds__(64, 2) void decode_mfma_kernel(MfmaDecodeArgs a, co
 }
 
 // Combine the partials of one split (sequence, kv head): o = sum_i o_i 2^(lse_i - M) / sum_i 2^(lse_i - M).
-// One workgroup of 128 lanes per (split, q head of the group).  The partials are fetched eight at a
-// time with all loads issued before any is used, and merged with a running maximum, so a split with up
-// to eight partials costs two dependent memory round trips (schedule entry, then data).  (Batches of 32
-// for the 32-piece splits of small batches were measured: 0.3 us less per launch there, 1.4 us more on
-// the large-batch workload, where most splits have two to four partials.)
-template <typename OT>
-__global__ __launch_bounds__(128) void decode_mfma_combine_kernel(const MfmaCombine* __restrict__ combos,
-                                                                  const float* __restrict__ part_o,
-                                                                  const float* __restrict__ part_lse, void* out,
-                                                                  float* lse, uint32_t num_qo_heads, uint32_t G) {
+// One workgroup per (split, q head of the group): 128 lanes (one per output dimension) x S slices.  A
+// slice fetches eight partials at a time with all loads issued before any is used and merges them with a
+// running maximum; slice s takes batches s, s+S, ...  With S = 1 (splits of up to 16 partials, what large
+// batches produce) that is two dependent memory round trips for up to eight partials.  A single long
+// sequence at small batch is cut into as many pieces as there are wave slots (256 partials per kv head
+// for one sequence on the whole chip): S = 4 or 8 slices then work side by side and are merged through
+// LDS, instead of 32 round trips one after the other.  (Batches of 32 per lane were measured as well:
+// slower on the large-batch workload, where most splits have two to four partials.)
+template <typename OT, int S>
+__global__ __launch_bounds__(128 * S) void decode_mfma_combine_kernel(const MfmaCombine* __restrict__ combos,
+                                                                      const float* __restrict__ part_o,
+                                                                      const float* __restrict__ part_lse, void* out,
+                                                                      float* lse, uint32_t num_qo_heads, uint32_t G) {
     const MfmaCombine c = combos[blockIdx.x];
-    const uint32_t g = blockIdx.y, d = threadIdx.x;
+    const uint32_t g = blockIdx.y, d = threadIdx.x, sl = threadIdx.y;
     float M = -INFINITY, wsum = 0.f, o = 0.f;
-    for (int i0 = 0; i0 < c.count; i0 += 8) {
+    for (int i0 = 8 * (int)sl; i0 < c.count; i0 += 8 * S) {
         float li[8], oi[8];
 #pragma unroll
         for (int k = 0; k < 8; ++k) {
@@ -553,6 +556,28 @@ __global__ __launch_bounds__(128) void decode_mfma_combine_kernel(const MfmaComb
             o += w * oi[k];
         }
         M = m2;
+    }
+    if constexpr (S > 1) {
+        __shared__ float sm_m[S][128], sm_w[S][128], sm_o[S][128];
+        sm_m[sl][d] = M;
+        sm_w[sl][d] = wsum;
+        sm_o[sl][d] = o;
+        __syncthreads();
+        if (sl != 0) return;
+        float mm = -INFINITY;
+#pragma unroll
+        for (int t = 0; t < S; ++t) mm = fmaxf(mm, sm_m[t][d]);
+        wsum = 0.f;
+        o = 0.f;
+        if (mm != -INFINITY) {
+#pragma unroll
+            for (int t = 0; t < S; ++t) {
+                const float sc = exp2f(sm_m[t][d] - mm); // an empty slice has M = -inf: weight 0
+                wsum += sm_w[t][d] * sc;
+                o += sm_o[t][d] * sc;
+            }
+        }
+        M = mm;
     }
     o = wsum > 0.f ? o / wsum : 0.f;
     const size_t hq = (size_t)c.seq * num_qo_heads + (size_t)c.kvh * G + g;
@@ -581,8 +606,16 @@ static int launch_mfma(const DecodePlan* p, const MfmaDecodeArgs& a, bool kv8, h
     BZ_LAUNCH_CHECK();
     if (p->time_stop) BZ_CHECK_HIP(hipEventRecord(p->time_stop, s));
     if (p->mfma_combos > 0) {
-        hipLaunchKernelGGL((decode_mfma_combine_kernel<OT>), dim3(p->mfma_combos, a.group), dim3(128), 0, s,
-                           p->mfma_combos_d, a.part_o, a.part_lse, a.out, a.lse, a.num_qo_heads, a.group);
+        const dim3 cgrid(p->mfma_combos, a.group);
+        if (p->mfma_max_count <= 16)
+            hipLaunchKernelGGL((decode_mfma_combine_kernel<OT, 1>), cgrid, dim3(128, 1), 0, s, p->mfma_combos_d,
+                               a.part_o, a.part_lse, a.out, a.lse, a.num_qo_heads, a.group);
+        else if (p->mfma_max_count <= 64)
+            hipLaunchKernelGGL((decode_mfma_combine_kernel<OT, 4>), cgrid, dim3(128, 4), 0, s, p->mfma_combos_d,
+                               a.part_o, a.part_lse, a.out, a.lse, a.num_qo_heads, a.group);
+        else
+            hipLaunchKernelGGL((decode_mfma_combine_kernel<OT, 8>), cgrid, dim3(128, 8), 0, s, p->mfma_combos_d,
+                               a.part_o, a.part_lse, a.out, a.lse, a.num_qo_heads, a.group);
         BZ_LAUNCH_CHECK();
     }
     return 0;

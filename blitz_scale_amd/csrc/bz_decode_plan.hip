@@ -350,8 +350,11 @@ extern "C" int bz_decode_plan(bz_decode_plan_t* plan_, void* float_buffer, size_
         p->mfma_partials = mfma_partials;
         int32_t last = -1;
         p->mfma_split_seqs = 0;
-        for (const MfmaCombine& c : mc)
+        p->mfma_max_count = 0;
+        for (const MfmaCombine& c : mc) {
             if (c.seq != last) { ++p->mfma_split_seqs; last = c.seq; }
+            p->mfma_max_count = std::max(p->mfma_max_count, (uint32_t)c.count);
+        }
     }
     // BZ_DECODE_PATH=general keeps the MFMA kernel out (used to test the general kernel on shapes
     // both kernels cover)

@@ -97,6 +97,7 @@ struct DecodePlan {
     bool mfma_ok = false;
     bool force_general = false; // tests: run the general kernel even where the MFMA path applies
     uint32_t mfma_slots = 0, mfma_combos = 0, mfma_partials = 0, mfma_pieces = 0, mfma_split_seqs = 0;
+    uint32_t mfma_max_count = 0; // most partials any split (sequence, kv head) has
     const MfmaPiece* mfma_pieces_d = nullptr;
     const MfmaCombine* mfma_combos_d = nullptr;
     const MfmaTile* mfma_tiles_d = nullptr;

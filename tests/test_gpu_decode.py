@@ -182,3 +182,25 @@ def test_plan_fits_the_workspace_it_reports():
         infos.append(info)
     assert infos[0]["workgroups"] == slots          # the matrix-core schedule was taken
     assert infos[1]["workgroups"] != slots          # no room for it: page-aligned segments x kv heads
+
+
+@pytest.mark.parametrize("ctx,expect_min_partials", [
+    ([20000], 65),            # one long sequence over the whole chip: hundreds of partials per kv head
+    ([1024] * 8, 17),         # small batch: every (sequence, kv head) cut into ~32 one-tile pieces
+    ([3000, 5], 17),
+])
+def test_splits_with_many_partials(ctx, expect_min_partials):
+    """The split-K combine takes its sliced form (4 or 8 slices merged through LDS) when a (sequence, kv
+    head) has more than 16 partials; results as for any other decode."""
+    from blitz_scale_amd import kernel as K
+    p = DecodeProblem(4242, ctx, 32, 8, 128, 16, BZ_BF16)
+    ref, ref_lse = oracle.batch_decode(p.q, p.dtype, p.oracle_kv(), p.Hq, want_lse=True, parallel=True)
+    dev = DeviceDecode(p)
+    dev.plan(2048)
+    counts = dev.handler.host_schedule(6)[:, 3]
+    assert counts.max() >= expect_min_partials
+    got32, lse = dev.decode(BZ_F32, BZ_ROPE_NONE, want_lse=True)
+    assert np.abs(got32 - ref).max() <= 2e-5
+    assert np.abs(lse - ref_lse).max() < 1e-3
+    got = dev.decode(None, BZ_ROPE_NONE)
+    assert (np.abs(got - ref) <= ulp_tol(ref, p.dtype)).all()
