@@ -469,11 +469,11 @@ static int build_prefill_items(PrefillPlan* p, const int32_t* qo_indptr_h, const
     for (uint32_t b = 0; b <= batch_size; ++b)
         if (qo_indptr_h[b] != kv_indptr_h[b]) return BZ_ERR_UNSUPPORTED;
     // One entry per workgroup, in launch order.  Workgroups are dealt round-robin to the 8 XCDs, each
-    // with its own L2, so launch index i runs on XCD i % 8.  Every (request, q head) pair is given to one
-    // XCD as a run of consecutive jobs: its q tiles then execute together on that XCD and share the
-    // pair's K/V (up to 2 MiB for 4096 tokens) through that L2 instead of each fetching it from HBM.
-    // Pairs go to the XCDs in turn, longest requests first and tiles from the last (most keys) to the
-    // first, so every XCD gets the same mix of work.
+    // with its own L2, so launch index i runs on XCD i % 8.  Every (request, kv head) unit is given to one
+    // XCD as a run of consecutive jobs: its q tiles (of all q heads of the group) then execute together on
+    // that XCD and share the unit's K/V (up to 2 MiB for 4096 tokens) through that L2 instead of each
+    // fetching it from HBM.  Units go to the XCDs in turn, longest requests first and tiles from the last
+    // (most keys) to the first, so every XCD gets the same mix of work.
     for (uint32_t b = 0; b < batch_size; ++b)
         if (qo_indptr_h[b + 1] < qo_indptr_h[b]) return BZ_ERR_BAD_ARG;
     std::vector<uint32_t> order(batch_size);
@@ -484,13 +484,23 @@ static int build_prefill_items(PrefillPlan* p, const int32_t* qo_indptr_h, const
     constexpr int kXcd = 8;
     std::vector<PrefillItem> per_xcd[kXcd];
     uint32_t pair = 0;
+    // Grouped-query attention: the q heads of one kv head read the same K/V, so they go to one XCD
+    // together, tile by tile (the same K/V tiles are then in flight for all of them at once) -- as long
+    // as that leaves at least two units of work per XCD; otherwise the group is cut into parts.
+    const uint32_t G = num_qo_heads / num_kv_heads;
+    uint32_t live = 0;
+    for (uint32_t b = 0; b < batch_size; ++b) live += qo_indptr_h[b + 1] > qo_indptr_h[b];
+    uint32_t parts = 1;
+    while (parts < G && (G % parts || (uint64_t)live * num_kv_heads * parts < 2 * kXcd)) ++parts;
+    const uint32_t per_part = G / parts;
     for (uint32_t b : order) {
         const int32_t len = qo_indptr_h[b + 1] - qo_indptr_h[b];
         if (len == 0) continue;
         const int32_t last_q0 = (len - 1) / kBM * kBM;
-        for (uint32_t h = 0; h < num_qo_heads; ++h, ++pair)
+        for (uint32_t unit = 0; unit < num_kv_heads * parts; ++unit, ++pair)
             for (int32_t q0 = last_q0; q0 >= 0; q0 -= kBM)
-                per_xcd[pair % kXcd].push_back({qo_indptr_h[b], len, q0, (int32_t)h});
+                for (uint32_t g = 0; g < per_part; ++g)
+                    per_xcd[pair % kXcd].push_back({qo_indptr_h[b], len, q0, (int32_t)(unit * per_part + g)});
     }
     size_t longest = 0;
     for (auto& v : per_xcd) longest = std::max(longest, v.size());

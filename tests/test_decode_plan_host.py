@@ -164,12 +164,14 @@ def test_fewer_compute_units_mean_fewer_longer_shares():
     ([20, 37], 4, 2),
     ([128, 129, 1, 4096, 0, 640], 8, 8),
     (None, 40, 40),  # config 4: 16 prompts U[128, 4096], 40 heads
+    ([512, 300, 2048, 77], 32, 8),  # grouped-query attention with enough units: whole groups stay together
+    ([4096], 32, 4),                # ... and with too few: the group of 8 is cut into parts
 ])
 def test_prefill_job_list_invariants(lens, Hq, Hkv):
     """The prefill plan (replacement of BatchPrefillRaggedHandler::plan, src/kernel/flashinfer_types.cu:24-49):
-    one job per (request, q head, 128-row q tile), each exactly once; the jobs of a (request, head) pair sit
-    in one column of the 8-wide launch order (one XCD, consecutive there), last tile first; longer requests
-    come first; padding entries have length 0."""
+    one job per (request, q head, 128-row q tile), each exactly once; the jobs of a (request, kv head) unit
+    sit in one column of the 8-wide launch order (one XCD, consecutive there), last tile first, the q heads
+    of the group side by side; longer requests come first; padding entries have length 0."""
     if lens is None:
         lens = np.random.default_rng(0x5EED).integers(128, 4097, 16)
     lens = np.asarray(lens, np.int64)
@@ -203,8 +205,16 @@ def test_prefill_job_list_invariants(lens, Hq, Hkv):
     for c in range(8):
         col = [int(ln) for (tok0, ln, q0, head) in items[c::8] if ln > 0]
         assert all(a >= b for a, b in zip(col, col[1:]))
-    # no column holds more than its share of pairs + 1
-    per_col = np.bincount(list(column.values()), minlength=8)
+    # grouped-query attention: the q heads of a kv head travel together (same column, same tile side by side)
+    # unless that would leave fewer than two units per column, in which case the group is cut into equal parts
+    G = Hq // Hkv
+    live = int((lens > 0).sum())
+    parts = next(p for p in range(1, G + 1) if G % p == 0 and (live * Hkv * p >= 16 or p == G))
+    per_part = G // parts
+    for (b, hd), c in column.items():
+        assert c == column[(b, hd - hd % per_part)]
+    # no column holds more than its share of units + 1
+    per_col = np.bincount([c for (b, hd), c in column.items() if hd % per_part == 0], minlength=8)
     assert per_col.max() - per_col.min() <= 1
     # a head size the kernel does not cover is refused on the host
     with pytest.raises(K.BzError):
