@@ -1,7 +1,8 @@
-// MFMA paged decode for gfx950 (head_dim 128, page_size a multiple of 16, f16/bf16 KV, up to 16
-// query heads per kv head).  One wave64 per workgroup walks a list of "pieces" (contiguous runs of
-// 32-token tiles of one (sequence, kv head)) that the host planner balanced over the wave slots
-// of the chip, so every K and V byte is read once and shared by all query heads of the group.
+// MFMA paged decode for gfx950 (head_dim 128, page_size a multiple of 16, f16/bf16/e4m3 KV, up to 16
+// query heads per scheduled unit; the planner cuts a larger group into equal parts).  One wave64 per
+// workgroup walks a list of "pieces" (contiguous runs of 32-token tiles of one (sequence, kv head)) that
+// the host planner balanced over the wave slots of the chip, so every K and V byte is read once and
+// shared by all query heads of the group.
 //
 // Per 32-token tile, with S^T = K Q^T so that the MFMA result layout of the scores is already the
 // A-operand layout of the P V product (no shuffles between the two contractions):
@@ -42,7 +43,7 @@ struct MfmaDecodeArgs {
     float* part_o;   // [num_partials][16][128]
     float* part_lse; // [num_partials][16]
     uint64_t stride_page, stride_n, stride_h; // elements
-    uint32_t page_size, num_qo_heads, group;
+    uint32_t page_size, num_qo_heads, group; // group: q heads per scheduled unit (<= 16)
     int rope_q;
     float sm_scale_log2;
     const float* k_scale; // e4m3 pool only: per-kv-head dequantisation factors (nullptr = 1)
@@ -123,7 +124,7 @@ __device__ __forceinline__ void wave_lds_sync() {
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 }
 
-constexpr int kInfoInts = 12; // per-tile description kept in LDS (see fetch_info): 9 ints, padded
+constexpr int kInfoInts = 12; // per-tile description kept in LDS (see fetch_info): 10 ints, padded
 
 // KV8: the pool holds e4m3 bytes.  K and V are widened to the 16-bit type of q in registers (exactly)
 // on their way to the matrix cores; the per-head scales are folded into the softmax scale and into
@@ -167,9 +168,9 @@ __global__ __launch_bounds__(64, 2) void decode_mfma_kernel(MfmaDecodeArgs a, co
     const int ahead = max(ahead_raw, 0);
 
     // ---- descriptions of 32 tiles at a time: lane l < 32 fetches the record of tile base+l, the two
-    // page ids it points at and the piece it belongs to, and leaves 9 ints in LDS:
-    //   [pid0, pid1, t, seq | kvh, flags (1: first tile of its piece, 2: last), partial, tok_end | seq_len]
-    struct Desc { int v[9]; };
+    // page ids it points at and the piece it belongs to, and leaves 10 ints in LDS:
+    //   [pid0, pid1, t, seq | kvh, flags (1: first tile of its piece, 2: last), partial, tok_end | seq_len, kv head]
+    struct Desc { int v[10]; };
     auto fetch_info = [&](int base) -> Desc {
         Desc d;
         const int g = base + (lane & 31);
@@ -187,6 +188,7 @@ __global__ __launch_bounds__(64, 2) void decode_mfma_kernel(MfmaDecodeArgs a, co
         d.v[6] = m1.x;                                             // partial slot or -1
         d.v[8] = max(m2.z - ahead, 0);                             // seq_len at present
         d.v[7] = min(m0.w * kTileTok, d.v[8]);                     // tok_end of the piece
+        d.v[9] = m2.w;                                             // kv head whose K/V are read (kvh is the scheduled unit)
         return d;
     };
     auto stash_info = [&](const Desc& d, int buf) {
@@ -194,21 +196,23 @@ __global__ __launch_bounds__(64, 2) void decode_mfma_kernel(MfmaDecodeArgs a, co
             int* dst = &info_lds[buf][lane][0];
             *reinterpret_cast<int4*>(dst) = make_int4(d.v[0], d.v[1], d.v[2], d.v[3]);
             *reinterpret_cast<int4*>(dst + 4) = make_int4(d.v[4], d.v[5], d.v[6], d.v[7]);
-            dst[8] = d.v[8];
+            *reinterpret_cast<int2*>(dst + 8) = make_int2(d.v[8], d.v[9]);
         }
     };
-    struct TileUni { int pid0, pid1, t, seq, kvh, flags, partial, tok_end, seq_len; }; // wave-uniform
+    struct TileUni { int pid0, pid1, t, seq, kvh, flags, partial, tok_end, seq_len, kvr; }; // wave-uniform
     auto read_info = [&](int buf, int i) -> TileUni {
         const int* src = &info_lds[buf][i][0];
         const int4 x = *reinterpret_cast<const int4*>(src);
         const int4 y = *reinterpret_cast<const int4*>(src + 4);
-        const int z = src[8];
+        const int2 z2 = *reinterpret_cast<const int2*>(src + 8);
+        const int z = z2.x;
         TileUni u;
         u.pid0 = __builtin_amdgcn_readfirstlane(x.x); u.pid1 = __builtin_amdgcn_readfirstlane(x.y);
         u.t = __builtin_amdgcn_readfirstlane(x.z); u.seq = __builtin_amdgcn_readfirstlane(x.w);
         u.kvh = __builtin_amdgcn_readfirstlane(y.x); u.flags = __builtin_amdgcn_readfirstlane(y.y);
         u.partial = __builtin_amdgcn_readfirstlane(y.z); u.tok_end = __builtin_amdgcn_readfirstlane(y.w);
         u.seq_len = __builtin_amdgcn_readfirstlane(z);
+        u.kvr = __builtin_amdgcn_readfirstlane(z2.y);
         return u;
     };
 
@@ -221,7 +225,7 @@ __global__ __launch_bounds__(64, 2) void decode_mfma_kernel(MfmaDecodeArgs a, co
 #pragma unroll
         for (int s = 0; s < 2; ++s) {
             const int slot0 = (u.t * kTileTok + 16 * s) % P; // a subtile past the last page reads the last page, masked later
-            r.b[s] = ((size_t)pid[s] * a.stride_page + (size_t)slot0 * a.stride_n + (size_t)u.kvh * a.stride_h) * ES;
+            r.b[s] = ((size_t)pid[s] * a.stride_page + (size_t)slot0 * a.stride_n + (size_t)u.kvr * a.stride_h) * ES;
         }
         return r;
     };
@@ -269,6 +273,7 @@ __global__ __launch_bounds__(64, 2) void decode_mfma_kernel(MfmaDecodeArgs a, co
     un.pid0 = indices[first.idx0];
     un.pid1 = indices[first.idx1];
     un.t = first.t; un.seq = first.seq; un.kvh = first.kvh; un.flags = first.flags; un.partial = first.partial;
+    un.kvr = first.kv_head;
     un.seq_len = max(first.seq_len - ahead, 0);
     un.tok_end = min(first.tile_end * kTileTok, un.seq_len);
     issue_q(un);
@@ -300,7 +305,7 @@ __global__ __launch_bounds__(64, 2) void decode_mfma_kernel(MfmaDecodeArgs a, co
         if (i == 24 && chunk_base + 32 < g_end) { stash_info(dnext, buf ^ 1); wave_lds_sync(); }
         const int t = uc.t, tok_end = uc.tok_end, seq_len = uc.seq_len;
         // (positive; the floor keeps masked scores at -inf instead of NaN should a head's K scale be zero)
-        const float score_scale = fmaxf(a.sm_scale_log2 * ((KV8 && a.k_scale) ? a.k_scale[uc.kvh] : 1.0f), 1e-30f);
+        const float score_scale = fmaxf(a.sm_scale_log2 * ((KV8 && a.k_scale) ? a.k_scale[uc.kvr] : 1.0f), 1e-30f);
 
         if (uc.flags & 1) { // ================= first tile of a piece =================
 #pragma unroll
@@ -487,7 +492,7 @@ __global__ __launch_bounds__(64, 2) void decode_mfma_kernel(MfmaDecodeArgs a, co
 
         if (uc.flags & 2) { // ================= last tile of a piece: final rows, or the split-K partial
             const int b = uc.seq, kvh = uc.kvh, partial = uc.partial;
-            const float inv_l = (l_run > 0.f ? 1.0f / l_run : 0.f) * ((KV8 && a.v_scale) ? a.v_scale[kvh] : 1.0f);
+            const float inv_l = (l_run > 0.f ? 1.0f / l_run : 0.f) * ((KV8 && a.v_scale) ? a.v_scale[uc.kvr] : 1.0f);
             const float lse2 = l_run > 0.f ? m_run + log2f(l_run) : -INFINITY;
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
@@ -639,7 +644,8 @@ int decode_fast_path(const DecodePlan* p, const void* q, void* out, float* lse, 
     a.pieces = p->mfma_pieces_d; a.tiles = p->mfma_tiles_d; a.heads = p->mfma_heads_d;
     a.part_o = p->mfma_part_o; a.part_lse = p->mfma_part_lse;
     a.stride_page = kv->stride_page; a.stride_n = kv->stride_n; a.stride_h = kv->stride_h;
-    a.page_size = kv->page_size; a.num_qo_heads = num_qo_heads; a.group = num_qo_heads / kv->num_kv_heads;
+    a.page_size = kv->page_size; a.num_qo_heads = num_qo_heads;
+    a.group = num_qo_heads / kv->num_kv_heads / p->mfma_parts;
     a.rope_q = rope_mode == BZ_ROPE_Q_ONLY;
     a.sm_scale_log2 = sm_scale_log2;
     a.k_scale = k_scale; a.v_scale = v_scale;

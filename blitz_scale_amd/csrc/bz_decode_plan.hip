@@ -120,15 +120,22 @@ static int build_schedule(DecodePlan* p, const int32_t* indptr_h, const int32_t*
     std::vector<MfmaCombine>& mc = p->h_mcombos;
     mp.clear(); mt.clear(); mptr.clear(); mc.clear();
     uint32_t mfma_partials = 0;
+    // A group of more than 16 q heads per kv head does not fit the 16 columns of the score tile: it is
+    // scheduled as `parts` equal parts, each a kv head of its own as far as the schedule goes (heads
+    // [u*gp, (u+1)*gp) of unit u = kvh*parts + part; the K/V of the kv head are read once per part).
     const uint32_t group = num_qo_heads / num_kv_heads;
-    const bool mfma_shape = head_dim == 128 && page_size % 16 == 0 && group <= 16;
+    uint32_t parts = (group + 15) / 16;
+    while (parts < group && group % parts) ++parts;
+    const bool mfma_shape = head_dim == 128 && page_size % 16 == 0 && group / parts <= 16 && parts <= 8;
+    p->mfma_parts = mfma_shape ? parts : 1;
+    const uint32_t num_units = num_kv_heads * (mfma_shape ? parts : 1); // kv heads as the matrix-core schedule sees them
     if (mfma_shape) {
         uint64_t total_tiles = 0;
         for (uint32_t b = 0; b < batch_size; ++b) {
             const int32_t np = indptr_h[b + 1] - indptr_h[b];
             if (np <= 0) continue;
             const int64_t len = (int64_t)(np - 1) * page_size + last_page_len_h[b];
-            total_tiles += (uint64_t)((len + 31) / 32) * num_kv_heads;
+            total_tiles += (uint64_t)((len + 31) / 32) * num_units;
         }
         int page_shift = -1; // log2(page_size) when it is a power of two
         if ((page_size & (page_size - 1)) == 0) { page_shift = 0; while ((1u << page_shift) < page_size) ++page_shift; }
@@ -163,7 +170,7 @@ static int build_schedule(DecodePlan* p, const int32_t* indptr_h, const int32_t*
             if (np <= 0) continue;
             const int64_t len = (int64_t)(np - 1) * page_size + last_page_len_h[b];
             const int32_t tiles = (int32_t)((len + 31) / 32);
-            for (uint32_t h = 0; h < num_kv_heads; ++h) {
+            for (uint32_t h = 0; h < num_units; ++h) {
                 const size_t first_piece = mp.size();
                 int32_t t = 0;
                 while (t < tiles) {
@@ -205,7 +212,7 @@ static int build_schedule(DecodePlan* p, const int32_t* indptr_h, const int32_t*
                         }
                     }
                     mp.push_back({(int32_t)b, (int32_t)h, t, t + take, -1, -1, 0, 0, indptr_h[b], np, (int32_t)len,
-                                  {0, 0, 0, 0, 0}});
+                                  (int32_t)(h / p->mfma_parts), {0, 0, 0, 0}});
                     t += take;
                 }
                 const size_t cnt = mp.size() - first_piece;
@@ -316,7 +323,7 @@ extern "C" int bz_decode_plan(bz_decode_plan_t* plan_, void* float_buffer, size_
                 hd.idx0 = r.idx0; hd.idx1 = r.idx1; hd.t = r.t;
                 hd.seq = pc.seq; hd.kvh = pc.kvh;
                 hd.flags = (r.t == pc.tile_begin ? 1 : 0) | (r.t + 1 == pc.tile_end ? 2 : 0);
-                hd.partial = pc.partial; hd.tile_end = pc.tile_end; hd.seq_len = pc.seq_len;
+                hd.partial = pc.partial; hd.tile_end = pc.tile_end; hd.seq_len = pc.seq_len; hd.kv_head = pc.kv_head;
             }
             heads[sl] = hd;
         }

@@ -28,7 +28,9 @@ struct MfmaPiece {
     int32_t partial;              // -1: whole (sequence, kv head) -> final rows; else partial slot
     int32_t combo, count, first;  // split (sequence, kv head): its index, number of partials, first slot
     int32_t ip0, npages, seq_len; // indptr[seq], pages and tokens of the sequence (from the host table)
-    int32_t pad[5];
+    int32_t kv_head;              // the kv head whose K/V the piece reads (kvh above is the scheduled unit:
+                                  // kv_head * parts + part when a kv head has more than 16 q heads)
+    int32_t pad[4];
 };
 
 // One 32-token tile of a wave slot's share, in processing order.
@@ -48,7 +50,7 @@ struct MfmaSlotHead {
     int32_t partial;      // -1 or partial slot
     int32_t tile_end;     // one past the last tile of the piece
     int32_t seq_len;
-    int32_t pad;
+    int32_t kv_head;      // kv head of the first tile's piece
 };
 
 // Growable array of plain records that does not clear what it hands out (the planner overwrites every
@@ -98,6 +100,7 @@ struct DecodePlan {
     bool force_general = false; // tests: run the general kernel even where the MFMA path applies
     uint32_t mfma_slots = 0, mfma_combos = 0, mfma_partials = 0, mfma_pieces = 0, mfma_split_seqs = 0;
     uint32_t mfma_max_count = 0; // most partials any split (sequence, kv head) has
+    uint32_t mfma_parts = 1;     // groups of more than 16 q heads are scheduled as this many equal parts per kv head
     const MfmaPiece* mfma_pieces_d = nullptr;
     const MfmaCombine* mfma_combos_d = nullptr;
     const MfmaTile* mfma_tiles_d = nullptr;

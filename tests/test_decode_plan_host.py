@@ -118,13 +118,20 @@ def check_general_schedule(s, P):
     ("never_split", [5000, 40, 900], 8, 8, 16, 0xFFFFFFFF),
     ("one_token", [1], 8, 1, 16, 0),
     ("page48", [100, 1000, 47, 48, 49], 32, 8, 48, 512),      # page size not a power of two
+    ("group32", [700, 64, 3000], 32, 1, 16, 2048),             # 32 q heads on one kv head: two parts of 16
+    ("group24", [700, 64, 3000], 48, 2, 16, 2048),             # 24 per kv head: two parts of 12
 ])
 def test_matrix_core_schedule_invariants(name, lens, Hq, Hkv, P, split):
     if lens is None:
         lens = wl.lognormal_ctx(np.random.default_rng(0x5EED), 128, 1024, 1.0, 64, 8192)
     s = schedule(lens, Hq, Hkv, 128, P, split)
-    assert len(s["tiles"]) == sum((int(l) + 31) // 32 for l in lens) * Hkv
-    check_mfma_schedule(s, Hkv, P, split)
+    # a kv head with more than 16 q heads is scheduled as equal parts, each a unit of its own
+    G = Hq // Hkv
+    parts = next(p for p in range((G + 15) // 16, G + 1) if G % p == 0)
+    units = Hkv * parts
+    assert len(s["tiles"]) == sum((int(l) + 31) // 32 for l in lens) * units
+    check_mfma_schedule(s, units, P, split)
+    assert (s["pieces"][:, 11] == s["pieces"][:, 1] // parts).all()  # the kv head whose K/V a piece reads
     n_partials = check_general_schedule(s, P)
     # reported workspace: the sections the kernels read, 256-byte aligned
     al = lambda x: (x + 255) // 256 * 256

@@ -204,3 +204,23 @@ def test_splits_with_many_partials(ctx, expect_min_partials):
     assert np.abs(lse - ref_lse).max() < 1e-3
     got = dev.decode(None, BZ_ROPE_NONE)
     assert (np.abs(got - ref) <= ulp_tol(ref, p.dtype)).all()
+
+
+@pytest.mark.parametrize("Hq,Hkv,kv_dtype", [(32, 1, None), (48, 2, None), (128, 2, None), (64, 2, BZ_E4M3)])
+def test_more_than_sixteen_q_heads_per_kv_head(Hq, Hkv, kv_dtype):
+    """Groups of 24, 32 and 64 q heads run on the matrix-core kernel as equal parts of at most 16 (each part
+    reads its kv head's K/V; with an e4m3 pool the scales are those of the kv head, not of the part)."""
+    p = DecodeProblem(515, [70, 1500, 16, 333, 2600], Hq, Hkv, 128, 16, BZ_BF16, kv_dtype=kv_dtype)
+    ref = oracle.batch_decode(p.q, p.dtype, p.oracle_kv(), Hq, k_scale=p.k_scale, v_scale=p.v_scale, parallel=True)
+    dev = DeviceDecode(p)
+    info = dev.plan(1024)
+    G = Hq // Hkv
+    parts = next(q for q in range((G + 15) // 16, G + 1) if G % q == 0)
+    pieces = dev.handler.host_schedule(5)
+    assert len(pieces) > 0 and pieces[:, 1].max() == Hkv * parts - 1   # the matrix-core schedule was built
+    got = dev.decode(None, BZ_ROPE_NONE)
+    base = 3e-2 if kv_dtype == BZ_E4M3 else 2e-3
+    assert (np.abs(got - ref) <= ulp_tol(ref, p.dtype, base)).all(), float(np.abs(got - ref).max())
+    if kv_dtype is None:
+        got32 = dev.decode(BZ_F32, BZ_ROPE_NONE)
+        assert np.abs(got32 - ref).max() <= 2e-5
