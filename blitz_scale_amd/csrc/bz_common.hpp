@@ -110,6 +110,11 @@ template <> struct Vec8<f16_t> {
     uint4 raw;
     __device__ __forceinline__ void load(const void* p) { raw = *reinterpret_cast<const uint4*>(p); }
     __device__ __forceinline__ void store(void* p) const { *reinterpret_cast<uint4*>(p) = raw; }
+    __device__ __forceinline__ void store_nt(void* p) const { // for data that is not read again soon
+        typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+        const u32x4 v = {raw.x, raw.y, raw.z, raw.w};
+        __builtin_nontemporal_store(v, reinterpret_cast<u32x4*>(p));
+    }
     __device__ __forceinline__ void to_float(float* f) const {
         const uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
 #pragma unroll
@@ -131,6 +136,11 @@ template <> struct Vec8<bf16_t> {
     uint4 raw;
     __device__ __forceinline__ void load(const void* p) { raw = *reinterpret_cast<const uint4*>(p); }
     __device__ __forceinline__ void store(void* p) const { *reinterpret_cast<uint4*>(p) = raw; }
+    __device__ __forceinline__ void store_nt(void* p) const { // for data that is not read again soon
+        typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+        const u32x4 v = {raw.x, raw.y, raw.z, raw.w};
+        __builtin_nontemporal_store(v, reinterpret_cast<u32x4*>(p));
+    }
     __device__ __forceinline__ void to_float(float* f) const {
         const uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
 #pragma unroll
@@ -152,6 +162,11 @@ template <> struct Vec8<e4m3_t> {
     uint2 raw;
     __device__ __forceinline__ void load(const void* p) { raw = *reinterpret_cast<const uint2*>(p); }
     __device__ __forceinline__ void store(void* p) const { *reinterpret_cast<uint2*>(p) = raw; }
+    __device__ __forceinline__ void store_nt(void* p) const {
+        typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
+        const u32x2 v = {raw.x, raw.y};
+        __builtin_nontemporal_store(v, reinterpret_cast<u32x2*>(p));
+    }
     __device__ __forceinline__ void to_float(float* f) const {
         e4m3x4_to_f32(raw.x, f);
         e4m3x4_to_f32(raw.y, f + 4);

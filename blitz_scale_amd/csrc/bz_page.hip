@@ -78,6 +78,12 @@ __global__ __launch_bounds__(256) void page_write_kernel(PageWriteArgs a) {
     }
 
     const int lane = threadIdx.x % LANES;
+    // Pages written at prefill are next read by a later decode step, long after they have left the
+    // caches: non-temporal stores leave the cache to the caller's q / k / v rows, which the attention
+    // call reads next (16 prompts of 128..4096 tokens, 40 heads: 362 -> 353 us).
+    auto pool_store = [](const Vec8<PT>& v, PT* p) {
+        if (PREFILL) v.store_nt(p); else v.store(p);
+    };
     const int Hq = (a.rope && a.q_inout) ? (int)a.num_qo_heads : 0;
     const int Hkv = (int)a.num_kv_heads;
     const int total_rows = Hq + 2 * Hkv;
@@ -120,8 +126,8 @@ __global__ __launch_bounds__(256) void page_write_kernel(PageWriteArgs a) {
                 Vec8<PT> l2, h2;
                 l2.raw = lo.raw;
                 h2.raw = hi.raw;
-                l2.store(dst + lane * 8);
-                h2.store(dst + D / 2 + lane * 8);
+                pool_store(l2, dst + lane * 8);
+                pool_store(h2, dst + D / 2 + lane * 8);
                 continue;
             }
         }
@@ -156,8 +162,8 @@ __global__ __launch_bounds__(256) void page_write_kernel(PageWriteArgs a) {
         Vec8<PT> l2, h2;
         l2.from_float(x);
         h2.from_float(y);
-        l2.store(dst + lane * 8);
-        h2.store(dst + D / 2 + lane * 8);
+        pool_store(l2, dst + lane * 8);
+        pool_store(h2, dst + D / 2 + lane * 8);
     }
 }
 
