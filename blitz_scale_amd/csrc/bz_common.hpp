@@ -109,6 +109,11 @@ template <typename T> struct Vec8;
 template <> struct Vec8<f16_t> {
     uint4 raw;
     __device__ __forceinline__ void load(const void* p) { raw = *reinterpret_cast<const uint4*>(p); }
+    __device__ __forceinline__ void load_nt(const void* p) { // for data that is read once
+        typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+        const u32x4 v = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(p));
+        raw = make_uint4(v.x, v.y, v.z, v.w);
+    }
     __device__ __forceinline__ void store(void* p) const { *reinterpret_cast<uint4*>(p) = raw; }
     __device__ __forceinline__ void store_nt(void* p) const { // for data that is not read again soon
         typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
@@ -135,6 +140,11 @@ template <> struct Vec8<f16_t> {
 template <> struct Vec8<bf16_t> {
     uint4 raw;
     __device__ __forceinline__ void load(const void* p) { raw = *reinterpret_cast<const uint4*>(p); }
+    __device__ __forceinline__ void load_nt(const void* p) { // for data that is read once
+        typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+        const u32x4 v = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(p));
+        raw = make_uint4(v.x, v.y, v.z, v.w);
+    }
     __device__ __forceinline__ void store(void* p) const { *reinterpret_cast<uint4*>(p) = raw; }
     __device__ __forceinline__ void store_nt(void* p) const { // for data that is not read again soon
         typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
@@ -161,6 +171,11 @@ template <> struct Vec8<bf16_t> {
 template <> struct Vec8<e4m3_t> {
     uint2 raw;
     __device__ __forceinline__ void load(const void* p) { raw = *reinterpret_cast<const uint2*>(p); }
+    __device__ __forceinline__ void load_nt(const void* p) {
+        typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
+        const u32x2 v = __builtin_nontemporal_load(reinterpret_cast<const u32x2*>(p));
+        raw = make_uint2(v.x, v.y);
+    }
     __device__ __forceinline__ void store(void* p) const { *reinterpret_cast<uint2*>(p) = raw; }
     __device__ __forceinline__ void store_nt(void* p) const {
         typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));

@@ -123,8 +123,8 @@ __global__ __launch_bounds__(256) void decode_general_kernel(DecodeArgs a) {
             const int64_t page = a.indices[ip0 + jc / (int)a.page_size];
             const size_t off =
                 ((size_t)page * a.stride_page + (size_t)(jc % (int)a.page_size) * a.stride_n) * esz + head_off;
-            kv[u].load(a.k_data + off);
-            vv[u].load(a.v_data + off);
+            kv[u].load_nt(a.k_data + off); // read once per launch (+2 to 3 % over plain loads)
+            vv[u].load_nt(a.v_data + off);
         }
 #pragma unroll
         for (int u = 0; u < UNROLL; ++u) {

@@ -24,8 +24,15 @@ namespace bz {
 // cover whole 128-byte lines; K loads cover half a line per instruction, and for one-byte pools the
 // hint on K costs 6 % (429 against 403 us at 256 x 4096 tokens) while the hint on V alone gains 2 %,
 // so one-byte pools keep plain K loads.  Mixing hinted and plain loads on the halves of one line is
-// worse than either (117.8 us).
-constexpr bool kNtK16 = true, kNtV16 = true, kNtK8 = false, kNtV8 = true;
+// worse than either (117.8 us).  A launch in which a wave slot has a single tile is bound by latency, not by
+// bandwidth, and runs 1.5 to 2 us slower with the hint (8 sequences x 1024 tokens: 14.1 -> 15.8 us), so
+// the planner switches the hint on (template parameter NT) only when every slot loops over two tiles or
+// more.  (Chosen per load by a wave-uniform run-time flag instead, the kernel ran six times slower.)
+#ifndef BZ_NT_MASK // build knob for A/B measurements: 1 = K of 16-bit pools, 8 = V of 16-bit pools, 4 / 2 = K / V of one-byte pools
+#define BZ_NT_MASK 11
+#endif
+constexpr bool kNtK16 = (BZ_NT_MASK & 1) != 0, kNtV16 = (BZ_NT_MASK & 8) != 0, kNtK8 = (BZ_NT_MASK & 4) != 0,
+               kNtV8 = (BZ_NT_MASK & 2) != 0;
 typedef unsigned int bz_u32x4_t __attribute__((ext_vector_type(4)));
 __device__ __forceinline__ uint4 ld_kv16(const char* p, bool nt) {
     if (nt) {
@@ -148,7 +155,8 @@ constexpr int kInfoInts = 12; // per-tile description kept in LDS (see fetch_inf
 // on their way to the matrix cores; the per-head scales are folded into the softmax scale and into
 // the final normalisation.  A lane then fetches 16 bytes = 16 elements of a K row, so the contraction
 // index of MFMA step ks, lane group j, element i is d = 64*(ks/2) + 16*j + 8*(ks%2) + i (q follows).
-template <bool BF16, typename OT, bool ROPE_Q, bool KV8>
+// NT: K/V loads carry the non-temporal hint (see kNtK16 above); chosen by the planner.
+template <bool BF16, typename OT, bool ROPE_Q, bool KV8, bool NT>
 __global__ __launch_bounds__(64, 2) void decode_mfma_kernel(MfmaDecodeArgs a, const char* __restrict__ q_ptr,
                                                             const char* __restrict__ k_data,
                                                             const char* __restrict__ v_data,
@@ -252,24 +260,24 @@ __global__ __launch_bounds__(64, 2) void decode_mfma_kernel(MfmaDecodeArgs a, co
         if constexpr (KV8) {
 #pragma unroll
             for (int p = 0; p < 2; ++p) { // 16 bytes feed MFMA steps 2p and 2p+1
-                kreg[0][p] = ld_kv16(k_data + base[0] + (size_t)n * row_bytes + p * 64 + j * 16, kNtK8);
-                kreg[1][p] = ld_kv16(k_data + base[1] + (size_t)n * row_bytes + p * 64 + j * 16, kNtK8);
+                kreg[0][p] = ld_kv16(k_data + base[0] + (size_t)n * row_bytes + p * 64 + j * 16, NT && kNtK8);
+                kreg[1][p] = ld_kv16(k_data + base[1] + (size_t)n * row_bytes + p * 64 + j * 16, NT && kNtK8);
             }
 #pragma unroll
             for (int w = 0; w < 4; ++w) { // rows 8w..8w+7 of the tile, 8 lanes x 16 B per 128-byte row
                 const int row = 8 * w + (lane >> 3);
-                vreg[w] = ld_kv16(v_data + base[row >> 4] + (size_t)(row & 15) * row_bytes + (lane & 7) * 16, kNtV8);
+                vreg[w] = ld_kv16(v_data + base[row >> 4] + (size_t)(row & 15) * row_bytes + (lane & 7) * 16, NT && kNtV8);
             }
         } else {
 #pragma unroll
             for (int ks = 0; ks < 4; ++ks) {
-                kreg[0][ks] = ld_kv16(k_data + base[0] + (size_t)n * row_bytes + ks * 64 + j * 16, kNtK16);
-                kreg[1][ks] = ld_kv16(k_data + base[1] + (size_t)n * row_bytes + ks * 64 + j * 16, kNtK16);
+                kreg[0][ks] = ld_kv16(k_data + base[0] + (size_t)n * row_bytes + ks * 64 + j * 16, NT && kNtK16);
+                kreg[1][ks] = ld_kv16(k_data + base[1] + (size_t)n * row_bytes + ks * 64 + j * 16, NT && kNtK16);
             }
 #pragma unroll
             for (int w = 0; w < 8; ++w) { // rows 4w..4w+3 of the tile, 16 lanes x 16 B per row
                 const int row = 4 * w + j;
-                vreg[w] = ld_kv16(v_data + base[row >> 4] + (size_t)(row & 15) * row_bytes + n * 16, kNtV16);
+                vreg[w] = ld_kv16(v_data + base[row >> 4] + (size_t)(row & 15) * row_bytes + n * 16, NT && kNtV16);
             }
         }
     };
@@ -612,8 +620,12 @@ struct DecodeArgs; // general-kernel argument block (bz_decode.hip); only its sc
 
 template <bool BF16, typename OT, bool ROPE_Q, bool KV8>
 static void launch_mfma_k(const DecodePlan* p, const MfmaDecodeArgs& a, hipStream_t s) {
-    hipLaunchKernelGGL((decode_mfma_kernel<BF16, OT, ROPE_Q, KV8>), dim3(p->mfma_slots), dim3(64), 0, s, a,
-                       (const char*)a.q, a.k_data, a.v_data, a.indices, a.pieces, a.tiles, a.heads);
+    if (p->mfma_streaming)
+        hipLaunchKernelGGL((decode_mfma_kernel<BF16, OT, ROPE_Q, KV8, true>), dim3(p->mfma_slots), dim3(64), 0, s, a,
+                           (const char*)a.q, a.k_data, a.v_data, a.indices, a.pieces, a.tiles, a.heads);
+    else
+        hipLaunchKernelGGL((decode_mfma_kernel<BF16, OT, ROPE_Q, KV8, false>), dim3(p->mfma_slots), dim3(64), 0, s, a,
+                           (const char*)a.q, a.k_data, a.v_data, a.indices, a.pieces, a.tiles, a.heads);
 }
 
 template <bool BF16, typename OT>

@@ -141,11 +141,14 @@ static int build_schedule(DecodePlan* p, const int32_t* indptr_h, const int32_t*
         if ((page_size & (page_size - 1)) == 0) { page_shift = 0; while ((1u << page_shift) < page_size) ++page_shift; }
         const uint64_t max_slots = (uint64_t)cus * 8;
         const uint64_t share = std::max<uint64_t>(1, (total_tiles + max_slots - 1) / max_slots);
+        p->mfma_streaming = share >= 2;
         const uint32_t cap_tiles = never_split ? 0x7fffffffu : std::max<uint32_t>(1, split_tokens / 32);
-        // Workgroups are dealt round-robin to the 8 XCDs, and on MI355X the odd XCDs stream HBM about
-        // a tenth slower than the even ones under full load (measured per wave with wall_clock64), so
-        // the slots that land on them get a smaller share.  BZ_DECODE_XCD_SKEW overrides the percentage.
-        double skew = 0.09;
+        // Workgroups are dealt round-robin to the 8 XCDs.  With plain K/V loads the odd XCDs streamed HBM
+        // about a tenth slower than the even ones under full load (measured per wave with wall_clock64)
+        // and a 9 % smaller share for their slots paid; with the non-temporal loads of the streaming
+        // kernel the difference is gone and equal shares are fastest (128 x 32/8 heads bf16: 107.8 us at
+        // 0 %, 108.7 at 3 %, 110.2 at 9 %, 108.3 at -4 %).  BZ_DECODE_XCD_SKEW sets the percentage.
+        double skew = 0.0;
         if (const char* e = getenv("BZ_DECODE_XCD_SKEW")) skew = atof(e) / 100.0;
         if (share < 8) skew = 0.0; // too few tiles per slot to express the difference
         const uint64_t nslots = std::min<uint64_t>(max_slots, (total_tiles + share - 1) / share);

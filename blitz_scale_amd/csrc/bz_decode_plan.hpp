@@ -100,6 +100,7 @@ struct DecodePlan {
     bool force_general = false; // tests: run the general kernel even where the MFMA path applies
     uint32_t mfma_slots = 0, mfma_combos = 0, mfma_partials = 0, mfma_pieces = 0, mfma_split_seqs = 0;
     uint32_t mfma_max_count = 0; // most partials any split (sequence, kv head) has
+    bool mfma_streaming = false; // every wave slot has two tiles or more (bandwidth-bound launch)
     uint32_t mfma_parts = 1;     // groups of more than 16 q heads are scheduled as this many equal parts per kv head
     const MfmaPiece* mfma_pieces_d = nullptr;
     const MfmaCombine* mfma_combos_d = nullptr;
