@@ -117,6 +117,8 @@ __device__ __forceinline__ uint32_t& pf_u4(uint4& v, int i) { return reinterpret
 
 // SPLIT_P: the probabilities enter the second contraction as head + tail of the storage type (two
 // MFMAs), used for bf16 whose 8-bit significand alone would eat the error budget.
+// XOR applied to the 16-byte chunk index of V rows in LDS, by row % 4: 0, 4, 10, 14 (see the staging comment)
+#define BZ_VSWZ(r) (((r) << 2) ^ (((r) >> 1) << 1))
 template <bool BF16, bool SPLIT_P>
 __global__ __launch_bounds__(256, 2) void prefill_kernel(PrefillArgs a, const char* __restrict__ q_ptr,
                                                          const char* __restrict__ k_ptr,
@@ -155,7 +157,11 @@ __global__ __launch_bounds__(256, 2) void prefill_kernel(PrefillArgs a, const ch
     // moves rows 16w .. 16w+15 of the tile with four instructions each for K and V.  What keeps the
     // operand reads free of bank conflicts is an XOR on the 16-byte column chunk instead of padding:
     //   K: chunk c of row r sits at position c ^ (r % 16)      (8 lanes read 8 rows, one chunk each)
-    //   V: chunk c of row r sits at position c ^ 2*(r % 4)     (a 16-lane group reads 4 rows x 32 B)
+    //   V: chunk c of row r sits at position c ^ g(r % 4), g = 0, 4, 10, 14.  The transposing read takes 8 B
+    //      per lane; a 16-lane group reads 4 rows x 32 B and two groups (32 lanes, 4 rows x 64 B) go through
+    //      the 64 banks together, so the 8 (row, group) pieces must land in 8 different 32-byte bank groups
+    //      (with c ^ 2*(r % 4), enough for 32 banks, the hardware counted a conflict on a third of the LDS
+    //      cycles; with g, 3.5 %)
     // and a lane of the copy simply fetches the chunk that belongs at its position.  Rows past the end
     // of the request re-read its last row (valid memory; masked later).
     const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) unsigned char*)smem;
@@ -165,7 +171,7 @@ __global__ __launch_bounds__(256, 2) void prefill_kernel(PrefillArgs a, const ch
     uint32_t kcol[4], kfast[4], vfast[4];
 #pragma unroll
     for (int i = 0; i < 4; ++i) kcol[i] = (uint32_t)((p16 ^ ((4 * i + r4) & 15)) * 16);
-    const uint32_t vcol = (uint32_t)((p16 ^ (r4 << 1)) * 16);
+    const uint32_t vcol = (uint32_t)((p16 ^ BZ_VSWZ(r4)) * 16);
 #pragma unroll
     for (int i = 0; i < 4; ++i) { // lane offsets of copy i inside the wave's 16 rows when no row needs clamping,
                                   // less the i KiB that the instruction offset of the grouped copy adds back
@@ -217,7 +223,7 @@ __global__ __launch_bounds__(256, 2) void prefill_kernel(PrefillArgs a, const ch
             asm volatile("" : "+v"(koff[ks])); // keep the sum: the compiler would re-add the base on every tile
         }
         const int srow = (lane & 15) >> 2;
-        const int zl = ((((lane >> 4) & 1) << 1) | ((lane & 3) >> 1)) ^ (srow << 1);
+        const int zl = ((((lane >> 4) & 1) << 1) | ((lane & 3) >> 1)) ^ BZ_VSWZ(srow);
 #pragma unroll
         for (int db = 0; db < 4; ++db) {
             voff[db] = lds0 + (uint32_t)((4 * h + srow) * 256 + ((((db << 2)) ^ zl) * 16) + (lane & 1) * 8);
