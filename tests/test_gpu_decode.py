@@ -124,6 +124,18 @@ def test_e4m3_kv_pool():
     check(p, f32_tol=2e-5, parallel=True)
 
 
+@pytest.mark.parametrize("batch", [12, 24])
+@pytest.mark.parametrize("dtype,kv_dtype,rope_mode", [(BZ_F16, None, BZ_ROPE_NONE), (BZ_BF16, None, BZ_ROPE_Q_ONLY),
+                                                       (BZ_F16, BZ_E4M3, BZ_ROPE_NONE), (BZ_BF16, BZ_E4M3, BZ_ROPE_Q_ONLY)])
+def test_both_sides_of_the_streaming_threshold(batch, dtype, kv_dtype, rope_mode):
+    """The planner picks the kernel instantiation whose K/V loads carry the non-temporal hint once every
+    wave slot has two tiles or more.  12 and 24 sequences of 512 tokens on 8 kv heads are 1 536 and 3 072
+    tiles, i.e. one tile per slot (plain loads) and two (hinted loads) on 256 compute units."""
+    ctx = [512] * (batch - 1) + [497]
+    p = DecodeProblem(40 + batch, ctx, 16, 8, 128, 16, dtype, kv_dtype=kv_dtype)
+    check(p, rope_mode=rope_mode, theta=5e5, f32_tol=1e-4, parallel=True)
+
+
 def test_c2_shape_reduced_batch():
     """Llama-2-7B MHA decode shape (32/32 heads, D 128, fp16, ctx U[512,2048]) at batch 8, q rotated in-kernel."""
     rng = np.random.default_rng(wl.DEFAULT_SEED)
