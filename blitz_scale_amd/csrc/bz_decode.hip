@@ -4,6 +4,7 @@
 // BlitzScale worker.
 #include <cmath>
 #include <algorithm>
+#include <mutex>
 #include <vector>
 #include <new>
 
@@ -286,9 +287,10 @@ static int launch_general_kv(const DecodeArgs& a, int kv_dtype, int q_dtype, int
 }
 
 template <typename OT>
-static void launch_combine(const DecodePlan* p, void* out, float* lse, uint32_t Hq, uint32_t D, hipStream_t s) {
-    hipLaunchKernelGGL((decode_combine_kernel<OT>), dim3(p->num_combos, Hq), dim3(D), 0, s, p->combos_d, p->part_o,
-                       p->part_lse, out, lse, Hq, D);
+static void launch_combine(const DecodePlan* p, const float* part_o, const float* part_lse, void* out, float* lse,
+                           uint32_t Hq, uint32_t D, hipStream_t s) {
+    hipLaunchKernelGGL((decode_combine_kernel<OT>), dim3(p->num_combos, Hq), dim3(D), 0, s, p->combos_d, part_o,
+                       part_lse, out, lse, Hq, D);
 }
 template <typename OT>
 static void launch_zero(const DecodePlan* p, void* out, uint32_t row_elems, hipStream_t s) {
@@ -297,18 +299,21 @@ static void launch_zero(const DecodePlan* p, void* out, uint32_t row_elems, hipS
 
 int decode_fast_path(const DecodePlan* p, const void* q, void* out, float* lse, int q_dtype, int out_dtype,
                      int rope_mode, float sm_scale_log2, const RopeFreqs& freqs, const bz_paged_kv_t* kv,
-                     uint32_t num_qo_heads, const float* k_scale, const float* v_scale,
-                     hipStream_t s); // bz_decode_mfma.hip
+                     uint32_t num_qo_heads, const float* k_scale, const float* v_scale, float* part_o,
+                     float* part_lse, hipStream_t s); // bz_decode_mfma.hip
 
-} // namespace bz
+// Where the split-K partial results of one call live: the plan's float workspace (bz_batch_decode) or the
+// library's own device array (bz_batch_decode_noalloc).  The two kernels never run in the same call, so
+// both pairs may point at the same memory.
+struct PartialBufs {
+    float *part_o, *part_lse;           // general kernel: [partials][Hq][D], [partials][Hq]
+    float *mfma_part_o, *mfma_part_lse; // matrix-core kernel: [partials][16][128], [partials][16]
+};
 
-using namespace bz;
-
-extern "C" int bz_batch_decode(bz_decode_plan_t* plan_, const void* q, int q_dtype, const bz_paged_kv_t* kv,
-                               void* out, int out_dtype, uint32_t num_qo_heads, int rope_mode, float rope_theta,
-                               float sm_scale, const float* k_scale, const float* v_scale, float* lse,
-                               void* stream) {
-    DecodePlan* p = reinterpret_cast<DecodePlan*>(plan_);
+static int batch_decode_impl(DecodePlan* p, const void* q, int q_dtype, const bz_paged_kv_t* kv, void* out,
+                             int out_dtype, uint32_t num_qo_heads, int rope_mode, float rope_theta, float sm_scale,
+                             const float* k_scale, const float* v_scale, float* lse, const PartialBufs* bufs_or_null,
+                             void* stream) {
     if (!p || !kv || !q || !out) return BZ_ERR_BAD_ARG;
     if (!p->planned) return BZ_ERR_NOT_PLANNED;
     // a table whose device pointers were cleared after the previous step (src/blitz/stub.h:1361-1363)
@@ -326,6 +331,8 @@ extern "C" int bz_batch_decode(bz_decode_plan_t* plan_, const void* q, int q_dty
     const int D = (int)kv->head_dim, G = (int)(num_qo_heads / kv->num_kv_heads);
     hipStream_t s = (hipStream_t)stream;
     if (p->batch_size == 0) return 0;
+    const PartialBufs from_plan = {p->part_o, p->part_lse, p->mfma_part_o, p->mfma_part_lse};
+    const PartialBufs& bufs = bufs_or_null ? *bufs_or_null : from_plan;
 
     DecodeArgs a;
     a.q = q; a.out = out; a.lse = lse;
@@ -333,7 +340,7 @@ extern "C" int bz_batch_decode(bz_decode_plan_t* plan_, const void* q, int q_dty
     a.indices = kv->indices; a.indptr = kv->indptr; a.last_page_len = kv->last_page_len;
     a.steps_ahead = kv->steps_ahead;
     a.segments = p->segments_d;
-    a.part_o = p->part_o; a.part_lse = p->part_lse;
+    a.part_o = bufs.part_o; a.part_lse = bufs.part_lse;
     a.k_scale = k_scale; a.v_scale = v_scale;
     a.stride_page = kv->stride_page; a.stride_n = kv->stride_n; a.stride_h = kv->stride_h;
     a.page_size = kv->page_size; a.num_qo_heads = num_qo_heads; a.num_kv_heads = kv->num_kv_heads;
@@ -347,7 +354,7 @@ extern "C" int bz_batch_decode(bz_decode_plan_t* plan_, const void* q, int q_dty
         int rc = BZ_ERR_UNSUPPORTED;
         if (!p->force_general)
             rc = decode_fast_path(p, q, out, lse, q_dtype, out_dtype, rope_mode, a.sm_scale_log2, a.freqs, kv,
-                                  num_qo_heads, k_scale, v_scale, s);
+                                  num_qo_heads, k_scale, v_scale, bufs.mfma_part_o, bufs.mfma_part_lse, s);
         if (rc == 0) {
             // the MFMA path brings its own combine; only empty sequences are left to do
             if (p->num_empty > 0) {
@@ -378,9 +385,9 @@ extern "C" int bz_batch_decode(bz_decode_plan_t* plan_, const void* q, int q_dty
         if (rc) return rc;
     }
     if (p->num_combos > 0) {
-        if (out_dtype == BZ_F32) launch_combine<float>(p, out, lse, num_qo_heads, D, s);
-        else if (out_dtype == BZ_F16) launch_combine<f16_t>(p, out, lse, num_qo_heads, D, s);
-        else launch_combine<bf16_t>(p, out, lse, num_qo_heads, D, s);
+        if (out_dtype == BZ_F32) launch_combine<float>(p, bufs.part_o, bufs.part_lse, out, lse, num_qo_heads, D, s);
+        else if (out_dtype == BZ_F16) launch_combine<f16_t>(p, bufs.part_o, bufs.part_lse, out, lse, num_qo_heads, D, s);
+        else launch_combine<bf16_t>(p, bufs.part_o, bufs.part_lse, out, lse, num_qo_heads, D, s);
         BZ_LAUNCH_CHECK();
     }
     if (p->num_empty > 0) {
@@ -391,4 +398,77 @@ extern "C" int bz_batch_decode(bz_decode_plan_t* plan_, const void* q, int q_dty
         BZ_LAUNCH_CHECK();
     }
     return 0;
+}
+
+} // namespace bz
+
+using namespace bz;
+
+// ------------------------------------------------------------------------------------------
+// The library's own split-K scratch: a fixed device array that exists from module load to process
+// exit, one copy per GPU.  Host code never passes the array's name to a kernel (on the host it is a
+// stand-in, not a device address): the address is looked up once per device and kept.
+// ------------------------------------------------------------------------------------------
+static __device__ __align__(256) unsigned char bz_decode_scratch[BZ_DECODE_NOALLOC_SCRATCH_BYTES];
+
+namespace bz {
+
+constexpr int kMaxDevices = 64;
+static std::mutex g_scratch_mutex;
+static void* g_scratch_ptr[kMaxDevices] = {nullptr};
+
+// Device address of this GPU's copy of the scratch array (looked up on the first call per device,
+// with that device current).
+static int decode_scratch_for_current_device(unsigned char** ptr) {
+    int dev = 0;
+    BZ_CHECK_HIP(hipGetDevice(&dev));
+    if (dev < 0 || dev >= kMaxDevices) return BZ_ERR_UNSUPPORTED;
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (!g_scratch_ptr[dev]) {
+        void* sym = nullptr;
+        BZ_CHECK_HIP(hipGetSymbolAddress(&sym, HIP_SYMBOL(bz_decode_scratch)));
+        if (!sym) return BZ_ERR_BAD_ARG;
+        g_scratch_ptr[dev] = sym;
+    }
+    *ptr = static_cast<unsigned char*>(g_scratch_ptr[dev]);
+    return 0;
+}
+
+static inline size_t scratch_align(size_t x) { return (x + 255) / 256 * 256; }
+
+} // namespace bz
+
+extern "C" int bz_batch_decode(bz_decode_plan_t* plan_, const void* q, int q_dtype, const bz_paged_kv_t* kv,
+                               void* out, int out_dtype, uint32_t num_qo_heads, int rope_mode, float rope_theta,
+                               float sm_scale, const float* k_scale, const float* v_scale, float* lse,
+                               void* stream) {
+    return batch_decode_impl(reinterpret_cast<DecodePlan*>(plan_), q, q_dtype, kv, out, out_dtype, num_qo_heads,
+                             rope_mode, rope_theta, sm_scale, k_scale, v_scale, lse, nullptr, stream);
+}
+
+extern "C" size_t bz_batch_decode_noalloc_scratch_bytes(void) { return BZ_DECODE_NOALLOC_SCRATCH_BYTES; }
+
+extern "C" int bz_batch_decode_noalloc(bz_decode_plan_t* plan_, const void* q, int q_dtype, const bz_paged_kv_t* kv,
+                                       void* out, int out_dtype, uint32_t num_qo_heads, int rope_mode,
+                                       float rope_theta, float sm_scale, const float* k_scale, const float* v_scale,
+                                       float* lse, void* stream) {
+    DecodePlan* p = reinterpret_cast<DecodePlan*>(plan_);
+    if (!p) return BZ_ERR_BAD_ARG;
+    if (!p->planned) return BZ_ERR_NOT_PLANNED;
+    // partial results of whichever kernel the call ends up running must fit the fixed array
+    const size_t gen_o = scratch_align((size_t)p->num_partials * p->num_qo_heads * p->head_dim * sizeof(float));
+    const size_t gen_l = scratch_align((size_t)p->num_partials * p->num_qo_heads * sizeof(float));
+    const size_t mf_o = p->mfma_ok ? scratch_align((size_t)p->mfma_partials * 16 * 128 * sizeof(float)) : 0;
+    const size_t mf_l = p->mfma_ok ? scratch_align((size_t)p->mfma_partials * 16 * sizeof(float)) : 0;
+    if (gen_o + gen_l > (size_t)BZ_DECODE_NOALLOC_SCRATCH_BYTES || mf_o + mf_l > (size_t)BZ_DECODE_NOALLOC_SCRATCH_BYTES)
+        return BZ_ERR_WORKSPACE;
+    unsigned char* base = nullptr;
+    const int rc = decode_scratch_for_current_device(&base);
+    if (rc) return rc;
+    // every partial row that the combine reads is written by the decode kernel of the same call first,
+    // so nothing in the array has to start at zero
+    const PartialBufs bufs = {reinterpret_cast<float*>(base), reinterpret_cast<float*>(base + gen_o),
+                              reinterpret_cast<float*>(base), reinterpret_cast<float*>(base + mf_o)};
+    return batch_decode_impl(p, q, q_dtype, kv, out, out_dtype, num_qo_heads, rope_mode, rope_theta, sm_scale, k_scale,
+                             v_scale, lse, &bufs, stream);
 }

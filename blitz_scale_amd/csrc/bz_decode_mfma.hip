@@ -658,7 +658,8 @@ static int launch_mfma(const DecodePlan* p, const MfmaDecodeArgs& a, bool kv8, h
 
 int decode_fast_path(const DecodePlan* p, const void* q, void* out, float* lse, int q_dtype, int out_dtype,
                      int rope_mode, float sm_scale_log2, const RopeFreqs& freqs, const bz_paged_kv_t* kv,
-                     uint32_t num_qo_heads, const float* k_scale, const float* v_scale, hipStream_t s) {
+                     uint32_t num_qo_heads, const float* k_scale, const float* v_scale, float* part_o,
+                     float* part_lse, hipStream_t s) {
     if (!p->mfma_ok || p->mfma_slots == 0) return BZ_ERR_UNSUPPORTED;
     const bool kv8 = kv->kv_dtype == BZ_E4M3;
     if ((!kv8 && kv->kv_dtype != q_dtype) || rope_mode == BZ_ROPE_FULL) return BZ_ERR_UNSUPPORTED;
@@ -672,7 +673,7 @@ int decode_fast_path(const DecodePlan* p, const void* q, void* out, float* lse, 
     a.indices = kv->indices; a.indptr = kv->indptr; a.last_page_len = kv->last_page_len;
     a.steps_ahead = kv->steps_ahead;
     a.pieces = p->mfma_pieces_d; a.tiles = p->mfma_tiles_d; a.heads = p->mfma_heads_d;
-    a.part_o = p->mfma_part_o; a.part_lse = p->mfma_part_lse;
+    a.part_o = part_o; a.part_lse = part_lse; // split-K partials: the plan's float workspace or the library's own array
     a.stride_page = kv->stride_page; a.stride_n = kv->stride_n; a.stride_h = kv->stride_h;
     a.page_size = kv->page_size; a.num_qo_heads = num_qo_heads;
     a.group = num_qo_heads / kv->num_kv_heads / p->mfma_parts;

@@ -229,6 +229,17 @@ def batch_decode_attention(handler, q_input, paged_kv, output, num_qo_heads, *, 
     check(rc, "batchDecodeAttention")
 
 
+def batch_decode_attention_noalloc(handler, q_input, paged_kv, output, num_qo_heads, *, rope_mode=BZ_ROPE_Q_ONLY,
+                                   rope_theta=1e4, sm_scale=0.0, k_scale=None, v_scale=None, lse=None, stream=None):
+    """batch_decode_attention with the split-K partials in the library's own fixed device array instead of
+    the plan's float workspace: the call allocates nothing (no counterpart in the reference)."""
+    s = paged_kv.as_struct()
+    rc = _lib.load().bz_batch_decode_noalloc(handler.get(), _ptr(q_input), bz_dtype(q_input), C.byref(s),
+                                             _ptr(output), bz_dtype(output), num_qo_heads, rope_mode, rope_theta,
+                                             sm_scale, _ptr(k_scale), _ptr(v_scale), _ptr(lse), _stream(stream))
+    check(rc, "batchDecodeAttention")
+
+
 def batch_prefill_attention(handler, q_input, qo_indptr, k_input, v_input, kv_indptr, output, batch_size,
                             num_qo_heads, num_kv_heads, head_size, *, causal=True, rope_mode=BZ_ROPE_NONE,
                             rope_theta=1e4, sm_scale=0.0, stream=None):

@@ -153,6 +153,26 @@ int bz_batch_decode(bz_decode_plan_t* plan, const void* q, int q_dtype, const bz
                     int out_dtype, uint32_t num_qo_heads, int rope_mode, float rope_theta, float sm_scale,
                     const float* k_scale, const float* v_scale, float* lse, void* stream);
 
+/*
+ * bz_batch_decode for callers that cannot allocate device memory or bring a float workspace along (code
+ * under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc).  No counterpart in the
+ * reference.  Same arguments, same kernels and bit-identical results as bz_batch_decode on the same plan,
+ * except that the split-K partial results go to a fixed device array inside the library
+ * (BZ_DECODE_NOALLOC_SCRATCH_BYTES per GPU, held from module load to process exit) instead of the float
+ * workspace given to bz_decode_plan; that workspace is not touched by this call.  The call itself performs
+ * no allocation, free, copy or synchronisation: it only launches kernels on `stream`.
+ * Limit: the plan's partial results must fit the array (8256 bytes per partial of the matrix-core kernel,
+ * 4*(head_dim+1)*num_qo_heads per partial of the general kernel); otherwise BZ_ERR_WORKSPACE is returned
+ * before anything is launched.  All calls on one GPU share that GPU's array: calls that overlap in time on
+ * one GPU (two streams, two threads) race; calls in stream order are safe, and nothing in the array has to
+ * be cleared between them (every partial the combine reads is written by the same call first).
+ */
+#define BZ_DECODE_NOALLOC_SCRATCH_BYTES (32u << 20)
+size_t bz_batch_decode_noalloc_scratch_bytes(void);
+int bz_batch_decode_noalloc(bz_decode_plan_t* plan, const void* q, int q_dtype, const bz_paged_kv_t* kv, void* out,
+                            int out_dtype, uint32_t num_qo_heads, int rope_mode, float rope_theta, float sm_scale,
+                            const float* k_scale, const float* v_scale, float* lse, void* stream);
+
 /* ---------------------------------------------------------------------------------------
  * Prefill plan: replaces BatchPrefillRaggedHandler::plan (flashinfer_types.h:12-41,
  * flashinfer_types.cu:24-49).  Builds the (request, q-tile) work list, longest first.
