@@ -13,6 +13,7 @@ LIB_PATH = os.environ.get("BZ_HIP_LIB") or os.path.join(HERE, "lib", "libbz_hip.
 BZ_F16, BZ_BF16, BZ_E4M3, BZ_F32 = 0, 1, 2, 3
 BZ_ROPE_NONE, BZ_ROPE_Q_ONLY, BZ_ROPE_FULL = 0, 1, 2
 BZ_LAYOUT_NHD, BZ_LAYOUT_HND = 0, 1
+BZ_NUM_TOKENS_FROM_INDPTR = 0xFFFFFFFF
 BZ_ERR_BAD_ARG, BZ_ERR_UNSUPPORTED, BZ_ERR_WORKSPACE, BZ_ERR_NOT_PLANNED, BZ_ERR_NO_PAGES = 10001, 10002, 10003, 10004, 10005
 
 

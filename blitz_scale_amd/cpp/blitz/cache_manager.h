@@ -71,6 +71,9 @@ class CacheManager {
         assert(needed_blocks_slots.size() + 1 == indptr.size());
         assert(needed_blocks_slots.size() == last_page_len.size());
         const std::vector<IdType> fresh = first_fit(num_blocks); // throws before anything is marked
+        // so does a table too large for its pinned chunk: checked here, before pages and the chunk are taken
+        if ((indices.size() + num_blocks + indptr.size() + last_page_len.size()) * sizeof(IdType) > chunk_bytes_)
+            throw std::runtime_error("page table does not fit its pinned chunk");
         const int meta = take_meta_slot();
         if (meta < 0) throw std::runtime_error("no free page-table chunk");
         *pinned_memory_idx = meta;
@@ -98,6 +101,8 @@ class CacheManager {
         for (size_t i = 0; i < B; ++i)
             if (last_page_len[i] == (IdType)page_size_) full.push_back(i);
         const std::vector<IdType> fresh = first_fit(full.size()); // all or nothing
+        if ((indices.size() + full.size() + indptr.size() + last_page_len.size()) * sizeof(IdType) > chunk_bytes_)
+            throw std::runtime_error("page table does not fit its pinned chunk");
         for (size_t i = 0; i < B; ++i)
             if (last_page_len[i] != (IdType)page_size_) last_page_len[i] += 1;
         if (full.empty()) {

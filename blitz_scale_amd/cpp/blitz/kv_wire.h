@@ -41,7 +41,7 @@ class KvWire {
         const bz_paged_kv_t kv = page_table.c_view();
         kernel::bz_throw(bz_kv_pages_pack(kv_data_, max_num_pages_, &kv, reinterpret_cast<const int32_t*>(page_ids_d),
                                           num_pages, start_layer, layer_cnt, wire, wire_dtype, k_scale, v_scale,
-                                          kernel::attention_options().stream),
+                                          page_table.opts().stream),
                          "PackKVPages");
     }
 
@@ -56,7 +56,7 @@ class KvWire {
         kernel::bz_throw(bz_kv_pages_unpack(kv_data_, max_num_pages_, &kv,
                                             reinterpret_cast<const int32_t*>(page_ids_d), num_pages, start_layer,
                                             layer_cnt, wire, wire_dtype, k_scale, v_scale,
-                                            kernel::attention_options().stream),
+                                            page_table.opts().stream),
                          "UnpackKVPages");
     }
 

@@ -7,29 +7,33 @@
 
 namespace blitz::kernel {
 
-/// src/kernel/attention.h:9-22.  Ragged causal self-attention; q and k are expected rotated already
-/// (store_prefill_kv_cache does it together with the page store) unless rope_in_call is set, in which
-/// case q and k are rotated in place here first.
+/// src/kernel/attention.h:9-22.  Ragged causal self-attention over q [N,Hq,D], k,v [N,Hkv,D].
+/// rope_mode < 0 takes handler.options.prefill_rope_mode, whose default BZ_ROPE_FULL is the reference's
+/// kRoPELlama (attention_prefill.cu:38): q and k rows are rotated by their offset inside the request, IN
+/// PLACE in the caller's buffers, before the contraction; k then holds what the cache must hold, and
+/// store_prefill_kv_cache that follows (src/layer/attn.h:188-193) must not rotate it again (its default).
+/// BZ_ROPE_NONE: q and k are used as they are (they were rotated while the pages were written).
 template<typename DType, typename IdType>
 void batch_prefill_attention(BatchPrefillRaggedHandler<DType, IdType>& handler, DType* q_input, IdType* qo_indptr,
                              DType* k_input, DType* v_input, IdType* kv_indptr, DType* output, uint32_t batch_size,
-                             uint32_t num_qo_heads, uint32_t num_kv_heads, uint32_t head_size,
-                             bool rope_in_call = false) {
-    const AttentionOptions& o = attention_options();
+                             uint32_t num_qo_heads, uint32_t num_kv_heads, uint32_t head_size, int rope_mode = -1) {
+    const AttentionOptions& o = handler.options;
     bz_throw(bz_batch_prefill_ragged(static_cast<bz_prefill_plan_t*>(handler.get()), q_input,
                                      reinterpret_cast<const int32_t*>(qo_indptr), k_input, v_input,
                                      reinterpret_cast<const int32_t*>(kv_indptr), output, bz_dtype<DType>::value,
                                      batch_size, num_qo_heads, num_kv_heads, head_size, /*causal=*/1,
-                                     rope_in_call ? BZ_ROPE_FULL : BZ_ROPE_NONE, o.rope_theta, o.sm_scale, o.stream),
+                                     rope_mode < 0 ? o.prefill_rope_mode : rope_mode, o.rope_theta, o.sm_scale, o.stream),
              "BatchPrefillWithRaggedKVCache");
 }
 
-/// src/kernel/attention.h:24-31.  q, output: [batch, num_qo_heads, head_size].
+/// src/kernel/attention.h:24-31.  q, output: [batch, num_qo_heads, head_size].  rope_mode < 0 takes
+/// handler.options.decode_rope_mode (default BZ_ROPE_Q_ONLY: q is rotated at position seq_len-1 inside the
+/// kernel, the caller's q stays as it is; cached K is rotated already).
 template<typename DType, typename IdType, typename KVType = DType>
 void batch_decode_attention(BlitzBatchDecodeHandler<DType, IdType>& handler, DType* q_input,
                             PageTable<KVType, IdType>& paged_kv, DType* output, const uint32_t num_qo_heads,
                             int rope_mode = -1, const float* k_scale = nullptr, const float* v_scale = nullptr) {
-    const AttentionOptions& o = attention_options();
+    const AttentionOptions& o = handler.options;
     const bz_paged_kv_t kv = paged_kv.c_view();
     bz_throw(bz_batch_decode(static_cast<bz_decode_plan_t*>(handler.get()), q_input, bz_dtype<DType>::value, &kv, output,
                              bz_dtype<DType>::value, num_qo_heads, rope_mode < 0 ? o.decode_rope_mode : rope_mode,

@@ -27,20 +27,36 @@ inline void bz_throw(int status, const char* what) {
     if (status != 0) throw std::runtime_error(std::string(what) + " error: " + bz_error_string(status));
 }
 
-/// Parameters the reference never passes (FlashInfer defaults apply there): RoPE base, softmax
-/// scale, RoPE handling and the stream.  One process-wide default keeps the reference's call
-/// signatures unchanged; a serving engine sets it once from the model config.
+/// Parameters the reference never passes (FlashInfer defaults apply there): RoPE base, softmax scale,
+/// where RoPE is applied, and the stream.  They travel with the objects the reference's calls already
+/// take -- every handler (BatchPrefillRaggedHandler, BlitzBatchDecodeHandler) holds its own copy and a
+/// PageTable may point at one -- so two models, or two host threads on two streams, do not share them;
+/// attention_options() is only the process-wide default a new handler starts from.
+///
+/// The RoPE defaults give the reference's kRoPELlama results (attention_prefill.cu:38,
+/// attention_decode.cu:35) under the reference's own call order (src/layer/attn.h:173-204) with K cached
+/// rotated:
+///   prefill: batch_prefill_attention rotates q and k (in place, in the caller's activation buffers),
+///            store_prefill_kv_cache then stores k as it finds it;
+///   decode : append_decode_kv_cache rotates the new K row on its way into the cache,
+///            batch_decode_attention rotates q inside the kernel and reads cached K as stored.
 struct AttentionOptions {
-    float rope_theta = 1e4f;          // Llama-2; Llama-3 uses 5e5
-    float sm_scale = 0.f;             // <= 0: 1/sqrt(head_dim)
-    int decode_rope_mode = BZ_ROPE_Q_ONLY;  // K is cached rotated (append/store rotate it)
-    bool rotate_k_on_write = true;    // append_decode_kv_cache / store_prefill_kv_cache rotate K
-    uint32_t split_tokens = 0;        // 0: library default (2048)
-    void* stream = nullptr;           // legacy default stream, as the reference
+    float rope_theta = 1e4f;                // Llama-2; Llama-3 uses 5e5
+    float sm_scale = 0.f;                   // <= 0: 1/sqrt(head_dim)
+    int prefill_rope_mode = BZ_ROPE_FULL;   // batch_prefill_attention: rotate q and k rows before the contraction
+    bool store_rotates_k = false;           // store_prefill_kv_cache: k was rotated by the attention call before it
+    bool append_rotates_k = true;           // append_decode_kv_cache rotates the new K row
+    int decode_rope_mode = BZ_ROPE_Q_ONLY;  // batch_decode_attention: rotate q only, cached K is rotated
+    uint32_t split_tokens = 0;              // 0: library default (2048)
+    void* stream = nullptr;                 // hipStream_t; nullptr = the legacy default stream the reference uses
 };
 inline AttentionOptions& attention_options() {
     static AttentionOptions opts;
     return opts;
 }
+
+/// "no stream argument given": the element-wise wrappers then launch on attention_options().stream
+inline void* const kStreamFromOptions = reinterpret_cast<void*>(~static_cast<uintptr_t>(0));
+inline void* resolve_stream(void* stream) { return stream == kStreamFromOptions ? attention_options().stream : stream; }
 
 } // namespace blitz::kernel

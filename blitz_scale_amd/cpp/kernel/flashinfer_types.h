@@ -19,12 +19,16 @@ class BatchPrefillRaggedHandler {
         bz_throw(bz_prefill_plan(static_cast<bz_prefill_plan_t*>(handler_), float_buffer, float_buffer_size, int_buffer,
                                  int_buffer_size, reinterpret_cast<const int32_t*>(qo_indptr_h),
                                  reinterpret_cast<const int32_t*>(kv_indptr_h), batch_size, num_qo_heads, num_kv_heads,
-                                 head_dim, page_size, attention_options().stream),
+                                 head_dim, page_size, options.stream),
                  "Handler plan:");
     }
     BatchPrefillRaggedHandler(void* handler_ptr = nullptr) : handler_(handler_ptr) {}
     void* get() noexcept { return handler_; }
     bool empty() noexcept { return handler_ == nullptr; }
+
+    /// RoPE base, softmax scale, RoPE placement and stream of the calls made through this handler
+    /// (a copy of the process-wide default at construction; set per model / per thread)
+    AttentionOptions options = attention_options();
 
   private:
     void* handler_;
@@ -37,7 +41,7 @@ class BlitzBatchDecodeHandler {
     void plan(void* float_buffer, size_t float_buffer_size, void* int_buffer, size_t int_buffer_size,
               IdType* qo_indptr_h, IdType* last_page_len_h, uint32_t batch_size, uint32_t num_qo_heads,
               uint32_t num_kv_heads, uint32_t head_dim, uint32_t page_size) {
-        const AttentionOptions& o = attention_options();
+        const AttentionOptions& o = options;
         bz_throw(bz_decode_plan(static_cast<bz_decode_plan_t*>(handler_), float_buffer, float_buffer_size, int_buffer,
                                 int_buffer_size, reinterpret_cast<const int32_t*>(qo_indptr_h),
                                 reinterpret_cast<const int32_t*>(last_page_len_h), batch_size, num_qo_heads,
@@ -47,6 +51,9 @@ class BlitzBatchDecodeHandler {
     BlitzBatchDecodeHandler(void* handler_ptr = nullptr) : handler_(handler_ptr) {}
     void* get() noexcept { return handler_; }
     bool empty() noexcept { return handler_ == nullptr; }
+
+    /// as for the prefill handler: this handler's own copy of the options
+    AttentionOptions options = attention_options();
 
   private:
     void* handler_;

@@ -45,6 +45,10 @@ struct PageTable {
     // optional device counter: the table describes the batch this many decode steps ahead of the present
     // (pages of the tokens to come already listed); nullptr = the table is the present
     IdType* steps_ahead_d = nullptr;
+    // RoPE base / placement and stream of the page writes made through this table: the model's own
+    // (e.g. &decode_handler.options), or nullptr = the process-wide default
+    const AttentionOptions* options = nullptr;
+    const AttentionOptions& opts() const { return options ? *options : attention_options(); }
 
     PageTable(uint32_t batch_size_, uint32_t page_size_, uint32_t num_heads_, uint32_t head_size_, DType* base_ptr,
               int layout_ = BZ_LAYOUT_HND) :
@@ -74,32 +78,52 @@ struct PageTable {
     }
 };
 
-/// src/kernel/page.h:66-67.  Token t of request b goes to page indices[indptr[b] + t/P], slot t%P.
-/// q (optional) is rotated in place with the same angles when K is rotated on the way in.
+/// Token t of request b goes to page indices[indptr[b] + t/P], slot t%P (src/kernel/page.cu:21-62).
+/// num_tokens: rows of k_data / v_data.  q_inout (optional, [N, num_qo_heads, D]): the fused RoPE of the
+/// prefill path -- K is rotated on its way into the pages and q and the caller's k rows are rotated in
+/// place by the same angles, so that batch_prefill_attention runs with BZ_ROPE_NONE afterwards.
+/// rotate: 1 / 0 force K rotation on / off, < 0 = on when q_inout is given, else opts().store_rotates_k.
 template<typename DType, typename IdType, typename SrcType = DType>
 void store_prefill_kv_cache(PageTable<DType, IdType>& page_table, SrcType* k_data, SrcType* v_data,
                             IdType* ragged_indptr, uint32_t num_tokens, SrcType* q_inout = nullptr,
                             uint32_t num_qo_heads = 0, const float* k_scale = nullptr,
-                            const float* v_scale = nullptr) {
+                            const float* v_scale = nullptr, int rotate = -1) {
     static_assert(sizeof(IdType) == 4, "page tables are int32");
-    const AttentionOptions& o = attention_options();
+    const AttentionOptions& o = page_table.opts();
     const bz_paged_kv_t kv = page_table.c_view();
+    const bool rot = rotate < 0 ? (q_inout != nullptr || o.store_rotates_k) : rotate != 0;
     bz_throw(bz_store_prefill_kv(&kv, k_data, v_data, bz_dtype<SrcType>::value,
                                  reinterpret_cast<const int32_t*>(ragged_indptr), num_tokens, q_inout, num_qo_heads,
-                                 o.rotate_k_on_write ? 1 : 0, o.rope_theta, k_scale, v_scale, o.stream),
+                                 rot ? 1 : 0, o.rope_theta, k_scale, v_scale, o.stream),
              "AppendPagedKVCache");
 }
 
-/// src/kernel/page.h:69-70.  One new row per sequence at position seq_len-1.
+/// src/kernel/page.h:66-67, the reference's own four arguments (called at src/layer/attn.h:188-193 right
+/// after batch_prefill_attention).  The token count is read on the device from ragged_indptr[batch_size],
+/// like the reference's launch, which is shaped by page size and batch alone (page.cu:84-89).  K is stored
+/// as it is found unless opts().store_rotates_k says otherwise: under the reference's call order the
+/// attention call has rotated it already.
+template<typename DType, typename IdType, typename SrcType = DType>
+void store_prefill_kv_cache(PageTable<DType, IdType>& page_table, SrcType* k_data, SrcType* v_data,
+                            IdType* ragged_indptr) {
+    store_prefill_kv_cache(page_table, k_data, v_data, ragged_indptr, BZ_NUM_TOKENS_FROM_INDPTR);
+}
+
+/// src/kernel/page.h:69-70.  One new row per sequence at position seq_len-1.  With the reference's three
+/// arguments the new K row is rotated on its way in (opts().append_rotates_k) and nothing else is touched;
+/// q_inout (optional, [B, num_qo_heads, D]) is the fused form: q is rotated in place as well, and
+/// batch_decode_attention runs with BZ_ROPE_NONE afterwards.
+/// rotate: 1 / 0 force K rotation on / off, < 0 = on when q_inout is given, else opts().append_rotates_k.
 template<typename DType, typename IdType, typename SrcType = DType>
 void append_decode_kv_cache(PageTable<DType, IdType>& page_table, SrcType* k_data, SrcType* v_data,
                             SrcType* q_inout = nullptr, uint32_t num_qo_heads = 0, const float* k_scale = nullptr,
-                            const float* v_scale = nullptr) {
+                            const float* v_scale = nullptr, int rotate = -1) {
     static_assert(sizeof(IdType) == 4, "page tables are int32");
-    const AttentionOptions& o = attention_options();
+    const AttentionOptions& o = page_table.opts();
     const bz_paged_kv_t kv = page_table.c_view();
-    bz_throw(bz_append_decode_kv(&kv, k_data, v_data, bz_dtype<SrcType>::value, q_inout, num_qo_heads,
-                                 o.rotate_k_on_write ? 1 : 0, o.rope_theta, k_scale, v_scale, o.stream),
+    const bool rot = rotate < 0 ? (q_inout != nullptr || o.append_rotates_k) : rotate != 0;
+    bz_throw(bz_append_decode_kv(&kv, k_data, v_data, bz_dtype<SrcType>::value, q_inout, num_qo_heads, rot ? 1 : 0,
+                                 o.rope_theta, k_scale, v_scale, o.stream),
              "AppendPagedKVCacheDecode");
 }
 

@@ -57,22 +57,28 @@ class Attention {
         DType* attn_state = v + N * Hkv_ * D_;
         DType* o_proj = input;
 
-        kernel::rms_norm(residual, norm_w_, input, num_tokens, hidden_);
+        // stream and RoPE base travel with the handlers (one set per model); the page writes take theirs
+        // from the table (page_table.options, which an engine points at the same handler's options)
+        void* stream = (qo_indptr_d ? prefill_->options : decode_->options).stream;
+        kernel::rms_norm(residual, norm_w_, input, num_tokens, hidden_, 1e-5f, stream);
         // Three projections into three planes.  (The reference batches them into one or two row-major
         // GEMMs, src/layer/attn.h:137-171, whose output would interleave q, k and v per token while the
         // attention kernels read separate planes; the planes are what the kernel contract needs.)
-        gemm_->gemm((int)N, (int)(Hq_ * D_), (int)hidden_, input, wq_, q);
-        gemm_->gemm((int)N, (int)(Hkv_ * D_), (int)hidden_, input, wk_, k);
-        gemm_->gemm((int)N, (int)(Hkv_ * D_), (int)hidden_, input, wv_, v);
+        using util::GemmOp;
+        gemm_->gemm(GemmOp::N, GemmOp::N, (int)N, (int)(Hq_ * D_), (int)hidden_, input, wq_, q);
+        gemm_->gemm(GemmOp::N, GemmOp::N, (int)N, (int)(Hkv_ * D_), (int)hidden_, input, wk_, k);
+        gemm_->gemm(GemmOp::N, GemmOp::N, (int)N, (int)(Hkv_ * D_), (int)hidden_, input, wv_, v);
         if (qo_indptr_d) {
+            // fused RoPE(q, k) + page store, then attention on the rotated rows
             kernel::store_prefill_kv_cache(page_table, k, v, qo_indptr_d, num_tokens, q, Hq_);
             kernel::batch_prefill_attention(*prefill_, q, qo_indptr_d, k, v, qo_indptr_d, attn_state,
-                                            page_table.batch_size, Hq_, Hkv_, D_);
+                                            page_table.batch_size, Hq_, Hkv_, D_, BZ_ROPE_NONE);
         } else {
+            // fused RoPE(q, new k) + append, then decode on the rotated q
             kernel::append_decode_kv_cache(page_table, k, v, q, Hq_);
             kernel::batch_decode_attention(*decode_, q, page_table, attn_state, Hq_, BZ_ROPE_NONE);
         }
-        gemm_->gemm((int)N, (int)hidden_, (int)(Hq_ * D_), attn_state, wo_, o_proj);
+        gemm_->gemm(GemmOp::N, GemmOp::N, (int)N, (int)hidden_, (int)(Hq_ * D_), attn_state, wo_, o_proj);
         if (tp_ > 1 && all_reduce_) all_reduce_(o_proj, N * hidden_);
     }
 

@@ -40,19 +40,24 @@ class GatedLinearUnit {
         DType* gate_up_state = input;
         DType* down_proj = gate_up_proj;
 
-        kernel::add_rms_norm(input, residual, norm_w_, num_tokens, hidden_);
-        gemm_->gemm((int)N, (int)(2 * inter_), (int)hidden_, input, gate_up_w_, gate_up_proj);
-        kernel::silu_and_mul(gate_up_proj, gate_up_state, num_tokens, inter_);
-        gemm_->gemm((int)N, (int)hidden_, (int)inter_, gate_up_state, down_w_, down_proj);
+        using util::GemmOp;
+        kernel::add_rms_norm(input, residual, norm_w_, num_tokens, hidden_, 1e-5f, stream_);
+        gemm_->gemm(GemmOp::N, GemmOp::N, (int)N, (int)(2 * inter_), (int)hidden_, input, gate_up_w_, gate_up_proj);
+        kernel::silu_and_mul(gate_up_proj, gate_up_state, num_tokens, inter_, stream_);
+        gemm_->gemm(GemmOp::N, GemmOp::N, (int)N, (int)hidden_, (int)inter_, gate_up_state, down_w_, down_proj);
         if (tp_ > 1 && all_reduce_) all_reduce_(down_proj, N * hidden_);
-        kernel::add_residual(down_proj, residual, num_tokens, hidden_);
+        kernel::add_residual(down_proj, residual, num_tokens, hidden_, stream_);
     }
+
+    /// stream of this block's element-wise kernels (default: the process-wide option); the GEMM wrapper has its own
+    void set_stream(void* stream) { stream_ = stream; }
 
   private:
     util::GemmWrapper* gemm_;
     AllReduce all_reduce_;
     const uint32_t hidden_, inter_, tp_;
     DType* workspace_;
+    void* stream_ = kernel::kStreamFromOptions;
     DType *norm_w_, *gate_up_w_, *down_w_;
 };
 

@@ -28,55 +28,14 @@ struct PageWriteArgs {
     RopeFreqs freqs;
 };
 
-// A row of D elements is handled by D/16 lanes; each lane owns 8 elements of the lower half and
-// the 8 elements of the upper half that form rotate-half pairs with them.
+// The rows of one token (q heads to rotate in place, then the k heads, then the v heads) on their way into
+// page `page`, slot `slot`.  A row of D elements is handled by D/16 lanes; each lane owns 8 elements of the
+// lower half and the 8 elements of the upper half that form rotate-half pairs with them.
 template <typename ST, typename PT, int D, bool PREFILL>
-__global__ __launch_bounds__(256) void page_write_kernel(PageWriteArgs a) {
+__device__ __forceinline__ void page_write_rows(const PageWriteArgs& a, int64_t page, int slot, size_t src_tok,
+                                                const float* s_cos, const float* s_sin) {
     constexpr int LANES = D / 16;
     constexpr int ROWS = 256 / LANES;
-    __shared__ float s_cos[D / 2], s_sin[D / 2];
-    __shared__ int s_b;
-
-    int b, pos;
-    size_t src_tok;
-    if (PREFILL) {
-        const int n = blockIdx.x; // global token index
-        if (threadIdx.x == 0) {
-            // largest b with ragged_indptr[b] <= n
-            int lo = 0, hi = (int)a.batch_size;
-            while (hi - lo > 1) {
-                const int mid = (lo + hi) / 2;
-                if (a.ragged_indptr[mid] <= n) lo = mid; else hi = mid;
-            }
-            s_b = lo;
-        }
-        __syncthreads();
-        b = s_b;
-        pos = n - a.ragged_indptr[b];
-        src_tok = (size_t)n;
-        if (n >= a.ragged_indptr[a.batch_size]) return;
-    } else {
-        b = blockIdx.x;
-        const int ahead = a.steps_ahead ? *a.steps_ahead : 0; // fetched together with the table entries
-        const int np = a.indptr[b + 1] - a.indptr[b];
-        if (np <= 0) return;
-        pos = (np - 1) * (int)a.page_size + a.last_page_len[b] - 1 - max(ahead, 0);
-        if (pos < 0) return; // the sequence has no token yet at the present step
-        src_tok = (size_t)b;
-    }
-    const int64_t page = a.indices[a.indptr[b] + pos / (int)a.page_size];
-    const int slot = pos % (int)a.page_size;
-
-    if (a.rope) {
-        for (int i = threadIdx.x; i < D / 2; i += 256) {
-            float s, c;
-            sincosf((float)pos * a.freqs.f[i], &s, &c);
-            s_cos[i] = c;
-            s_sin[i] = s;
-        }
-        __syncthreads();
-    }
-
     const int lane = threadIdx.x % LANES;
     // Pages written at prefill are next read by a later decode step, long after they have left the
     // caches: non-temporal stores leave the cache to the caller's q / k / v rows, which the attention
@@ -164,6 +123,57 @@ __global__ __launch_bounds__(256) void page_write_kernel(PageWriteArgs a) {
         h2.from_float(y);
         pool_store(l2, dst + lane * 8);
         pool_store(h2, dst + D / 2 + lane * 8);
+    }
+}
+
+template <typename ST, typename PT, int D, bool PREFILL>
+__global__ __launch_bounds__(256) void page_write_kernel(PageWriteArgs a) {
+    __shared__ float s_cos[D / 2], s_sin[D / 2];
+
+    // Prefill: one token per workgroup and pass.  The launch has one workgroup per token when the host
+    // knows the token count, otherwise a fixed number of workgroups that stride over the tokens counted
+    // by the ragged index itself (ragged_indptr[batch_size], read on the device).
+    const int total = PREFILL ? (int)min((uint32_t)max(a.ragged_indptr[a.batch_size], 0), a.num_tokens) : (int)a.batch_size;
+    for (int unit = blockIdx.x; unit < total; unit += gridDim.x) {
+        int b, pos;
+        size_t src_tok;
+        if (PREFILL) {
+            const int n = unit; // global token index; largest b with ragged_indptr[b] <= n (wave-uniform search)
+            int lo = 0, hi = (int)a.batch_size;
+            while (hi - lo > 1) {
+                const int mid = (lo + hi) / 2;
+                if (a.ragged_indptr[mid] <= n) lo = mid; else hi = mid;
+            }
+            b = lo;
+            pos = n - a.ragged_indptr[b];
+            src_tok = (size_t)n;
+            // a request longer than the pages its table row lists (the reference asserts seq_len >= append
+            // length, src/kernel/page.cu:43): the tokens without a page are dropped, nothing is written
+            // outside the listed pages
+            if (pos / (int)a.page_size >= a.indptr[b + 1] - a.indptr[b]) continue;
+        } else {
+            b = unit;
+            const int ahead = a.steps_ahead ? *a.steps_ahead : 0; // fetched together with the table entries
+            const int np = a.indptr[b + 1] - a.indptr[b];
+            if (np <= 0) continue;
+            pos = (np - 1) * (int)a.page_size + a.last_page_len[b] - 1 - max(ahead, 0);
+            if (pos < 0) continue; // the sequence has no token yet at the present step
+            src_tok = (size_t)b;
+        }
+        const int64_t page = a.indices[a.indptr[b] + pos / (int)a.page_size];
+        const int slot = pos % (int)a.page_size;
+
+        if (a.rope) {
+            __syncthreads(); // the previous pass has finished with the table
+            for (int i = threadIdx.x; i < D / 2; i += 256) {
+                float s, c;
+                sincosf((float)pos * a.freqs.f[i], &s, &c);
+                s_cos[i] = c;
+                s_sin[i] = s;
+            }
+            __syncthreads();
+        }
+        page_write_rows<ST, PT, D, PREFILL>(a, page, slot, src_tok, s_cos, s_sin);
     }
 }
 
@@ -352,7 +362,11 @@ extern "C" int bz_store_prefill_kv(const bz_paged_kv_t* kv, void* k, const void*
     a.ragged_indptr = ragged_indptr;
     a.num_tokens = num_tokens;
     if (kv->batch_size == 0) return 0;
-    return launch_page_write<true>(a, src_dtype, kv->kv_dtype, (int)kv->head_dim, num_tokens, (hipStream_t)stream);
+    // One workgroup per token when the caller knows the count; otherwise (the reference's four-argument
+    // call, src/kernel/page.h:66-67, whose launch is shaped by page size and batch alone, page.cu:84-89) a
+    // fixed launch whose workgroups stride over the tokens that ragged_indptr[batch_size] counts.
+    const uint32_t grid = num_tokens == BZ_NUM_TOKENS_FROM_INDPTR ? 8192u : num_tokens;
+    return launch_page_write<true>(a, src_dtype, kv->kv_dtype, (int)kv->head_dim, grid, (hipStream_t)stream);
 }
 
 extern "C" int bz_append_decode_kv(const bz_paged_kv_t* kv, const void* k, const void* v, int src_dtype,

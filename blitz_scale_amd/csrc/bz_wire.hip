@@ -75,7 +75,15 @@ __global__ __launch_bounds__(256) void wire_kernel(WireArgs a) {
         const uint32_t c = (uint32_t)(g / a.vecs_per_chunk), e = (uint32_t)(g % a.vecs_per_chunk) * 8;
         const uint32_t i = c / a.layer_cnt, l = c % a.layer_cnt;
         const int32_t page = a.page_ids[i];
-        if ((uint64_t)(uint32_t)page >= a.max_pages) { live[u] = false; continue; } // not a page of this pool: skipped
+        if ((uint64_t)(uint32_t)page >= a.max_pages) { // not a page of this pool: nothing is read from or written to
+            live[u] = false;                           // the pool; a packed stream carries zeros in its place
+            if (PACK) {
+                Vec8<DT> z;
+                z.raw = decltype(z.raw){};
+                wire_store(z, reinterpret_cast<DT*>(a.wire) + g * 8);
+            }
+            continue;
+        }
         pool_off[u] = ((uint64_t)(a.start_layer + l) * a.max_pages + (uint64_t)page) * a.stride_page + e;
         if (sizeof(PT) != sizeof(WT)) {
             const uint32_t half = (uint32_t)(a.stride_page / 2);

@@ -217,7 +217,12 @@ int bz_batch_prefill_ragged(bz_prefill_plan_t* plan, void* q, const int32_t* qo_
  * rope != 0 rotates K at position t on the way in.  With q_inout (optional, [N, Hq, D],
  * num_qo_heads) given as well, q AND the caller's k rows are rotated in place by the same angles:
  * the fused RoPE of the prefill path, after which bz_batch_prefill_ragged runs with BZ_ROPE_NONE.
- * k_scale / v_scale: device fp32 [Hkv]; for an e4m3 pool the value stored is quant(x / scale). */
+ * k_scale / v_scale: device fp32 [Hkv]; for an e4m3 pool the value stored is quant(x / scale).
+ * num_tokens: N, or BZ_NUM_TOKENS_FROM_INDPTR when the host does not know it (the reference's call has no
+ * such argument and shapes its launch from page size and batch, page.cu:84-89).  Tokens of a request beyond
+ * the pages its table row lists are dropped (the reference asserts seq_len >= append length, page.cu:43);
+ * nothing is ever written outside the listed pages. */
+#define BZ_NUM_TOKENS_FROM_INDPTR 0xFFFFFFFFu /* num_tokens: take ragged_indptr[batch_size], read on the device */
 int bz_store_prefill_kv(const bz_paged_kv_t* kv, void* k, const void* v, int src_dtype,
                         const int32_t* ragged_indptr, uint32_t num_tokens, void* q_inout, uint32_t num_qo_heads,
                         int rope, float rope_theta, const float* k_scale, const float* v_scale, void* stream);
@@ -282,8 +287,8 @@ int bz_batch_find_max(uint32_t* output_indices, const void* input, int dtype, ui
  *   wire_dtype: the pool's type (bit copy), or BZ_E4M3 for a 16-bit pool: elements travel as
  *               e4m3(x / scale) and arrive as e4m3 * scale, scale = k_scale / v_scale[l*num_kv_heads +
  *               head] (device arrays [layer_cnt][num_kv_heads]; NULL = 1), half the bytes.
- * Page ids outside [0, max_pages) are skipped (their chunk of `wire` is left untouched by pack, ignored
- * by unpack).  Pages listed twice in an unpack race.  Launch only; no allocation, copy or synchronisation.
+ * Page ids outside [0, max_pages) are skipped (pack writes zeros into their chunk of `wire`, unpack ignores
+ * it).  Pages listed twice in an unpack race.  Launch only; no allocation, copy or synchronisation.
  * ------------------------------------------------------------------------------------- */
 uint64_t bz_kv_wire_bytes(uint32_t num_pages, uint32_t layer_cnt, const bz_paged_kv_t* kv, int wire_dtype);
 int bz_kv_pages_pack(const void* pool_base, uint64_t max_pages, const bz_paged_kv_t* kv, const int32_t* page_ids,

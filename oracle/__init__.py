@@ -318,6 +318,25 @@ def kv_pages_unpack(pool_bits, kv_dtype, max_pages, stride_page, page_ids, start
     return pool_bits
 
 
+def gemm_strided_batched(a_bits, b_bits, dtype, m, n, k, transa=False, transb=False, alpha=1.0, beta=0.0, c_bits=None,
+                         stride_a=None, stride_b=None, stride_c=None, batch=1, parallel=False):
+    """Row-major C[b] = alpha op(A[b]) op(B[b]) + beta C[b] with the argument meaning of
+    util::CublasWrapper::gemmStridedBatched (src/util/cublas_wrapper.h:33-88); returns C's storage bits."""
+    stride_a = m * k if stride_a is None else stride_a
+    stride_b = k * n if stride_b is None else stride_b
+    stride_c = m * n if stride_c is None else stride_c
+    a, b = _c(a_bits, storage_np(dtype)), _c(b_bits, storage_np(dtype))
+    need_c = (batch - 1) * stride_c + m * n
+    c = np.zeros(need_c, storage_np(dtype)) if c_bits is None else _c(c_bits, storage_np(dtype)).reshape(-1).copy()
+    assert c.size >= need_c
+    fn = lib(parallel).bzo_gemm_strided_batched
+    fn.restype = None
+    fn.argtypes = [C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, C.c_float, C.c_void_p, C.c_int64, C.c_void_p, C.c_int64,
+                   C.c_float, C.c_void_p, C.c_int64, C.c_int, C.c_int]
+    fn(int(transa), int(transb), m, n, k, alpha, _p(a), stride_a, _p(b), stride_b, beta, _p(c), stride_c, batch, dtype)
+    return c
+
+
 def prefill_reservation(lens, page_size):
     lens = _c(lens, np.int32)
     B = len(lens)

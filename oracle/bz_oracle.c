@@ -19,6 +19,7 @@
  *   gather_last_token / batch_find_max src/kernel/sampler.h:8-26, sampler.cu:7-25,80-109
  *   host page table build / grow ..... src/blitz/batch.h:236-257,
  *                                      src/blitz/cache_manager.h:161-184,197-324
+ *   row-major (batched) GEMM ......... src/util/cublas_wrapper.h:33-88,144-207
  *
  * The arithmetic behind the attention / norm / activation calls lives in a
  * FlashInfer fork that is absent from the reference checkout
@@ -554,6 +555,43 @@ int bzo_first_fit(uint8_t* free_mask, int max_pages, int n, int32_t* out) {
     if (cnt < n) return cnt; /* caller treats as allocation failure; mask untouched */
     for (int i = 0; i < n; ++i) free_mask[out[i]] = 0;
     return cnt;
+}
+
+/* ------------------------------------------------------------------ */
+/* Row-major strided-batched GEMM with the argument meaning of          */
+/* util::CublasWrapper::gemmStridedBatched (src/util/cublas_wrapper.h:  */
+/* 33-88; operand swap for the column-major library at :183-207):       */
+/*   C[b] (m x n, ld n) = alpha * op(A[b]) * op(B[b]) + beta * C[b]     */
+/*   A[b] stored m x k (ld k) if !transa else k x m (ld m)              */
+/*   B[b] stored k x n (ld n) if !transb else n x k (ld k)              */
+/* fp32 accumulation in index order, alpha and beta applied in fp32,    */
+/* one rounding to the storage type.  (The reference asks cuBLAS for    */
+/* fp16 accumulation on half, :144-146; fp32 is the stricter checker.)  */
+/* ------------------------------------------------------------------ */
+void bzo_gemm_strided_batched(int transa, int transb, int m, int n, int k, float alpha, const void* A,
+                              int64_t stride_a, const void* B, int64_t stride_b, float beta, void* C,
+                              int64_t stride_c, int batch, int dtype) {
+    const size_t es = dtype_size(dtype);
+    for (int b = 0; b < batch; ++b) {
+        const char* Ab = (const char*)A + (size_t)b * (size_t)stride_a * es;
+        const char* Bb = (const char*)B + (size_t)b * (size_t)stride_b * es;
+        char* Cb = (char*)C + (size_t)b * (size_t)stride_c * es;
+#ifdef _OPENMP
+#pragma omp parallel for schedule(static)
+#endif
+        for (int r = 0; r < m; ++r)
+            for (int c = 0; c < n; ++c) {
+                float acc = 0.0f;
+                for (int i = 0; i < k; ++i) {
+                    const float a = load_as_f32(Ab, dtype, transa ? (size_t)i * m + r : (size_t)r * k + i);
+                    const float bb = load_as_f32(Bb, dtype, transb ? (size_t)c * k + i : (size_t)i * n + c);
+                    acc += a * bb;
+                }
+                float v = alpha * acc;
+                if (beta != 0.0f) v += beta * load_as_f32(Cb, dtype, (size_t)r * n + c);
+                store_from_f32(Cb, dtype, (size_t)r * n + c, v);
+            }
+    }
 }
 
 /* number of threads the parallel build uses (1 for the scalar build) */

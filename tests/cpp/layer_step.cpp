@@ -1,8 +1,8 @@
 // One Llama-2-7B-shaped decoder layer (hidden 4096, 32 heads, intermediate 11008) stepping a decode
 // batch of 64 sequences through the C++ drop-in headers with every GEMM on hipBLASLt: the "single-layer decode step" of
 // a Llama-2-7B decode benchmark with the four GEMMs in.  Checks
-//   1. blitz::util::HipblasLtGemm against a naive fp32-accumulate GEMM on a few shapes,
-//   2. the layer's residual stream against the same layer run with the naive GEMM,
+//   1. blitz::util::HipblasLtGemm, in every call form of the reference's GEMM wrapper, against the CPU checker's GEMM,
+//   2. the layer's residual stream against the same layer run with a naive one-thread-per-element GEMM,
 // and prints the time of a layer step.  Runs on the GPU box; built without a GPU.
 #include <algorithm>
 #include <cmath>
@@ -39,11 +39,22 @@ __global__ void naive_gemm(int m, int n, int k, const __half* A, const __half* B
     C[(size_t)row * n + col] = __float2half_rn(acc);
 }
 struct NaiveGemm : blitz::util::GemmWrapper {
-    void gemm(int m, int n, int k, const void* A, const void* B, void* C) override {
+    using GemmWrapper::gemmStridedBatched;
+    void gemmStridedBatched(blitz::util::GemmOp ta, blitz::util::GemmOp tb, int m, int n, int k, float alpha, const void* A,
+                            long long int, const void* B, long long int, float beta, void* C, long long int,
+                            int batch) override {
+        if (ta != blitz::util::GemmOp::N || tb != blitz::util::GemmOp::N || alpha != 1.f || beta != 0.f || batch != 1) {
+            printf("NaiveGemm: only the plain product the layers call\n");
+            exit(5);
+        }
         hipLaunchKernelGGL(naive_gemm, dim3((n + 127) / 128, m), dim3(128), 0, 0, m, n, k, (const __half*)A,
                            (const __half*)B, (__half*)C);
     }
 };
+// the CPU checker's GEMM (oracle/bz_oracle.c): fp32 accumulation in index order, one rounding
+extern "C" void bzo_gemm_strided_batched(int transa, int transb, int m, int n, int k, float alpha, const void* A,
+                                         int64_t stride_a, const void* B, int64_t stride_b, float beta, void* C,
+                                         int64_t stride_c, int batch, int dtype);
 // device fill: uniform(-scale, scale) + mean from a counter hash (no host buffers of gigabytes)
 __global__ void fill_uniform(__half* p, size_t n, float scale, float mean, uint64_t seed) {
     for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x) {
@@ -77,27 +88,56 @@ int main() {
     blitz::util::HipblasLtGemm lt(HIP_R_16F);
     NaiveGemm naive;
 
-    // ---- 1. the GEMM wrapper against the naive product (inputs O(1)/sqrt(k): results O(1))
-    const int shapes[][3] = {{64, 512, 256}, {7, 1024, 384}, {1, 4096, 4096}, {64, 12288, 4096}, {57, 264, 128}};
-    for (auto& s : shapes) {
-        const int m = s[0], n = s[1], k = s[2];
-        __half *A, *B, *C0, *C1;
-        HIP_OK(hipMalloc(&A, (size_t)m * k * 2));
-        HIP_OK(hipMalloc(&B, (size_t)k * n * 2));
-        HIP_OK(hipMalloc(&C0, (size_t)m * n * 2));
-        HIP_OK(hipMalloc(&C1, (size_t)m * n * 2));
-        fill(A, (size_t)m * k, 1.0f, 0.f, 11);
-        fill(B, (size_t)k * n, 1.7f / sqrtf((float)k), 0.f, 12);
-        naive.gemm(m, n, k, A, B, C0);
-        lt.gemm(m, n, k, A, B, C1);
+    // ---- 1. the GEMM wrapper against the CPU checker's GEMM: every call form of the reference's wrapper
+    // (src/util/cublas_wrapper.h:71-131) -- transposes, alpha/beta, strided batches -- on shapes the layers use
+    // (inputs O(1)/sqrt(k): results O(1))
+    using blitz::util::GemmOp;
+    struct Case { int m, n, k, ta, tb, batch; float alpha, beta; int pad; };
+    const Case cases[] = {
+        {64, 512, 256, 0, 0, 1, 1.f, 0.f, 0},    {7, 1024, 384, 0, 0, 1, 1.f, 0.f, 0},
+        {1, 4096, 4096, 0, 0, 1, 1.f, 0.f, 0},   {64, 4096, 4096, 0, 0, 1, 1.f, 0.f, 0},   // a 7B projection at batch 64
+        {57, 264, 128, 0, 0, 1, 1.f, 0.f, 0},    {33, 136, 72, 1, 0, 1, 1.f, 0.f, 0},
+        {33, 136, 72, 0, 1, 1, 1.f, 0.f, 0},     {33, 136, 72, 1, 1, 1, 0.5f, 0.f, 0},
+        {16, 128, 64, 0, 0, 5, 1.f, 0.f, 0},     {16, 128, 64, 0, 1, 3, 2.f, -1.f, 24},    // batched, strides padded by 24 elements
+        {40, 96, 200, 1, 0, 4, 1.f, 0.25f, 8},
+    };
+    for (const Case& c : cases) {
+        const int m = c.m, n = c.n, k = c.k;
+        const long long sa = (long long)m * k + c.pad, sb = (long long)k * n + c.pad, sc = (long long)m * n + c.pad;
+        const size_t na = (size_t)sa * c.batch, nb = (size_t)sb * c.batch, nc = (size_t)sc * c.batch;
+        __half *A, *B, *C1;
+        HIP_OK(hipMalloc(&A, na * 2));
+        HIP_OK(hipMalloc(&B, nb * 2));
+        HIP_OK(hipMalloc(&C1, nc * 2));
+        fill(A, na, 1.0f, 0.f, 11);
+        fill(B, nb, 1.7f / sqrtf((float)k), 0.f, 12);
+        fill(C1, nc, 1.0f, 0.f, 13); // previous contents of C: read when beta != 0, and the padding must survive
+        std::vector<__half> hA(na), hB(nb), hC(nc), got(nc);
+        HIP_OK(hipMemcpy(hA.data(), A, na * 2, hipMemcpyDeviceToHost));
+        HIP_OK(hipMemcpy(hB.data(), B, nb * 2, hipMemcpyDeviceToHost));
+        HIP_OK(hipMemcpy(hC.data(), C1, nc * 2, hipMemcpyDeviceToHost));
+        const GemmOp ta = c.ta ? GemmOp::T : GemmOp::N, tb = c.tb ? GemmOp::T : GemmOp::N;
+        if (c.batch == 1 && c.alpha == 1.f && c.beta == 0.f) lt.gemm(ta, tb, m, n, k, A, B, C1);
+        else if (c.pad == 0 && c.alpha == 1.f && c.beta == 0.f) lt.gemmBatched(ta, tb, m, n, k, A, B, C1, c.batch);
+        else lt.gemmStridedBatched(ta, tb, m, n, k, c.alpha, A, sa, B, sb, c.beta, C1, sc, c.batch);
         HIP_OK(hipDeviceSynchronize());
-        double ref = 0;
-        const double e = max_abs_diff_dev(C1, C0, (size_t)m * n, &ref);
+        HIP_OK(hipMemcpy(got.data(), C1, nc * 2, hipMemcpyDeviceToHost));
+        bzo_gemm_strided_batched(c.ta, c.tb, m, n, k, c.alpha, hA.data(), sa, hB.data(), sb, c.beta, hC.data(), sc, c.batch, 0);
+        double e = 0, ref = 0;
+        bool pad_ok = true;
+        for (size_t i = 0; i < nc; ++i) {
+            const double x = __half2float(got[i]), y = __half2float(hC[i]);
+            if ((long long)(i % (size_t)sc) >= (long long)m * n) { pad_ok = pad_ok && x == y; continue; }
+            e = fmax(e, fabs(x - y));
+            ref = fmax(ref, fabs(y));
+            if (!(x == x)) e = INFINITY;
+        }
         // both accumulate in fp32 and round once; the summation order differs: a few f16 steps at |c| ~ 2
-        const bool good = e <= 4e-3 * fmax(1.0, ref);
-        printf("gemm %5d x %5d x %5d: max |hipblaslt - naive| = %.3e (max |c| %.2f) %s\n", m, n, k, e, ref, good ? "ok" : "BAD");
+        const bool good = e <= 4e-3 * fmax(1.0, ref) && pad_ok;
+        printf("gemm %c%c %5d x %5d x %5d, batch %d, alpha %.2f beta %.2f: max |hipblaslt - cpu checker| = %.3e (max |c| %.2f) %s\n",
+               c.ta ? 'T' : 'N', c.tb ? 'T' : 'N', m, n, k, c.batch, c.alpha, c.beta, e, ref, good ? "ok" : "BAD");
         ok = ok && good;
-        (void)hipFree(A); (void)hipFree(B); (void)hipFree(C0); (void)hipFree(C1);
+        (void)hipFree(A); (void)hipFree(B); (void)hipFree(C1);
     }
 
     // ---- 2. a Llama-2-7B-shaped layer, decode batch of 64, contexts U[512, 2048]

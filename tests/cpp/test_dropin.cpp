@@ -73,7 +73,14 @@ __global__ void naive_gemm(int m, int n, int k, const uint16_t* A, const uint16_
     Cm[(size_t)row * n + col] = __half_as_ushort(__float2half_rn(acc));
 }
 struct NaiveGemm : blitz::util::GemmWrapper {
-    void gemm(int m, int n, int k, const void* A, const void* B, void* C) override {
+    using GemmWrapper::gemmStridedBatched;
+    void gemmStridedBatched(blitz::util::GemmOp ta, blitz::util::GemmOp tb, int m, int n, int k, float alpha, const void* A,
+                            long long int, const void* B, long long int, float beta, void* C, long long int,
+                            int batch) override {
+        if (ta != blitz::util::GemmOp::N || tb != blitz::util::GemmOp::N || alpha != 1.f || beta != 0.f || batch != 1) {
+            printf("NaiveGemm: only the plain product the layers call\n");
+            exit(5);
+        }
         hipLaunchKernelGGL(naive_gemm, dim3((n + 127) / 128, m), dim3(128), 0, 0, m, n, k, (const uint16_t*)A,
                            (const uint16_t*)B, (uint16_t*)C);
     }

@@ -123,3 +123,54 @@ def test_append_quantises_to_e4m3():
     K.append_decode_kv_cache(dev.pt, to_dev(k, BZ_BF16), to_dev(v, BZ_BF16), k_scale=dev.k_scale, v_scale=dev.v_scale)
     torch.cuda.synchronize()
     assert np.array_equal(to_host_bits(dev.pool), want)  # x / scale and RNE-saturating e4m3: bit exact
+
+
+@pytest.mark.parametrize("rope", [False, True])
+def test_store_prefill_token_count_from_the_ragged_index(rope):
+    """The reference's four-argument call does not pass a token count (src/kernel/page.h:66-67): the kernel
+    reads ragged_indptr[batch] on the device and a fixed launch strides over the tokens.  Same pool bits as
+    the launch with the count given, and as the checker; long enough that workgroups take several tokens."""
+    from blitz_scale_amd._lib import BZ_NUM_TOKENS_FROM_INDPTR
+    rng = np.random.default_rng(60)
+    lens, Hkv, D, P, dtype = [1, 4000, 16, 5000, 333, 3000], 4, 128, 16, BZ_F16
+    p, fill = _setup(61, lens, 8, Hkv, D, P, dtype, BZ_LAYOUT_HND)
+    ri = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+    assert ri[-1] > 8192
+    k, v = wl.randn_bits(rng, (ri[-1], Hkv, D), dtype), wl.randn_bits(rng, (ri[-1], Hkv, D), dtype)
+    want = p.pool.copy()
+    oracle.store_prefill_kv(p.oracle_kv(want), k, v, dtype, ri, rope=rope, rope_theta=1e4)
+    ri_d = to_dev(ri.view(np.float32), 3).view(torch.int32)
+    pools = []
+    for n in (int(ri[-1]), BZ_NUM_TOKENS_FROM_INDPTR):
+        dev = DeviceDecode(p)
+        kd = to_dev(k, dtype)
+        K.store_prefill_kv_cache(dev.pt, kd, to_dev(v, dtype), ri_d, num_tokens=n, rope=rope, rope_theta=1e4)
+        torch.cuda.synchronize()
+        pools.append(to_host_bits(dev.pool))
+        assert np.array_equal(to_host_bits(kd), k)  # without q the caller's k rows are left alone
+    assert np.array_equal(pools[0], pools[1])
+    if rope:  # rotated rows: the device's sincosf may differ from the host's in the last place
+        assert np.abs(wl.to_f32(pools[1], dtype) - wl.to_f32(want, dtype)).max() <= 2.0 ** -8
+        assert (pools[1] != want).mean() < 2e-3
+    else:
+        assert np.array_equal(pools[1], want)
+
+
+def test_store_prefill_drops_tokens_beyond_the_listed_pages():
+    """A ragged length longer than the pages of its table row (the reference asserts against it,
+    src/kernel/page.cu:43): the tokens without a page are dropped and no other page is touched."""
+    rng = np.random.default_rng(62)
+    Hkv, D, P, dtype = 2, 128, 16, BZ_F16
+    p, fill = _setup(63, [20, 40], 4, Hkv, D, P, dtype, BZ_LAYOUT_HND, reserve_extra=0)  # 2 and 3 pages
+    lens_claimed = [20, 100]                                                              # request 1 claims 7 pages' worth
+    ri = np.concatenate([[0], np.cumsum(lens_claimed)]).astype(np.int32)
+    k, v = wl.randn_bits(rng, (ri[-1], Hkv, D), dtype), wl.randn_bits(rng, (ri[-1], Hkv, D), dtype)
+    want = p.pool.copy()
+    ri_fit = np.array([0, 20, 20 + 48], np.int32)  # what fits: 3 pages x 16 slots of request 1
+    k_fit = np.concatenate([k[:20], k[20:68]])
+    v_fit = np.concatenate([v[:20], v[20:68]])
+    oracle.store_prefill_kv(p.oracle_kv(want), k_fit, v_fit, dtype, ri_fit)
+    dev = DeviceDecode(p)
+    K.store_prefill_kv_cache(dev.pt, to_dev(k, dtype), to_dev(v, dtype), to_dev(ri.view(np.float32), 3).view(torch.int32))
+    torch.cuda.synchronize()
+    assert np.array_equal(to_host_bits(dev.pool), want)

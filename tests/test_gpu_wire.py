@@ -144,7 +144,7 @@ def test_empty_and_rejected_arguments():
     K.pack_kv_pages(pt, 4, torch.zeros(1, dtype=torch.int32, device="cuda"), 0, 0, wire)  # no layers
     torch.cuda.synchronize()
     assert (wire.cpu().numpy() == 0xA5).all()
-    # a page id that is not in the pool is skipped, not dereferenced
+    # a page id that is not in the pool is not dereferenced; its chunk of the stream carries zeros
     bad = torch.tensor([1, 4, -1, 1 << 30, 2], dtype=torch.int32, device="cuda")
     sp = 2 * 2 * 4 * 16
     big = wire_tensor(5 * 2 * sp * 2)
@@ -154,7 +154,7 @@ def test_empty_and_rejected_arguments():
     pool3 = bits.reshape(2, 4, sp)
     for i, pg in enumerate([1, None, None, None, 2]):
         if pg is None:
-            assert (got[i] == 0xA5A5).all()
+            assert not got[i].any()
         else:
             assert np.array_equal(got[i], np.concatenate([pool3[0, pg], pool3[1, pg]]))
     with pytest.raises(BzError):  # a 16-bit wire for the other 16-bit type is not a format of this library

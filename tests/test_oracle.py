@@ -375,3 +375,51 @@ def test_prefill_reservation_matches_reference_rule():
     assert all(1 <= x <= P for x in lpl)
     # the table describes len+1 slots through the kernel's seq_len formula (page.cu:38-40)
     assert list((np.diff(indptr) - 1) * P + lpl) == [l + 1 for l in lens]
+
+
+# ---- row-major (batched) GEMM of the layers' GEMM boundary ------------------------------------------
+@pytest.mark.parametrize("transa", [False, True])
+@pytest.mark.parametrize("transb", [False, True])
+def test_gemm_against_numpy_matmul(transa, transb):
+    """Pinned by numpy.matmul on the logical operands: small integers make every product and sum exact, so
+    any index, transpose or stride mistake changes bits; m, n, k and the batch strides are all different."""
+    rng = np.random.default_rng(5)
+    m, n, k, batch = 5, 7, 11, 3
+    sa, sb, sc = m * k + 3, k * n + 5, m * n + 2          # padded strides between the matrices of a batch
+    A = rng.integers(-4, 5, size=(batch, m, k)).astype(np.float32)
+    B = rng.integers(-4, 5, size=(batch, k, n)).astype(np.float32)
+    C0 = rng.integers(-8, 9, size=(batch, m, n)).astype(np.float32)
+    a_store = np.zeros(batch * sa, np.float32)
+    b_store = np.zeros(batch * sb, np.float32)
+    c_store = np.full(batch * sc, 77.0, np.float32)       # the gaps between matrices must stay untouched
+    for b in range(batch):
+        a_store[b * sa:b * sa + m * k] = (A[b].T if transa else A[b]).reshape(-1)
+        b_store[b * sb:b * sb + k * n] = (B[b].T if transb else B[b]).reshape(-1)
+        c_store[b * sc:b * sc + m * n] = C0[b].reshape(-1)
+    for dt in (oracle.F16, oracle.BF16):
+        got = oracle.gemm_strided_batched(oracle.from_f32(a_store, dt), oracle.from_f32(b_store, dt), dt, m, n, k,
+                                          transa=transa, transb=transb, alpha=2.0, beta=-1.0,
+                                          c_bits=oracle.from_f32(c_store, dt), stride_a=sa, stride_b=sb, stride_c=sc,
+                                          batch=batch)
+        got = oracle.to_f32(got, dt)
+        for b in range(batch):
+            want = 2.0 * np.matmul(A[b].astype(np.float64), B[b].astype(np.float64)) - C0[b]
+            assert np.array_equal(got[b * sc:b * sc + m * n].reshape(m, n), want.astype(np.float32))
+            assert np.all(got[b * sc + m * n:(b + 1) * sc] == 77.0)
+
+
+def test_gemm_rounding_and_defaults():
+    """alpha = 1, beta = 0, contiguous batch (what gemm / gemmBatched of the reference reduce to): one
+    rounding of an fp32 sum; C's previous contents (NaN here) are not read when beta is 0."""
+    rng = np.random.default_rng(6)
+    m, n, k = 9, 33, 257
+    A = wl.randn_bits(rng, (2, m, k), BZ_F16)
+    B = wl.randn_bits(rng, (2, k, n), BZ_F16, std=1.0 / np.sqrt(k))
+    c0 = np.full(2 * m * n, 0x7E00, np.uint16)
+    got = oracle.to_f32(oracle.gemm_strided_batched(A, B, oracle.F16, m, n, k, c_bits=c0, batch=2), oracle.F16)
+    want = np.matmul(wl.to_f32(A, BZ_F16).astype(np.float64), wl.to_f32(B, BZ_F16).astype(np.float64))
+    want16 = want.astype(np.float16).astype(np.float64)
+    # fp32 accumulation error (~1e-6) can only move a result across a rounding boundary: at most one f16 step
+    step = 2.0 ** (np.floor(np.log2(np.maximum(np.abs(want), 2.0 ** -14))) - 10)
+    assert (np.abs(got.reshape(2, m, n) - want16) <= step).all()
+    assert (got.reshape(2, m, n) == want16).mean() > 0.99
