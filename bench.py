@@ -2,10 +2,12 @@
 
 Default workload (the headline, BASELINE config 3): Llama-3-8B-shaped GQA paged decode, bf16, batch
 128, 32/8 heads, head_dim 128, page_size 16, log-normal contexts.  A step is one layer's decode-time
-attention block over the whole batch: the fused RoPE + KV append of the new token followed by batch
-decode over the paged KV cache (src/layer/attn.h:196-203 of the reference).  Steps cycle over several
-layer planes of the pool, as a model's layer loop does, so the KV a step reads has not just been read
-by the previous step.  plan() runs once per model step in the reference (src/model/llama.h:363-375),
+attention block over the whole batch: the KV append of the new token (K rotated) and the batch decode
+over the paged KV cache (src/layer/attn.h:196-203 of the reference), issued as the library's one-call
+decode step (bz_decode_step: two launches).  Steps cycle over several layer planes of the pool, as a
+model's layer loop does, so the KV a step reads has not just been read by the previous step; the value
+reported is the step replayed from one HIP graph of that layer loop (the eagerly launched step is
+reported beside it).  plan() runs once per model step in the reference (src/model/llama.h:363-375),
 outside the layer loop, and is timed separately.
 
 --workload C2 | C4 | C5 run the other configurations (C2 adds the RMSNorm and SiLU-gate kernels of the
@@ -40,6 +42,11 @@ def parse():
                     help="tokens per KV page for the decode workloads (default: the configuration's 16; the "
                          "reference's production value is 64, src/server/disaggregate.cc:310)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--two-call", action="store_true",
+                    help="decode workloads: issue the step as append_decode_kv_cache + batch_decode_attention "
+                         "(three launches) instead of the one-call decode step")
+    ap.add_argument("--no-graph", action="store_true", help="decode workloads: skip the HIP-graph replay pass")
+    ap.add_argument("--no-rope", action="store_true", help="decode workloads: leave RoPE out of the step (diagnostic)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also launch a few plain device copies of 1 GiB (reference point for rocprofv3 --pmc byte counters)")
     args = ap.parse_args()
@@ -114,7 +121,7 @@ def bench_decode(args, name):
     import torch
 
     from blitz_scale_amd import kernel as K, workloads as wl
-    from blitz_scale_amd._lib import BZ_BF16, BZ_E4M3, BZ_F16, BZ_LAYOUT_HND, BZ_ROPE_NONE
+    from blitz_scale_amd._lib import BZ_BF16, BZ_E4M3, BZ_F16, BZ_LAYOUT_HND, BZ_ROPE_NONE, BZ_ROPE_Q_ONLY
 
     dev = "cuda"
     cfg = dict(wl.CONFIGS[name])
@@ -191,22 +198,35 @@ def bench_decode(args, name):
 
     kev = HipEvents(steps)  # recorded by the library around the decode kernel launch itself
 
-    def step(i, ev):
+    rope = theta is not None and not args.no_rope
+
+    def attention(stream=None):
+        """One layer's append + decode.  One call (two launches: decode kernel over the cached tokens, then the
+        kernel that appends the new token, adds its term and folds the split-K partials), or with --two-call
+        the reference's two calls (three launches); either way q, k and v stay as the projection left them."""
+        if args.two_call:
+            K.append_decode_kv_cache(pt, k_new, v_new, rope=rope, rope_theta=theta or 1e4, k_scale=k_scale,
+                                     v_scale=v_scale, stream=stream)
+            K.batch_decode_attention(handler, q, pt, out, Hq, rope_mode=BZ_ROPE_Q_ONLY if rope else BZ_ROPE_NONE,
+                                     rope_theta=theta or 1e4, k_scale=k_scale, v_scale=v_scale, stream=stream)
+        else:
+            K.decode_step(handler, q, k_new, v_new, pt, out, Hq, rope=rope, rope_theta=theta or 1e4, k_scale=k_scale,
+                          v_scale=v_scale, stream=stream)
+
+    def step(i, ev, stream=None):
         pt.set_layer(i % L, pool_pages)
-        K.append_decode_kv_cache(pt, k_new, v_new, q=q, num_qo_heads=Hq, rope=theta is not None,
-                                 rope_theta=theta or 1e4, k_scale=k_scale, v_scale=v_scale)
-        if ev == "call":      # informational pass: torch events around the whole decode call
+        if ev == "call":      # informational pass: torch events around the attention call(s)
             call_ev[i][0].record()
         elif ev is not None:  # timed pass: the library records a HIP event pair around the decode kernel launch
             handler.set_timing_events(*kev.pair(i))
-        K.batch_decode_attention(handler, q, pt, out, Hq, rope_mode=BZ_ROPE_NONE, k_scale=k_scale, v_scale=v_scale)
+        attention(stream)
         if ev == "call":
             call_ev[i][1].record()
         if name == "C2":
-            K.add_rms_norm(x, res, w, B, h)
-            K.silu_and_mul(gate_up, act, B, I)
+            K.add_rms_norm(x, res, w, B, h, stream=stream)
+            K.silu_and_mul(gate_up, act, B, I, stream=stream)
 
-    ms_per_step, _ = timed(step, steps, warmup, torch_events=False)
+    eager_ms, _ = timed(step, steps, warmup, torch_events=False)
     handler.set_timing_events(None, None)
     kern_ms = np.array([kev.elapsed_ms(i) for i in range(steps)])
     ncall = min(steps, 100)
@@ -215,9 +235,39 @@ def bench_decode(args, name):
         step(i, "call")
     torch.cuda.synchronize()
     dec_ms = np.array([a.elapsed_time(b) for a, b in call_ev])
+
+    # ---- the same steps as a layer loop would issue them in production: L consecutive layers' steps recorded
+    # into one HIP graph and replayed (no host work between the launches); outputs compared with the eager step
+    ms_per_step, graph_note = eager_ms, "eager launches (no graph pass)"
+    if not args.no_graph:
+        step(L - 1, None)
+        torch.cuda.synchronize()
+        want = out.clone()
+        side = torch.cuda.Stream()
+        with torch.cuda.stream(side):
+            step(0, None, side.cuda_stream)  # warm-up on the capture stream, outside the capture
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=side):
+            for l in range(L):
+                step(l, None, torch.cuda.current_stream().cuda_stream)
+        torch.cuda.synchronize()
+        out.zero_()
+        graph.replay()
+        torch.cuda.synchronize()
+        same = bool(torch.equal(out.view(torch.int16), want.view(torch.int16)))
+        reps = max(1, steps // L)
+        wreps = max(1, warmup // L)
+        g_ms, _ = timed(lambda i, e: graph.replay(), reps, wreps, torch_events=False)
+        ms_per_step = g_ms / L
+        steps, warmup = reps * L, wreps * L
+        graph_note = (f"one HIP graph of {L} consecutive layers' steps, replayed {reps} times; last layer's output "
+                      f"bit-identical to the eager step: {same}")
     alg_bytes = wl.decode_algorithmic_bytes(ctx, Hq, Hkv, D, kv_bytes, 2, P)
     achieved = alg_bytes / (float(kern_ms.mean()) * 1e-3) / 1e9
     traffic = measured_traffic(name, args)
+    frac_call = alg_bytes / (float(dec_ms.mean()) * 1e-3) / 1e9 / HBM_PEAK_GBPS
+    frac_step = alg_bytes / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBPS
     res_json = {
         "metric": "paged_decode_us_per_step", "value": round(ms_per_step * 1e3, 3), "unit": "us/step",
         "n_gpus": 1, "steps": steps, "warmup": warmup, "ms_per_step": round(ms_per_step, 6),
@@ -226,7 +276,7 @@ def bench_decode(args, name):
         "config": dict({
             "workload": {"C2": "C2: Llama-2-7B-shaped MHA decode step of one layer (fused RoPE+append, batch decode, "
                                "add+RMSNorm, SiLU-gate)",
-                         "C3": "C3: Llama-3-8B-shaped GQA paged decode, one layer per step (fused RoPE+append, batch decode)",
+                         "C3": "C3: Llama-3-8B-shaped GQA paged decode, one layer per step (KV append with RoPE + batch decode)",
                          "C5": "C5: Llama-3-70B-shaped GQA decode with e4m3 KV, one layer per step (quantising append, "
                                "batch decode)"}[name],
             "batch": B, "num_qo_heads": Hq, "num_kv_heads": Hkv, "head_dim": D, "page_size": P, "ctx": ctx_desc,
@@ -235,13 +285,24 @@ def bench_decode(args, name):
             "seed": hex(args.seed), "plan": info}, **extra),
         "tokens_per_s": round(B / (ms_per_step * 1e-3), 1),
         "plan_ms_per_model_step": round(plan_ms, 4),
+        "step_launch": graph_note,
+        "step_calls": "append_decode_kv_cache + batch_decode_attention (3 launches)" if args.two_call
+                      else "bz_decode_step (2 launches: decode kernel, then append + new-token term + split-K fold)",
+        "eager_us_per_step": round(eager_ms * 1e3, 3),
         "decode_call_us": pct(dec_ms),
         "decode_kernel_us": pct(kern_ms),
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                     "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": traffic,
+                     "frac": round(achieved / HBM_PEAK_GBPS, 4),
+                     "frac_call": round(frac_call, 4), "frac_step": round(frac_step, 4),
+                     "traffic": traffic,
+                     "traffic_source": "offline: rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this workload "
+                                       "(profiles/), not measured in this run",
                      "algorithmic_bytes_per_launch": int(alg_bytes),
-                     "kernel": "decode kernel (bz::decode_mfma_kernel), HIP events recorded by the library on the launch "
-                               "stream right around its launch; decode_call_us also holds the split-K combine launch"},
+                     "kernel": "decode kernel (bz::decode_mfma_kernel): `achieved` and `frac` are the algorithmic bytes "
+                               "of the step over that kernel's own duration (HIP events recorded by the library on the "
+                               "launch stream right around its launch); frac_call is the same bytes over the whole "
+                               "attention call(s) of the step (decode_call_us: every launch needed for the result), "
+                               "frac_step over ms_per_step"},
     }
     if not args.no_cpu_baseline:
         import oracle  # the checker, used here only as the timed CPU baseline
@@ -346,6 +407,8 @@ def bench_prefill(args):
         "attention_kernel_us": pct(att_ms),
         "roofline": {"bound": "mfma", "achieved": round(achieved, 1), "peak": MFMA_PEAK_TFLOPS, "unit": "TFLOP/s",
                      "frac": round(achieved / MFMA_PEAK_TFLOPS, 4), "traffic": measured_traffic("C4", args),
+                     "traffic_source": "offline: rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this workload "
+                                       "(profiles/), not measured in this run",
                      "algorithmic_flops_per_launch": flops,
                      "kernel": "ragged causal prefill attention, HIP events on the launch stream"},
     }

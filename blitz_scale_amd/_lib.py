@@ -57,6 +57,7 @@ SIGNATURES = {
     "bz_decode_plan_info": (_i32, [_vp, C.POINTER(_u32), C.POINTER(_u32), C.POINTER(_u32)]),
     "bz_decode_plan_set_timing_events": (_i32, [_vp, _vp, _vp]),
     "bz_batch_decode": (_i32, [_vp, _vp, _i32, _kvp, _vp, _i32, _u32, _i32, _f32, _f32, _vp, _vp, _vp, _vp]),
+    "bz_decode_step": (_i32, [_vp, _vp, _i32, _vp, _vp, _kvp, _vp, _i32, _u32, _i32, _f32, _f32, _vp, _vp, _vp, _vp]),
     "bz_batch_decode_noalloc_scratch_bytes": (_sz, []),
     "bz_batch_decode_noalloc": (_i32, [_vp, _vp, _i32, _kvp, _vp, _i32, _u32, _i32, _f32, _f32, _vp, _vp, _vp, _vp]),
     "bz_prefill_plan_create": (_vp, []),

@@ -41,4 +41,20 @@ void batch_decode_attention(BlitzBatchDecodeHandler<DType, IdType>& handler, DTy
              "batchDecodeAttention");
 }
 
+/// append_decode_kv_cache followed by batch_decode_attention (src/layer/attn.h:196-203) as ONE call, two
+/// launches instead of three (no counterpart in the reference): the new K row (rotated when
+/// handler.options.append_rotates_k) and V row go into the cache, q is rotated inside the kernels, and q, k, v
+/// stay as the projection left them.  Same cache bits as the two calls, same result to rounding.
+template<typename DType, typename IdType, typename KVType = DType>
+void decode_attention_step(BlitzBatchDecodeHandler<DType, IdType>& handler, DType* q_input, DType* k_new, DType* v_new,
+                           PageTable<KVType, IdType>& paged_kv, DType* output, const uint32_t num_qo_heads,
+                           const float* k_scale = nullptr, const float* v_scale = nullptr) {
+    const AttentionOptions& o = handler.options;
+    const bz_paged_kv_t kv = paged_kv.c_view();
+    bz_throw(bz_decode_step(static_cast<bz_decode_plan_t*>(handler.get()), q_input, bz_dtype<DType>::value, k_new, v_new,
+                            &kv, output, bz_dtype<DType>::value, num_qo_heads, o.append_rotates_k ? 1 : 0, o.rope_theta,
+                            o.sm_scale, k_scale, v_scale, nullptr, o.stream),
+             "batchDecodeAttention");
+}
+
 } // namespace blitz::kernel

@@ -1,7 +1,8 @@
 // Attention block of one transformer layer: the call-site contract of src/layer/attn.h of the
 // BlitzScale worker (same constructor roles, same forward() signature and workspace planes), with the
 // attention-side work routed to the gfx950 kernels:
-//   decode : fused RoPE(q, new k) + KV append, then paged batch decode
+//   decode : the one-call decode step (paged batch decode over the cached tokens, then a kernel that rotates
+//            and appends the new K/V rows, adds the new token's term and folds the split-K partials)
 //   prefill: fused RoPE(q, k) + KV page store, then ragged causal attention on the rotated rows
 // K is cached rotated, so no kernel ever rotates cached K again.
 #pragma once
@@ -74,9 +75,8 @@ class Attention {
             kernel::batch_prefill_attention(*prefill_, q, qo_indptr_d, k, v, qo_indptr_d, attn_state,
                                             page_table.batch_size, Hq_, Hkv_, D_, BZ_ROPE_NONE);
         } else {
-            // fused RoPE(q, new k) + append, then decode on the rotated q
-            kernel::append_decode_kv_cache(page_table, k, v, q, Hq_);
-            kernel::batch_decode_attention(*decode_, q, page_table, attn_state, Hq_, BZ_ROPE_NONE);
+            // append (new K rotated on its way in) + decode (q rotated inside the kernels) as one call
+            kernel::decode_attention_step(*decode_, q, k, v, page_table, attn_state, Hq_);
         }
         gemm_->gemm(GemmOp::N, GemmOp::N, (int)N, (int)hidden_, (int)(Hq_ * D_), attn_state, wo_, o_proj);
         if (tp_ > 1 && all_reduce_) all_reduce_(o_proj, N * hidden_);

@@ -300,7 +300,12 @@ static void launch_zero(const DecodePlan* p, void* out, uint32_t row_elems, hipS
 int decode_fast_path(const DecodePlan* p, const void* q, void* out, float* lse, int q_dtype, int out_dtype,
                      int rope_mode, float sm_scale_log2, const RopeFreqs& freqs, const bz_paged_kv_t* kv,
                      uint32_t num_qo_heads, const float* k_scale, const float* v_scale, float* part_o,
-                     float* part_lse, hipStream_t s); // bz_decode_mfma.hip
+                     float* part_lse, bool step_mode, hipStream_t s); // bz_decode_mfma.hip
+
+int decode_step_fast_path(const DecodePlan* p, const void* q, const void* k_new, const void* v_new, void* out,
+                          float* lse, int q_dtype, int out_dtype, int rope, float sm_scale_log2,
+                          const RopeFreqs& freqs, const bz_paged_kv_t* kv, uint32_t num_qo_heads, const float* k_scale,
+                          const float* v_scale, hipStream_t s); // bz_decode_mfma.hip
 
 // Where the split-K partial results of one call live: the plan's float workspace (bz_batch_decode) or the
 // library's own device array (bz_batch_decode_noalloc).  The two kernels never run in the same call, so
@@ -354,7 +359,7 @@ static int batch_decode_impl(DecodePlan* p, const void* q, int q_dtype, const bz
         int rc = BZ_ERR_UNSUPPORTED;
         if (!p->force_general)
             rc = decode_fast_path(p, q, out, lse, q_dtype, out_dtype, rope_mode, a.sm_scale_log2, a.freqs, kv,
-                                  num_qo_heads, k_scale, v_scale, bufs.mfma_part_o, bufs.mfma_part_lse, s);
+                                  num_qo_heads, k_scale, v_scale, bufs.mfma_part_o, bufs.mfma_part_lse, false, s);
         if (rc == 0) {
             // the MFMA path brings its own combine; only empty sequences are left to do
             if (p->num_empty > 0) {
@@ -444,6 +449,46 @@ extern "C" int bz_batch_decode(bz_decode_plan_t* plan_, const void* q, int q_dty
                                void* stream) {
     return batch_decode_impl(reinterpret_cast<DecodePlan*>(plan_), q, q_dtype, kv, out, out_dtype, num_qo_heads,
                              rope_mode, rope_theta, sm_scale, k_scale, v_scale, lse, nullptr, stream);
+}
+
+extern "C" int bz_decode_step(bz_decode_plan_t* plan_, const void* q, int q_dtype, const void* k_new, const void* v_new,
+                              const bz_paged_kv_t* kv, void* out, int out_dtype, uint32_t num_qo_heads, int rope,
+                              float rope_theta, float sm_scale, const float* k_scale, const float* v_scale, float* lse,
+                              void* stream) {
+    DecodePlan* p = reinterpret_cast<DecodePlan*>(plan_);
+    if (!p || !kv || !q || !k_new || !v_new || !out) return BZ_ERR_BAD_ARG;
+    if (!p->planned) return BZ_ERR_NOT_PLANNED;
+    if (!kv->k_data || !kv->v_data || !kv->indices || !kv->indptr || !kv->last_page_len) return BZ_ERR_BAD_ARG;
+    if (kv->batch_size != p->batch_size || kv->page_size != p->page_size || kv->num_kv_heads != p->num_kv_heads ||
+        kv->head_dim != p->head_dim || num_qo_heads != p->num_qo_heads)
+        return BZ_ERR_BAD_ARG;
+    if (q_dtype != BZ_F16 && q_dtype != BZ_BF16) return BZ_ERR_UNSUPPORTED;
+    if (out_dtype != q_dtype && out_dtype != BZ_F32) return BZ_ERR_UNSUPPORTED;
+    if (kv->kv_dtype != q_dtype && kv->kv_dtype != BZ_E4M3) return BZ_ERR_UNSUPPORTED;
+    hipStream_t s = (hipStream_t)stream;
+    if (p->batch_size == 0) return 0;
+    int rc = BZ_ERR_UNSUPPORTED;
+    if (!p->force_general && p->num_segments > 0) {
+        const int D = (int)kv->head_dim;
+        const float scale = sm_scale > 0.f ? sm_scale : 1.0f / sqrtf((float)D);
+        const RopeFreqs freqs = make_rope_freqs(D, rope_theta > 0.f ? rope_theta : 1e4f);
+        rc = decode_step_fast_path(p, q, k_new, v_new, out, lse, q_dtype, out_dtype, rope, scale * 1.4426950408889634f,
+                                   freqs, kv, num_qo_heads, k_scale, v_scale, s);
+        if (rc == 0 && p->num_empty > 0) { // sequences without pages: nothing to append, zero rows
+            const uint32_t row = num_qo_heads * D;
+            if (out_dtype == BZ_F32) launch_zero<float>(p, out, row, s);
+            else if (out_dtype == BZ_F16) launch_zero<f16_t>(p, out, row, s);
+            else launch_zero<bf16_t>(p, out, row, s);
+            BZ_LAUNCH_CHECK();
+        }
+    }
+    if (rc != BZ_ERR_UNSUPPORTED) return rc;
+    // shapes the matrix-core kernel does not take, or a workspace without room for one partial per piece:
+    // the same result from the two calls the step stands for
+    rc = bz_append_decode_kv(kv, k_new, v_new, q_dtype, nullptr, 0, rope, rope_theta, k_scale, v_scale, stream);
+    if (rc) return rc;
+    return batch_decode_impl(p, q, q_dtype, kv, out, out_dtype, num_qo_heads, rope ? BZ_ROPE_Q_ONLY : BZ_ROPE_NONE,
+                             rope_theta, sm_scale, k_scale, v_scale, lse, nullptr, stream);
 }
 
 extern "C" size_t bz_batch_decode_noalloc_scratch_bytes(void) { return BZ_DECODE_NOALLOC_SCRATCH_BYTES; }

@@ -70,6 +70,9 @@ struct MfmaDecodeArgs {
     uint64_t stride_page, stride_n, stride_h; // elements
     uint32_t page_size, num_qo_heads, group; // group: q heads per scheduled unit (<= 16)
     int rope_q;
+    int step_mode; // 1 = first half of the one-call decode step: the last token of every sequence is left to the
+                   // finishing kernel (which also appends it), q is rotated at its position, and every piece,
+                   // split or not, leaves a partial result in the slot numbered like the piece
     float sm_scale_log2;
     const float* k_scale; // e4m3 pool only: per-kv-head dequantisation factors (nullptr = 1)
     const float* v_scale;
@@ -150,6 +153,12 @@ __device__ __forceinline__ void wave_lds_sync() {
 }
 
 constexpr int kInfoInts = 12; // per-tile description kept in LDS (see fetch_info): 10 ints, padded
+constexpr int kInfoChunk = 16; // tile descriptions fetched per round trip (one lane per tile)
+
+// (Measured and not kept: K rows fetched like V -- four whole 256-byte rows per wave instruction, so that the
+// non-temporal hint covers whole 128-byte lines -- parked in LDS with an XOR swizzle and read back in the
+// A-operand layout.  Same results, but 125 us against 109 us on 128 sequences x 32/8 heads bf16 and 234 against
+// 208 us on 64 x 32/32 heads: the extra LDS round trip sits between a tile's arrival and its arithmetic.)
 
 // KV8: the pool holds e4m3 bytes.  K and V are widened to the 16-bit type of q in registers (exactly)
 // on their way to the matrix cores; the per-head scales are folded into the softmax scale and into
@@ -166,7 +175,8 @@ __global__ __launch_bounds__(64, 2) void decode_mfma_kernel(MfmaDecodeArgs a, co
                                                             const MfmaSlotHead* __restrict__ heads) {
     using M = Mma<BF16>;
     __shared__ __attribute__((aligned(16))) unsigned char v_lds[kTileTok * kVRowBytes];
-    __shared__ __attribute__((aligned(16))) int info_lds[2][32][kInfoInts];
+    __shared__ __attribute__((aligned(16))) int info_lds[2][kInfoChunk][kInfoInts];
+
     // cos / sin of position * frequency i for the piece being opened: one sincosf per lane instead of
     // sixteen (each lane needs the angles of its own 16 contraction indices)
     __shared__ float rope_cs[ROPE_Q ? 2 : 1][64];
@@ -193,13 +203,13 @@ __global__ __launch_bounds__(64, 2) void decode_mfma_kernel(MfmaDecodeArgs a, co
     if (g_begin >= g_end) return;
     const int ahead = max(ahead_raw, 0);
 
-    // ---- descriptions of 32 tiles at a time: lane l < 32 fetches the record of tile base+l, the two
+    // ---- descriptions of kInfoChunk tiles at a time: lane l < kInfoChunk fetches the record of tile base+l, the two
     // page ids it points at and the piece it belongs to, and leaves 10 ints in LDS:
     //   [pid0, pid1, t, seq | kvh, flags (1: first tile of its piece, 2: last), partial, tok_end | seq_len, kv head]
     struct Desc { int v[10]; };
     auto fetch_info = [&](int base) -> Desc {
         Desc d;
-        const int g = base + (lane & 31);
+        const int g = base + (lane & (kInfoChunk - 1));
         const bool live = g < g_end;
         const MfmaTile rec = live ? tiles[g] : MfmaTile{0, 0, 0, 0};
         const int4 m0 = live ? *reinterpret_cast<const int4*>(&pieces[rec.piece]) : make_int4(0, 0, 0, 0);
@@ -211,14 +221,14 @@ __global__ __launch_bounds__(64, 2) void decode_mfma_kernel(MfmaDecodeArgs a, co
         d.v[3] = m0.x;                                             // seq
         d.v[4] = m0.y;                                             // kvh
         d.v[5] = (rec.t == m0.z ? 1 : 0) | (rec.t + 1 == m0.w ? 2 : 0);
-        d.v[6] = m1.x;                                             // partial slot or -1
-        d.v[8] = max(m2.z - ahead, 0);                             // seq_len at present
+        d.v[6] = a.step_mode ? rec.piece : m1.x;                   // partial slot or -1
+        d.v[8] = max(m2.z - ahead - a.step_mode, 0);               // tokens attended over at present
         d.v[7] = min(m0.w * kTileTok, d.v[8]);                     // tok_end of the piece
         d.v[9] = m2.w;                                             // kv head whose K/V are read (kvh is the scheduled unit)
         return d;
     };
     auto stash_info = [&](const Desc& d, int buf) {
-        if (lane < 32) {
+        if (lane < kInfoChunk) {
             int* dst = &info_lds[buf][lane][0];
             *reinterpret_cast<int4*>(dst) = make_int4(d.v[0], d.v[1], d.v[2], d.v[3]);
             *reinterpret_cast<int4*>(dst + 4) = make_int4(d.v[4], d.v[5], d.v[6], d.v[7]);
@@ -298,9 +308,10 @@ __global__ __launch_bounds__(64, 2) void decode_mfma_kernel(MfmaDecodeArgs a, co
     TileUni un; // description of the tile whose loads are issued next
     un.pid0 = indices[first.idx0];
     un.pid1 = indices[first.idx1];
-    un.t = first.t; un.seq = first.seq; un.kvh = first.kvh; un.flags = first.flags; un.partial = first.partial;
+    un.t = first.t; un.seq = first.seq; un.kvh = first.kvh; un.flags = first.flags;
+    un.partial = a.step_mode ? first.piece : first.partial;
     un.kvr = first.kv_head;
-    un.seq_len = max(first.seq_len - ahead, 0);
+    un.seq_len = max(first.seq_len - ahead - a.step_mode, 0);
     un.tok_end = min(first.tile_end * kTileTok, un.seq_len);
     issue_q(un);
     issue_loads(tile_base(un));
@@ -321,14 +332,15 @@ __global__ __launch_bounds__(64, 2) void decode_mfma_kernel(MfmaDecodeArgs a, co
         // wave has nothing in flight.
         TileBase nb;
         if (g + 1 < g_end) {
-            const int nbuf = (i + 1 == 32) ? buf ^ 1 : buf;
-            un = read_info(nbuf, (i + 1) & 31);
+            const int nbuf = (i + 1 == kInfoChunk) ? buf ^ 1 : buf;
+            un = read_info(nbuf, (i + 1) & (kInfoChunk - 1));
             nb = tile_base(un);
         }
         __builtin_amdgcn_sched_barrier(0);
-        // descriptions of the next 32 tiles: fetched at i == 8, parked in the other LDS buffer at i == 24
-        if (i == 8 && chunk_base + 32 < g_end) dnext = fetch_info(chunk_base + 32);
-        if (i == 24 && chunk_base + 32 < g_end) { stash_info(dnext, buf ^ 1); wave_lds_sync(); }
+        // descriptions of the next chunk of tiles: fetched a quarter into this chunk, parked in the other LDS
+        // buffer at three quarters
+        if (i == kInfoChunk / 4 && chunk_base + kInfoChunk < g_end) dnext = fetch_info(chunk_base + kInfoChunk);
+        if (i == 3 * kInfoChunk / 4 && chunk_base + kInfoChunk < g_end) { stash_info(dnext, buf ^ 1); wave_lds_sync(); }
         const int t = uc.t, tok_end = uc.tok_end, seq_len = uc.seq_len;
         // (positive; the floor keeps masked scores at -inf instead of NaN should a head's K scale be zero)
         const float score_scale = fmaxf(a.sm_scale_log2 * ((KV8 && a.k_scale) ? a.k_scale[uc.kvr] : 1.0f), 1e-30f);
@@ -338,7 +350,7 @@ __global__ __launch_bounds__(64, 2) void decode_mfma_kernel(MfmaDecodeArgs a, co
             for (int ks = 0; ks < 4; ++ks) { qhi[ks] = qnext[ks]; qlo[ks] = make_uint4(0, 0, 0, 0); }
             if (ROPE_Q) {
                 float sn1, cs1;
-                sincosf((float)(seq_len - 1) * a.freqs.f[lane], &sn1, &cs1);
+                sincosf((float)(seq_len - 1 + a.step_mode) * a.freqs.f[lane], &sn1, &cs1); // q sits at the last token
                 wave_lds_sync(); // the previous piece's reads of the table are done
                 rope_cs[0][lane] = cs1;
                 rope_cs[ROPE_Q ? 1 : 0][lane] = sn1; // (the index keeps the one-row dummy of the other instantiations in bounds)
@@ -419,7 +431,7 @@ __global__ __launch_bounds__(64, 2) void decode_mfma_kernel(MfmaDecodeArgs a, co
         // registers, so the loads go out before the contraction.
         auto issue_next = [&]() {
             if (g + 1 < g_end) {
-                if (i + 1 == 32) { chunk_base += 32; buf ^= 1; }
+                if (i + 1 == kInfoChunk) { chunk_base += kInfoChunk; buf ^= 1; }
                 if (un.flags & 1) issue_q(un); // next tile opens a new piece
                 issue_loads(nb);
             }
@@ -616,6 +628,235 @@ __global__ __launch_bounds__(128 * S) void decode_mfma_combine_kernel(const Mfma
     if (lse && d == 0) lse[hq] = (M + log2f(wsum)) * 0.6931471805599453f;
 }
 
+// ---- second half of the one-call decode step -------------------------------------------------------------
+// The decode kernel above has attended over every token but the newest of each sequence and left one partial
+// result per piece.  This kernel takes the newest token from the caller's rows instead of from the pool: it
+// rotates the new K row (and q, in registers) at position seq_len-1, writes K and V into their page slot -- the
+// append -- and folds the token's own term exp(q.k) v into the merge of the partials.  One workgroup per
+// (sequence, scheduled unit, q head): 128 lanes (one per output dimension) x S slices over the partials, as in
+// the combine kernel.  The appended rows carry the same bits the append kernel writes.
+template <typename T> __device__ __forceinline__ float pool_to_f32(T v) { return to_f32(v); }
+template <> __device__ __forceinline__ float pool_to_f32<e4m3_t>(e4m3_t v) {
+    return __builtin_amdgcn_cvt_f32_fp8((int)v.bits, 0);
+}
+template <typename T> __device__ __forceinline__ T pool_from_f32(float f) { return StoreCvt<T>::from(f); }
+template <> __device__ __forceinline__ e4m3_t pool_from_f32<e4m3_t>(float f) { return e4m3_t{f32_to_e4m3_bits(f)}; }
+
+struct StepFinishArgs {
+    const void* q;
+    const void* k_new;
+    const void* v_new;
+    char* k_data;
+    char* v_data;
+    const int32_t* indices;
+    const int32_t* indptr;
+    const int32_t* last_page_len;
+    const int32_t* steps_ahead;
+    const MfmaUnit* units;
+    const float* part_o;   // [pieces][16][128]
+    const float* part_lse; // [pieces][16]
+    void* out;
+    float* lse;
+    const float* k_scale;
+    const float* v_scale;
+    uint64_t stride_page, stride_n, stride_h;
+    uint32_t page_size, num_qo_heads, num_kv_heads, group, parts;
+    int rope;
+    float sm_scale_log2;
+    RopeFreqs freqs;
+};
+
+// Thread layout: 32 lanes per q head, four consecutive output dimensions per lane (16-byte loads of the partial
+// rows); HB heads of the unit share a workgroup (threadIdx.y) and with it the angles of the new token's
+// position; S slices (threadIdx.z) split a long list of partials.  The kernel is short enough that the number
+// of instructions its waves issue, not the bytes they move, sets its duration.
+template <typename T> __device__ __forceinline__ void load4_f32(const T* p, float* f) { // four 16-bit elements
+    const uint2 w = *reinterpret_cast<const uint2*>(p);
+    f[0] = to_f32(T{(uint16_t)(w.x & 0xffffu)});
+    f[1] = to_f32(T{(uint16_t)(w.x >> 16)});
+    f[2] = to_f32(T{(uint16_t)(w.y & 0xffffu)});
+    f[3] = to_f32(T{(uint16_t)(w.y >> 16)});
+}
+template <typename T> __device__ __forceinline__ void store4(T* p, const T* v) { // four 16-bit elements
+    *reinterpret_cast<uint2*>(p) = make_uint2((uint32_t)v[0].bits | ((uint32_t)v[1].bits << 16),
+                                              (uint32_t)v[2].bits | ((uint32_t)v[3].bits << 16));
+}
+template <> __device__ __forceinline__ void store4<e4m3_t>(e4m3_t* p, const e4m3_t* v) {
+    *reinterpret_cast<uint32_t*>(p) = (uint32_t)v[0].bits | ((uint32_t)v[1].bits << 8) | ((uint32_t)v[2].bits << 16) |
+                                      ((uint32_t)v[3].bits << 24);
+}
+template <> __device__ __forceinline__ void store4<float>(float* p, const float* v) {
+    *reinterpret_cast<float4*>(p) = make_float4(v[0], v[1], v[2], v[3]);
+}
+
+template <typename QT, typename PT, typename OT, int S, int HB>
+__global__ __launch_bounds__(32 * HB * S) void decode_step_finish_kernel(StepFinishArgs a) {
+    __shared__ float s_cos[64], s_sin[64];
+    const MfmaUnit u = a.units[blockIdx.x];
+    const uint32_t t = threadIdx.x, hl = threadIdx.y, sl = threadIdx.z;
+    const uint32_t g_raw = blockIdx.y * HB + hl;
+    const bool head_live = g_raw < a.group;           // a group that is no multiple of HB leaves lanes idle
+    const uint32_t g = head_live ? g_raw : a.group - 1;
+    const int b = u.seq;
+    const int kvr = u.unit / (int)a.parts; // the kv head whose K/V the unit reads
+    const uint32_t hq = (uint32_t)u.unit * a.group + g;
+    const uint32_t d0 = 4 * t;             // this lane's four output dimensions
+    const bool upper = d0 >= 64;           // they are the second elements of their rotate-half pairs
+    const uint32_t i0 = d0 & 63, dp = upper ? d0 - 64 : d0 + 64;
+    // Everything that depends on the unit record alone is requested at once: the caller's rows, the scales
+    // and the first four partial results of this slice.  (The sequence's length and its place in the page
+    // list come with the unit record, from the host table the plan was made from, like the lengths the
+    // decode kernel works with.)
+    const int ahead_raw = a.steps_ahead ? *a.steps_ahead : 0;
+    const QT* qrow = reinterpret_cast<const QT*>(a.q) + ((size_t)b * a.num_qo_heads + hq) * 128;
+    const QT* krow = reinterpret_cast<const QT*>(a.k_new) + ((size_t)b * a.num_kv_heads + kvr) * 128;
+    const QT* vrow = reinterpret_cast<const QT*>(a.v_new) + ((size_t)b * a.num_kv_heads + kvr) * 128;
+    float q_own[4], q_par[4], k_own[4], k_par[4], v_in[4];
+    load4_f32(qrow + d0, q_own);
+    load4_f32(qrow + dp, q_par);
+    load4_f32(krow + d0, k_own);
+    load4_f32(krow + dp, k_par);
+    load4_f32(vrow + d0, v_in);
+    const float ksc = a.k_scale ? a.k_scale[kvr] : 1.0f, vsc = a.v_scale ? a.v_scale[kvr] : 1.0f;
+    constexpr int NB = 4; // partials per batch of loads
+    auto load_batch = [&](int j0, float* li, float4* oi) {
+#pragma unroll
+        for (int k = 0; k < NB; ++k) {
+            const bool live = j0 + k < u.count;
+            const size_t slot = (size_t)(u.first_piece + (live ? j0 + k : 0));
+            li[k] = live ? a.part_lse[slot * 16 + g] : -INFINITY;
+            oi[k] = *reinterpret_cast<const float4*>(a.part_o + (slot * 16 + g) * 128 + d0);
+        }
+    };
+    float li0[NB];
+    float4 oi0[NB];
+    load_batch(NB * (int)sl, li0, oi0);
+
+    const int seq_len = u.seq_len - max(ahead_raw, 0);
+    OT* orow = reinterpret_cast<OT*>(a.out) + ((size_t)b * a.num_qo_heads + hq) * 128;
+    if (seq_len <= 0) { // no token at present: nothing to append, a zero row
+        const OT z[4] = {StoreCvt<OT>::from(0.f), StoreCvt<OT>::from(0.f), StoreCvt<OT>::from(0.f), StoreCvt<OT>::from(0.f)};
+        if (sl == 0 && head_live) store4(orow + d0, z);
+        if (a.lse && sl == 0 && head_live && t == 0) a.lse[(size_t)b * a.num_qo_heads + hq] = -INFINITY;
+        return;
+    }
+    const int pos = seq_len - 1;
+
+    // ---- the newest token: rotated q and K elements of this lane, the bits the cache gets, the score
+    float v_term[4], s_new;
+    {
+        float qd[4], kd[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) { qd[e] = q_own[e]; kd[e] = k_own[e]; }
+        if (a.rope) {
+            const uint32_t tid = t + 32 * (hl + HB * sl);
+            for (uint32_t i = tid; i < 64; i += 32 * HB * S) {
+                float sn0, cs0;
+                sincosf((float)pos * a.freqs.f[i], &sn0, &cs0);
+                s_cos[i] = cs0;
+                s_sin[i] = sn0;
+            }
+            __syncthreads();
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const float sn = s_sin[i0 + e], cs = s_cos[i0 + e];
+                float xr, yr;
+                rope_pair(upper ? q_par[e] : q_own[e], upper ? q_own[e] : q_par[e], cs, sn, xr, yr);
+                qd[e] = upper ? yr : xr;
+                rope_pair(upper ? k_par[e] : k_own[e], upper ? k_own[e] : k_par[e], cs, sn, xr, yr);
+                kd[e] = upper ? yr : xr;
+            }
+        }
+        PT k_st[4], v_st[4];
+        float dot = 0.f;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            k_st[e] = pool_from_f32<PT>(a.k_scale ? kd[e] / ksc : kd[e]);
+            v_st[e] = pool_from_f32<PT>(a.v_scale ? v_in[e] / vsc : v_in[e]);
+            // the score against the K bits as cached, exactly as a later step will see them
+            dot += qd[e] * pool_to_f32(k_st[e]);
+            v_term[e] = pool_to_f32(v_st[e]) * vsc;
+        }
+        if (g_raw == 0 && sl == 0 && u.unit % (int)a.parts == 0) { // the append: one head's lanes per (sequence, kv head)
+            const int64_t page = a.indices[u.ip0 + pos / (int)a.page_size];
+            const size_t off = (size_t)page * a.stride_page + (size_t)(pos % (int)a.page_size) * a.stride_n +
+                               (size_t)kvr * a.stride_h + d0;
+            store4(reinterpret_cast<PT*>(a.k_data) + off, k_st);
+            store4(reinterpret_cast<PT*>(a.v_data) + off, v_st);
+        }
+#pragma unroll
+        for (int o = 16; o > 0; o >>= 1) dot += __shfl_xor(dot, o, 64); // over the 32 lanes of the head
+        s_new = dot * a.sm_scale_log2 * ksc;
+    }
+
+    // ---- the partial results of the older tokens (normalised rows and base-2 log-sum-exp per piece)
+    float M = -INFINITY, wsum = 0.f, o[4] = {0.f, 0.f, 0.f, 0.f};
+    auto merge_batch = [&](const float* li, const float4* oi) {
+        float m2 = M;
+#pragma unroll
+        for (int k = 0; k < NB; ++k) m2 = fmaxf(m2, li[k]);
+        if (m2 == -INFINITY) return;
+        const float sc = __builtin_amdgcn_exp2f(M - m2); // 0 while nothing has been merged yet
+        wsum *= sc;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) o[e] *= sc;
+#pragma unroll
+        for (int k = 0; k < NB; ++k) {
+            const float w = __builtin_amdgcn_exp2f(li[k] - m2); // -inf -> 0 (and the row read for a dead slot is finite)
+            wsum += w;
+            o[0] += w * oi[k].x;
+            o[1] += w * oi[k].y;
+            o[2] += w * oi[k].z;
+            o[3] += w * oi[k].w;
+        }
+        M = m2;
+    };
+    merge_batch(li0, oi0);
+    for (int j0 = NB * (int)sl + NB * S; j0 < u.count; j0 += NB * S) {
+        float li[NB];
+        float4 oi[NB];
+        load_batch(j0, li, oi);
+        merge_batch(li, oi);
+    }
+    if constexpr (S > 1) {
+        __shared__ float sm_m[S][HB][32], sm_w[S][HB][32];
+        __shared__ float4 sm_o[S][HB][32];
+        sm_m[sl][hl][t] = M;
+        sm_w[sl][hl][t] = wsum;
+        sm_o[sl][hl][t] = make_float4(o[0], o[1], o[2], o[3]);
+        __syncthreads();
+        if (sl != 0) return;
+        float mm = -INFINITY;
+#pragma unroll
+        for (int z = 0; z < S; ++z) mm = fmaxf(mm, sm_m[z][hl][t]);
+        wsum = 0.f;
+        o[0] = o[1] = o[2] = o[3] = 0.f;
+        if (mm != -INFINITY) {
+#pragma unroll
+            for (int z = 0; z < S; ++z) {
+                const float sc = __builtin_amdgcn_exp2f(sm_m[z][hl][t] - mm); // an empty slice has M = -inf: weight 0
+                const float4 oz = sm_o[z][hl][t];
+                wsum += sm_w[z][hl][t] * sc;
+                o[0] += oz.x * sc;
+                o[1] += oz.y * sc;
+                o[2] += oz.z * sc;
+                o[3] += oz.w * sc;
+            }
+        }
+        M = mm;
+    }
+    // ---- the newest token joins with weight 2^(s_new - max)
+    const float m_all = fmaxf(M, s_new);
+    const float sc_old = __builtin_amdgcn_exp2f(M - m_all); // 0 when there are no older tokens
+    const float w_new = __builtin_amdgcn_exp2f(s_new - m_all);
+    const float denom = wsum * sc_old + w_new, inv = 1.0f / denom;
+    OT res[4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) res[e] = StoreCvt<OT>::from((o[e] * sc_old + w_new * v_term[e]) * inv);
+    if (head_live) store4(orow + d0, res);
+    if (a.lse && head_live && t == 0) a.lse[(size_t)b * a.num_qo_heads + hq] = (m_all + log2f(denom)) * 0.6931471805599453f;
+}
+
 struct DecodeArgs; // general-kernel argument block (bz_decode.hip); only its scalar fields are forwarded here
 
 template <bool BF16, typename OT, bool ROPE_Q, bool KV8>
@@ -640,6 +881,7 @@ static int launch_mfma(const DecodePlan* p, const MfmaDecodeArgs& a, bool kv8, h
     }
     BZ_LAUNCH_CHECK();
     if (p->time_stop) BZ_CHECK_HIP(hipEventRecord(p->time_stop, s));
+    if (a.step_mode) return 0; // the finishing kernel of the one-call step folds the partials
     if (p->mfma_combos > 0) {
         const dim3 cgrid(p->mfma_combos, a.group);
         if (p->mfma_max_count <= 16)
@@ -659,7 +901,7 @@ static int launch_mfma(const DecodePlan* p, const MfmaDecodeArgs& a, bool kv8, h
 int decode_fast_path(const DecodePlan* p, const void* q, void* out, float* lse, int q_dtype, int out_dtype,
                      int rope_mode, float sm_scale_log2, const RopeFreqs& freqs, const bz_paged_kv_t* kv,
                      uint32_t num_qo_heads, const float* k_scale, const float* v_scale, float* part_o,
-                     float* part_lse, hipStream_t s) {
+                     float* part_lse, bool step_mode, hipStream_t s) {
     if (!p->mfma_ok || p->mfma_slots == 0) return BZ_ERR_UNSUPPORTED;
     const bool kv8 = kv->kv_dtype == BZ_E4M3;
     if ((!kv8 && kv->kv_dtype != q_dtype) || rope_mode == BZ_ROPE_FULL) return BZ_ERR_UNSUPPORTED;
@@ -678,12 +920,78 @@ int decode_fast_path(const DecodePlan* p, const void* q, void* out, float* lse, 
     a.page_size = kv->page_size; a.num_qo_heads = num_qo_heads;
     a.group = num_qo_heads / kv->num_kv_heads / p->mfma_parts;
     a.rope_q = rope_mode == BZ_ROPE_Q_ONLY;
+    a.step_mode = step_mode ? 1 : 0;
     a.sm_scale_log2 = sm_scale_log2;
     a.k_scale = k_scale; a.v_scale = v_scale;
     a.freqs = freqs;
     if (q_dtype == BZ_BF16)
         return out_dtype == BZ_F32 ? launch_mfma<true, float>(p, a, kv8, s) : launch_mfma<true, bf16_t>(p, a, kv8, s);
     return out_dtype == BZ_F32 ? launch_mfma<false, float>(p, a, kv8, s) : launch_mfma<false, f16_t>(p, a, kv8, s);
+}
+
+template <typename QT, typename PT, typename OT>
+static int launch_step_finish(const DecodePlan* p, const StepFinishArgs& a, hipStream_t s) {
+    // heads of a unit per workgroup: 4 where the group allows it (two waves), else 2 (one wave), 1 for single heads
+    const uint32_t G = a.group;
+    if (p->mfma_unit_max_count <= 16) { // what large batches produce
+        if (G >= 4)
+            hipLaunchKernelGGL((decode_step_finish_kernel<QT, PT, OT, 1, 4>), dim3(p->mfma_units, (G + 3) / 4), dim3(32, 4, 1), 0, s, a);
+        else if (G >= 2)
+            hipLaunchKernelGGL((decode_step_finish_kernel<QT, PT, OT, 1, 2>), dim3(p->mfma_units, (G + 1) / 2), dim3(32, 2, 1), 0, s, a);
+        else
+            hipLaunchKernelGGL((decode_step_finish_kernel<QT, PT, OT, 1, 1>), dim3(p->mfma_units, G), dim3(32, 1, 1), 0, s, a);
+    } else if (p->mfma_unit_max_count <= 64) {
+        hipLaunchKernelGGL((decode_step_finish_kernel<QT, PT, OT, 4, 2>), dim3(p->mfma_units, (G + 1) / 2), dim3(32, 2, 4), 0, s, a);
+    } else {
+        hipLaunchKernelGGL((decode_step_finish_kernel<QT, PT, OT, 8, 2>), dim3(p->mfma_units, (G + 1) / 2), dim3(32, 2, 8), 0, s, a);
+    }
+    BZ_LAUNCH_CHECK();
+    return 0;
+}
+
+template <typename QT, typename OT>
+static int launch_step_finish_kv(const DecodePlan* p, const StepFinishArgs& a, bool kv8, hipStream_t s) {
+    return kv8 ? launch_step_finish<QT, e4m3_t, OT>(p, a, s) : launch_step_finish<QT, QT, OT>(p, a, s);
+}
+
+// The one-call decode step on the matrix-core kernel: BZ_ERR_UNSUPPORTED when the shape, the plan or the
+// float workspace does not allow it (the caller then runs the append and the decode as two calls).
+int decode_step_fast_path(const DecodePlan* p, const void* q, const void* k_new, const void* v_new, void* out,
+                          float* lse, int q_dtype, int out_dtype, int rope, float sm_scale_log2,
+                          const RopeFreqs& freqs, const bz_paged_kv_t* kv, uint32_t num_qo_heads, const float* k_scale,
+                          const float* v_scale, hipStream_t s) {
+    if (!p->mfma_ok || p->mfma_slots == 0 || !p->mfma_units_d || p->mfma_units == 0) return BZ_ERR_UNSUPPORTED;
+    // one partial per piece, in the float workspace the plan was given
+    const size_t part_o_bytes = ((size_t)p->mfma_pieces * 16 * 128 * sizeof(float) + 255) / 256 * 256;
+    const size_t part_lse_bytes = ((size_t)p->mfma_pieces * 16 * sizeof(float) + 255) / 256 * 256;
+    if (part_o_bytes + part_lse_bytes > p->float_buffer_bytes) return BZ_ERR_UNSUPPORTED;
+    float* part_o = p->mfma_part_o;
+    float* part_lse = reinterpret_cast<float*>(reinterpret_cast<char*>(p->mfma_part_o) + part_o_bytes);
+    const int rc = decode_fast_path(p, q, out, lse, q_dtype, out_dtype, rope ? BZ_ROPE_Q_ONLY : BZ_ROPE_NONE,
+                                    sm_scale_log2, freqs, kv, num_qo_heads, k_scale, v_scale, part_o, part_lse, true, s);
+    if (rc) return rc;
+    StepFinishArgs a;
+    a.q = q; a.k_new = k_new; a.v_new = v_new;
+    a.k_data = (char*)kv->k_data; a.v_data = (char*)kv->v_data;
+    a.indices = kv->indices; a.indptr = kv->indptr; a.last_page_len = kv->last_page_len;
+    a.steps_ahead = kv->steps_ahead;
+    a.units = p->mfma_units_d;
+    a.part_o = part_o; a.part_lse = part_lse;
+    a.out = out; a.lse = lse;
+    a.k_scale = k_scale; a.v_scale = v_scale;
+    a.stride_page = kv->stride_page; a.stride_n = kv->stride_n; a.stride_h = kv->stride_h;
+    a.page_size = kv->page_size; a.num_qo_heads = num_qo_heads; a.num_kv_heads = kv->num_kv_heads;
+    a.parts = p->mfma_parts;
+    a.group = num_qo_heads / kv->num_kv_heads / p->mfma_parts;
+    a.rope = rope ? 1 : 0;
+    a.sm_scale_log2 = sm_scale_log2;
+    a.freqs = freqs;
+    const bool kv8 = kv->kv_dtype == BZ_E4M3;
+    if (q_dtype == BZ_BF16)
+        return out_dtype == BZ_F32 ? launch_step_finish_kv<bf16_t, float>(p, a, kv8, s)
+                                   : launch_step_finish_kv<bf16_t, bf16_t>(p, a, kv8, s);
+    return out_dtype == BZ_F32 ? launch_step_finish_kv<f16_t, float>(p, a, kv8, s)
+                               : launch_step_finish_kv<f16_t, f16_t>(p, a, kv8, s);
 }
 
 } // namespace bz

@@ -54,6 +54,7 @@ struct ScheduleCounts {
 struct ScheduleLayout {
     size_t seg_bytes, combo_bytes, empty_bytes, base_total, part_o_bytes, part_lse_bytes;
     size_t mp_bytes, nheads, mptr_bytes, mc_bytes, cnt_bytes, mpart_o_bytes, mpart_lse_bytes;
+    size_t unit_bytes, step_part_o_bytes, step_part_lse_bytes; // one-call decode step: unit list, one partial per piece
 };
 
 // Pure host work: fills the plan's host scratch (h_*) from the host copies of the page table.
@@ -118,7 +119,8 @@ static int build_schedule(DecodePlan* p, const int32_t* indptr_h, const int32_t*
     RawArray<MfmaTile>& mt = p->h_tiles;
     std::vector<int32_t>& mptr = p->h_slot_ptr; // tiles of slot s: [mptr[s], mptr[s+1]); uploaded as one MfmaSlotHead per slot
     std::vector<MfmaCombine>& mc = p->h_mcombos;
-    mp.clear(); mt.clear(); mptr.clear(); mc.clear();
+    std::vector<MfmaUnit>& mu = p->h_units;
+    mp.clear(); mt.clear(); mptr.clear(); mc.clear(); mu.clear();
     uint32_t mfma_partials = 0;
     // A group of more than 16 q heads per kv head does not fit the 16 columns of the score tile: it is
     // scheduled as `parts` equal parts, each a kv head of its own as far as the schedule goes (heads
@@ -219,6 +221,7 @@ static int build_schedule(DecodePlan* p, const int32_t* indptr_h, const int32_t*
                     t += take;
                 }
                 const size_t cnt = mp.size() - first_piece;
+                mu.push_back({(int32_t)b, (int32_t)h, (int32_t)first_piece, (int32_t)cnt, indptr_h[b], (int32_t)len, {0, 0}});
                 if (cnt > 1) {
                     mc.push_back({(int32_t)b, (int32_t)h, (int32_t)mfma_partials, (int32_t)cnt});
                     for (size_t i = 0; i < cnt; ++i) {
@@ -257,6 +260,9 @@ static ScheduleLayout schedule_layout(const DecodePlan* p, const ScheduleCounts&
     L.cnt_bytes = align_up(p->h_tiles.size() * sizeof(MfmaTile), 256); // tile records
     L.mpart_o_bytes = align_up((size_t)c.mfma_partials * 16 * 128 * sizeof(float), 256);
     L.mpart_lse_bytes = align_up((size_t)c.mfma_partials * 16 * sizeof(float), 256);
+    L.unit_bytes = align_up(p->h_units.size() * sizeof(MfmaUnit), 256);
+    L.step_part_o_bytes = align_up(p->h_pieces.size() * 16 * 128 * sizeof(float), 256);
+    L.step_part_lse_bytes = align_up(p->h_pieces.size() * 16 * sizeof(float), 256);
     return L;
 }
 
@@ -296,7 +302,10 @@ extern "C" int bz_decode_plan(bz_decode_plan_t* plan_, void* float_buffer, size_
     // the MFMA schedule is optional: without room for it the general kernel runs
     const bool mfma_ok = mfma_shape && !mp.empty() && base_total + mp_bytes + mptr_bytes + mc_bytes + cnt_bytes <= int_buffer_bytes &&
                          mpart_o_bytes + mpart_lse_bytes <= float_buffer_bytes;
-    const size_t total = mfma_ok ? base_total + mp_bytes + mptr_bytes + mc_bytes + cnt_bytes : base_total;
+    const size_t mfma_total = base_total + mp_bytes + mptr_bytes + mc_bytes + cnt_bytes;
+    // the unit list of the one-call decode step is optional on top of that
+    const bool units_ok = mfma_ok && mfma_total + L.unit_bytes <= int_buffer_bytes;
+    const size_t total = mfma_ok ? mfma_total + (units_ok ? L.unit_bytes : 0) : base_total;
 
     hipStream_t s = (hipStream_t)stream;
     if (!p->upload_done) BZ_CHECK_HIP(hipEventCreateWithFlags(&p->upload_done, hipEventDisableTiming));
@@ -319,7 +328,7 @@ extern "C" int bz_decode_plan(bz_decode_plan_t* plan_, void* float_buffer, size_
         MfmaSlotHead* heads = reinterpret_cast<MfmaSlotHead*>(st + base_total + mp_bytes);
         for (size_t sl = 0; sl < nheads; ++sl) {
             const int32_t b0 = mptr[sl], e0 = mptr[sl + 1];
-            MfmaSlotHead hd = {b0, e0, 0, 0, 0, 0, 0, 0, -1, 0, 0, 0};
+            MfmaSlotHead hd = {b0, e0, 0, 0, 0, 0, 0, 0, -1, 0, 0, 0, 0, {0, 0, 0}};
             if (b0 < e0) {
                 const MfmaTile& r = mt[(size_t)b0];
                 const MfmaPiece& pc = mp[(size_t)r.piece];
@@ -327,11 +336,13 @@ extern "C" int bz_decode_plan(bz_decode_plan_t* plan_, void* float_buffer, size_
                 hd.seq = pc.seq; hd.kvh = pc.kvh;
                 hd.flags = (r.t == pc.tile_begin ? 1 : 0) | (r.t + 1 == pc.tile_end ? 2 : 0);
                 hd.partial = pc.partial; hd.tile_end = pc.tile_end; hd.seq_len = pc.seq_len; hd.kv_head = pc.kv_head;
+                hd.piece = r.piece;
             }
             heads[sl] = hd;
         }
         if (!mc.empty()) memcpy(st + base_total + mp_bytes + mptr_bytes, mc.data(), mc.size() * sizeof(MfmaCombine));
         memcpy(st + base_total + mp_bytes + mptr_bytes + mc_bytes, mt.data(), mt.size() * sizeof(MfmaTile));
+        if (units_ok && !p->h_units.empty()) memcpy(st + mfma_total, p->h_units.data(), p->h_units.size() * sizeof(MfmaUnit));
     }
     if (total) BZ_CHECK_HIP(hipMemcpyAsync(int_buffer, st, total, hipMemcpyHostToDevice, s));
     BZ_CHECK_HIP(hipEventRecord(p->upload_done, s));
@@ -339,6 +350,7 @@ extern "C" int bz_decode_plan(bz_decode_plan_t* plan_, void* float_buffer, size_
     p->segments_d = (const DecodeSegment*)int_buffer;
     p->combos_d = (const DecodeCombine*)((char*)int_buffer + seg_bytes);
     p->empty_d = (const int32_t*)((char*)int_buffer + seg_bytes + combo_bytes);
+    p->float_buffer_bytes = float_buffer_bytes;
     p->part_o = (float*)float_buffer;
     p->part_lse = (float*)((char*)float_buffer + part_o_bytes);
     p->batch_size = batch_size; p->num_qo_heads = num_qo_heads; p->num_kv_heads = num_kv_heads;
@@ -354,6 +366,10 @@ extern "C" int bz_decode_plan(bz_decode_plan_t* plan_, void* float_buffer, size_
         p->mfma_tiles_d = (const MfmaTile*)((char*)int_buffer + base_total + mp_bytes + mptr_bytes + mc_bytes);
         p->mfma_part_o = (float*)float_buffer; // the two paths never run in the same call: same workspace
         p->mfma_part_lse = (float*)((char*)float_buffer + mpart_o_bytes);
+        p->mfma_units_d = units_ok ? (const MfmaUnit*)((char*)int_buffer + mfma_total) : nullptr;
+        p->mfma_units = (uint32_t)p->h_units.size();
+        p->mfma_unit_max_count = 0;
+        for (const MfmaUnit& u : p->h_units) p->mfma_unit_max_count = std::max(p->mfma_unit_max_count, (uint32_t)u.count);
         p->mfma_slots = (uint32_t)mptr.size() - 1;
         p->mfma_pieces = (uint32_t)mp.size();
         p->mfma_combos = (uint32_t)mc.size();
@@ -391,10 +407,13 @@ extern "C" int bz_decode_plan_workspace(bz_decode_plan_t* plan_, const int32_t* 
     if (rc) return rc;
     const ScheduleLayout L = schedule_layout(p, counts, num_qo_heads, head_dim);
     const bool mfma = counts.mfma_shape && !p->h_pieces.empty();
+    // (the one-call decode step keeps one partial per piece, split or not, and reads the unit list)
     if (float_buffer_bytes)
-        *float_buffer_bytes = std::max(L.part_o_bytes + L.part_lse_bytes, mfma ? L.mpart_o_bytes + L.mpart_lse_bytes : 0);
+        *float_buffer_bytes = std::max(L.part_o_bytes + L.part_lse_bytes,
+                                       mfma ? std::max(L.mpart_o_bytes + L.mpart_lse_bytes,
+                                                       L.step_part_o_bytes + L.step_part_lse_bytes) : 0);
     if (int_buffer_bytes)
-        *int_buffer_bytes = L.base_total + (mfma ? L.mp_bytes + L.mptr_bytes + L.mc_bytes + L.cnt_bytes : 0);
+        *int_buffer_bytes = L.base_total + (mfma ? L.mp_bytes + L.mptr_bytes + L.mc_bytes + L.cnt_bytes + L.unit_bytes : 0);
     return 0;
 }
 
@@ -410,6 +429,7 @@ extern "C" int bz_decode_plan_host_schedule(const bz_decode_plan_t* plan_, int w
     case 4: *data = p->h_slot_ptr.data(); *num_records = p->h_slot_ptr.size(); *ints_per_record = 1; break;
     case 5: *data = (const int32_t*)p->h_pieces.data(); *num_records = p->h_pieces.size(); *ints_per_record = sizeof(MfmaPiece) / 4; break;
     case 6: *data = (const int32_t*)p->h_mcombos.data(); *num_records = p->h_mcombos.size(); *ints_per_record = sizeof(MfmaCombine) / 4; break;
+    case 7: *data = (const int32_t*)p->h_units.data(); *num_records = p->h_units.size(); *ints_per_record = sizeof(MfmaUnit) / 4; break;
     default: return BZ_ERR_BAD_ARG;
     }
     return 0;

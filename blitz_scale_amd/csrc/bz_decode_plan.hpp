@@ -51,6 +51,17 @@ struct MfmaSlotHead {
     int32_t tile_end;     // one past the last tile of the piece
     int32_t seq_len;
     int32_t kv_head;      // kv head of the first tile's piece
+    int32_t piece;        // index of the first tile's piece (its partial slot in the one-call decode step)
+    int32_t pad[3];
+};
+
+// One (sequence, scheduled kv-head unit) with its pieces, for the finishing kernel of the one-call decode
+// step: pieces [first_piece, first_piece + count) are consecutive, and in that mode piece i writes partial
+// slot i.
+struct MfmaUnit {
+    int32_t seq, unit, first_piece, count;
+    int32_t ip0, seq_len; // indptr[seq] and the tokens of the sequence, from the host table the plan was made from
+    int32_t pad[2];
 };
 
 // Growable array of plain records that does not clear what it hands out (the planner overwrites every
@@ -106,6 +117,10 @@ struct DecodePlan {
     const MfmaCombine* mfma_combos_d = nullptr;
     const MfmaTile* mfma_tiles_d = nullptr;
     const MfmaSlotHead* mfma_heads_d = nullptr; // one per wave slot
+    const MfmaUnit* mfma_units_d = nullptr;     // every (sequence with pages, unit); nullptr when it did not fit
+    uint32_t mfma_units = 0;
+    uint32_t mfma_unit_max_count = 0;           // most pieces any (sequence, unit) has
+    size_t float_buffer_bytes = 0;              // size of the float workspace given to plan()
     float* mfma_part_o = nullptr;
     float* mfma_part_lse = nullptr;
     // host scratch of plan(), kept between calls so that a step's plan neither allocates nor faults in
@@ -116,6 +131,7 @@ struct DecodePlan {
     std::vector<MfmaPiece> h_pieces;
     RawArray<MfmaTile> h_tiles;
     std::vector<MfmaCombine> h_mcombos;
+    std::vector<MfmaUnit> h_units;
     // pinned staging for the schedule upload and the event that guards its reuse
     void* staging = nullptr;
     size_t staging_bytes = 0;

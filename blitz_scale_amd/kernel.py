@@ -229,6 +229,17 @@ def batch_decode_attention(handler, q_input, paged_kv, output, num_qo_heads, *, 
     check(rc, "batchDecodeAttention")
 
 
+def decode_step(handler, q_input, k_new, v_new, paged_kv, output, num_qo_heads, *, rope=True, rope_theta=1e4,
+                sm_scale=0.0, k_scale=None, v_scale=None, lse=None, stream=None):
+    """append_decode_kv_cache followed by batch_decode_attention (src/layer/attn.h:196-203) as one call: the
+    new K (rotated when rope) and V rows go into the cache, q is rotated inside the kernels and left as it is."""
+    s = paged_kv.as_struct()
+    rc = _lib.load().bz_decode_step(handler.get(), _ptr(q_input), bz_dtype(q_input), _ptr(k_new), _ptr(v_new), C.byref(s),
+                                    _ptr(output), bz_dtype(output), num_qo_heads, int(rope), rope_theta, sm_scale,
+                                    _ptr(k_scale), _ptr(v_scale), _ptr(lse), _stream(stream))
+    check(rc, "decodeStep")
+
+
 def batch_decode_attention_noalloc(handler, q_input, paged_kv, output, num_qo_heads, *, rope_mode=BZ_ROPE_Q_ONLY,
                                    rope_theta=1e4, sm_scale=0.0, k_scale=None, v_scale=None, lse=None, stream=None):
     """batch_decode_attention with the split-K partials in the library's own fixed device array instead of

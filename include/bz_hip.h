@@ -129,7 +129,9 @@ int bz_decode_plan_workspace(bz_decode_plan_t* plan, const int32_t* indptr_h, co
  * matrix-core kernel, in processing order {position in indices[] of the page of tokens 32t.., of tokens
  * 32t+16.., t, piece}; 4: wave-slot boundaries into those records; 5: pieces {seq, kv head, tile_begin,
  * tile_end, partial | -1, combine index | -1, partials of its (seq, kv head), first of them, indptr[seq],
- * pages, tokens, ...}; 6: split (seq, kv head)s {seq, kv head, first partial, count}. */
+ * pages, tokens, ...}; 6: split (seq, kv head)s {seq, kv head, first partial, count}; 7: every (seq with
+ * pages, kv head) with its run of pieces {seq, kv head, first piece, count, indptr[seq], tokens, ...} (read by
+ * bz_decode_step). */
 int bz_decode_plan_host_schedule(const bz_decode_plan_t* plan, int which, const int32_t** data, size_t* num_records,
                                  uint32_t* ints_per_record);
 /* introspection for tests and the bench: number of segments / of sequences that were split */
@@ -152,6 +154,23 @@ int bz_decode_plan_set_timing_events(bz_decode_plan_t* plan, void* start_event, 
 int bz_batch_decode(bz_decode_plan_t* plan, const void* q, int q_dtype, const bz_paged_kv_t* kv, void* out,
                     int out_dtype, uint32_t num_qo_heads, int rope_mode, float rope_theta, float sm_scale,
                     const float* k_scale, const float* v_scale, float* lse, void* stream);
+
+/*
+ * One layer's decode-time attention step as ONE call: what append_decode_kv_cache followed by
+ * batch_decode_attention compute (src/layer/attn.h:196-203), i.e. bz_append_decode_kv(kv, k_new, v_new, rope)
+ * and then bz_batch_decode(q, rope ? BZ_ROPE_Q_ONLY : BZ_ROPE_NONE), in two launches instead of three and with
+ * the append off the critical path: the decode kernel attends over every token but the newest (it does not
+ * wait for the append), and a finishing kernel rotates and appends the new K/V rows, adds the new token's own
+ * term from the caller's rows and folds the split-K partials.  q [B,Hq,D], k_new, v_new [B,Hkv,D] are read
+ * only (q is rotated in registers); the pool receives the same bits bz_append_decode_kv writes; `out` agrees
+ * with the two-call sequence to rounding (the summation order differs).  Needs a float workspace with room
+ * for one partial per piece (bz_decode_plan_workspace reports it); where the matrix-core kernel does not
+ * apply, or the workspace is too small, the call runs the two-call sequence itself.  Launch only.
+ */
+int bz_decode_step(bz_decode_plan_t* plan, const void* q, int q_dtype, const void* k_new, const void* v_new,
+                   const bz_paged_kv_t* kv, void* out, int out_dtype, uint32_t num_qo_heads, int rope,
+                   float rope_theta, float sm_scale, const float* k_scale, const float* v_scale, float* lse,
+                   void* stream);
 
 /*
  * bz_batch_decode for callers that cannot allocate device memory or bring a float workspace along (code

@@ -24,7 +24,7 @@ def schedule(lens, Hq, Hkv, D, P, split_tokens=0, cus=CUS):
     indices, indptr, lpl = wl.page_table_for(lens, P, max(1, 2 * need), rng)
     h = K.BlitzBatchDecodeHandler()
     fb, ib = h.workspace(indptr, lpl, len(lens), Hq, Hkv, D, P, split_tokens=split_tokens, num_compute_units=cus)
-    names = ["segments", "combos", "empty", "tiles", "slot_ptr", "pieces", "mcombos"]
+    names = ["segments", "combos", "empty", "tiles", "slot_ptr", "pieces", "mcombos", "units"]
     s = {n: h.host_schedule(i) for i, n in enumerate(names)}
     s.update(indptr=np.asarray(indptr), lens=lens, float_bytes=fb, int_bytes=ib)
     return s
@@ -137,10 +137,22 @@ def test_matrix_core_schedule_invariants(name, lens, Hq, Hkv, P, split):
     al = lambda x: (x + 255) // 256 * 256
     n_mp = int(s["mcombos"][:, 3].sum()) if len(s["mcombos"]) else 0  # partial slots of the matrix-core path
     assert s["int_bytes"] == (al(len(s["segments"]) * 16) + al(len(s["combos"]) * 16) + al(len(s["empty"]) * 4) +
-                              al(len(s["pieces"]) * 64) + al((len(s["slot_ptr"]) - 1) * 48) +
-                              al(len(s["mcombos"]) * 16) + al(len(s["tiles"]) * 16))
+                              al(len(s["pieces"]) * 64) + al((len(s["slot_ptr"]) - 1) * 64) +
+                              al(len(s["mcombos"]) * 16) + al(len(s["tiles"]) * 16) + al(len(s["units"]) * 32))
+    # (the one-call decode step keeps one partial per piece, split or not)
     assert s["float_bytes"] == max(al(n_partials * Hq * 128 * 4) + al(n_partials * Hq * 4),
-                                   al(n_mp * 16 * 128 * 4) + al(n_mp * 16 * 4))
+                                   al(n_mp * 16 * 128 * 4) + al(n_mp * 16 * 4),
+                                   al(len(s["pieces"]) * 16 * 128 * 4) + al(len(s["pieces"]) * 16 * 4))
+    # every (sequence with pages, unit) is listed once with its consecutive run of pieces
+    un = s["units"]
+    live = [b for b, l in enumerate(lens) if l > 0]
+    assert [tuple(r[:2]) for r in un] == [(b, h) for b in live for h in range(units)]
+    assert (un[:, 3] >= 1).all() and (un[1:, 2] == un[:-1, 2] + un[:-1, 3]).all() and un[0, 2] == 0
+    assert un[-1, 2] + un[-1, 3] == len(s["pieces"])
+    for b, h, first, cnt, ip0, ntok in un[:: max(1, len(un) // 50), :6]:
+        pc = s["pieces"][first:first + cnt]
+        assert (pc[:, 0] == b).all() and (pc[:, 1] == h).all()
+        assert ip0 == s["indptr"][b] and ntok == lens[b]
 
 
 def test_shapes_outside_the_matrix_core_kernel_get_segments_only():

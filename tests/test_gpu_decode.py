@@ -176,24 +176,28 @@ def test_error_codes():
 
 
 def test_plan_fits_the_workspace_it_reports():
-    """bz_decode_plan_workspace names the bytes plan() needs for the matrix-core kernel: buffers of exactly
-    that size are enough, one section less and the plan falls back to the general kernel (same results)."""
+    """bz_decode_plan_workspace names the bytes plan() needs for the matrix-core kernel and the one-call step:
+    buffers of exactly that size are enough; without room for the last section (the unit list of the one-call
+    step) the matrix-core schedule is still taken; one more section less and the plan falls back to the general
+    kernel (same results every time)."""
     from blitz_scale_amd import kernel as K
     p = DecodeProblem(77, [3000, 40, 900, 2100, 64, 1], 32, 8, 128, 16, BZ_BF16)
     ref = oracle.batch_decode(p.q, p.dtype, p.oracle_kv(), p.Hq)
     h = K.BlitzBatchDecodeHandler()
     fb, ib = h.workspace(p.indptr, p.last_page_len, p.B, p.Hq, p.Hkv, p.D, p.P, split_tokens=1024)
     slots = len(h.host_schedule(4)) - 1
-    assert fb > 0 and ib > 0 and slots > 0
+    unit_bytes = (len(h.host_schedule(7)) * 32 + 255) // 256 * 256
+    assert fb > 0 and ib > 0 and slots > 0 and unit_bytes > 0
     infos = []
-    for int_bytes in (ib, ib - 256):
+    for int_bytes in (ib, ib - 256, ib - unit_bytes - 256):
         dev = DeviceDecode(p, float_ws_bytes=fb, int_ws_bytes=int_bytes)
         info = dev.plan(1024)
         got = dev.decode(None, BZ_ROPE_NONE)
         assert (np.abs(got - ref) <= ulp_tol(ref, p.dtype)).all()
         infos.append(info)
     assert infos[0]["workgroups"] == slots          # the matrix-core schedule was taken
-    assert infos[1]["workgroups"] != slots          # no room for it: page-aligned segments x kv heads
+    assert infos[1]["workgroups"] == slots          # still: only the one-call step's unit list is missing
+    assert infos[2]["workgroups"] != slots          # no room for it: page-aligned segments x kv heads
 
 
 @pytest.mark.parametrize("ctx,expect_min_partials", [

@@ -1,0 +1,160 @@
+"""GPU parity at the FULL batch sizes of BASELINE configs 2 and 5 (and one whole request of config 4).
+
+At these sizes the checker would take minutes over the whole batch, so the HIP path runs the full batch (the
+planner regime of thousands of wave slots, the instantiation with hinted loads, megabytes of tile records) and
+is compared
+  * with the checker on a seeded subset of sequences, all heads (2e-3 for f16 results; 3e-2 with the e4m3 pool),
+  * on ALL rows through size-independent properties: every output lies in the convex hull of its sequence's V
+    rows, and moving every page to another place in the pool (table updated) leaves the output bit-identical.
+The pools are generated on the device (seeded); only the subset's pages travel to the host for the checker.
+"""
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from blitz_scale_amd import kernel as K
+from blitz_scale_amd import workloads as wl
+from blitz_scale_amd._lib import BZ_BF16, BZ_E4M3, BZ_F16, BZ_F32, BZ_LAYOUT_HND, BZ_ROPE_NONE, BZ_ROPE_Q_ONLY
+
+from _gpu import TORCH_OF, to_host_bits
+from _util import ulp_tol
+
+pytestmark = pytest.mark.gpu
+
+
+class FullBatch:
+    def __init__(self, seed, ctx, Hq, Hkv, D, P, dtype, kv_dtype):
+        self.rng = np.random.default_rng(seed)
+        self.ctx = np.asarray(ctx, np.int64)
+        self.B, self.Hq, self.Hkv, self.D, self.P, self.dtype, self.kv_dtype = len(ctx), Hq, Hkv, D, P, dtype, kv_dtype
+        self.pool_pages = int(((self.ctx + P - 1) // P).sum())
+        self.indices, self.indptr, self.lpl = wl.page_table_for(self.ctx, P, self.pool_pages, self.rng)
+        self.stride_page, self.stride_n, self.stride_h = wl.strides(BZ_LAYOUT_HND, Hkv, P, D)
+        g = torch.Generator(device="cuda")
+        g.manual_seed(seed)
+        tdt = TORCH_OF[dtype]
+        self.k_scale = self.v_scale = None
+        n = self.pool_pages * self.stride_page
+        if kv_dtype == BZ_E4M3:
+            # N(0,1) values; per-kv-head scale amax/448 with amax taken over the whole plane (first pass), then
+            # e4m3 bytes (second pass with the same seeds, chunk by chunk)
+            chunk_pages = 512
+            amax = torch.zeros((2, Hkv), dtype=torch.float32, device="cuda")
+            for c0 in range(0, self.pool_pages, chunk_pages):
+                npg = min(chunk_pages, self.pool_pages - c0)
+                g.manual_seed(seed * 1000003 + c0)
+                x = torch.randn((npg, 2, Hkv, P, D), dtype=torch.float32, device="cuda", generator=g)
+                amax = torch.maximum(amax, x.abs().amax(dim=(0, 3, 4)))
+            scale = amax / 448.0
+            self.k_scale_d, self.v_scale_d = scale[0].contiguous(), scale[1].contiguous()
+            self.k_scale, self.v_scale = self.k_scale_d.cpu().numpy(), self.v_scale_d.cpu().numpy()
+            self.pool = torch.empty(n, dtype=torch.uint8, device="cuda")
+            pv = self.pool.view(self.pool_pages, 2, Hkv, P, D)
+            for c0 in range(0, self.pool_pages, chunk_pages):
+                npg = min(chunk_pages, self.pool_pages - c0)
+                g.manual_seed(seed * 1000003 + c0)
+                x = torch.randn((npg, 2, Hkv, P, D), dtype=torch.float32, device="cuda", generator=g)
+                pv[c0:c0 + npg] = (x / scale[None, :, :, None, None]).to(torch.float8_e4m3fn).view(torch.uint8)
+        else:
+            self.k_scale_d = self.v_scale_d = None
+            self.pool = torch.empty(n, dtype=tdt, device="cuda")
+            self.pool.normal_(generator=g)
+        self.q = torch.randn((self.B, Hq, D), dtype=torch.float32, device="cuda", generator=g).to(tdt)
+        self.float_ws = torch.empty(128 << 20, dtype=torch.uint8, device="cuda")  # the reference's sizes, src/model/llama.h:111-112
+        self.int_ws = torch.empty(8 << 20, dtype=torch.uint8, device="cuda")
+        self.handler = K.BlitzBatchDecodeHandler()
+
+    def table(self, pool, indices):
+        pt = K.PageTable(self.B, self.P, self.Hkv, self.D, pool, layout=BZ_LAYOUT_HND)
+        pt.indices, pt.indptr, pt.last_page_len = indices, self.indptr, self.lpl
+        return pt.upload()
+
+    def decode(self, pt, out_dtype, rope_mode, theta):
+        self.handler.plan(self.float_ws, self.float_ws.numel(), self.int_ws, self.int_ws.numel(), self.indptr, self.lpl,
+                          self.B, self.Hq, self.Hkv, self.D, self.P, split_tokens=2048)
+        out = torch.full((self.B, self.Hq, self.D), float("nan"), dtype=TORCH_OF[out_dtype], device="cuda")
+        K.batch_decode_attention(self.handler, self.q, pt, out, self.Hq, rope_mode=rope_mode, rope_theta=theta,
+                                 k_scale=self.k_scale_d, v_scale=self.v_scale_d)
+        torch.cuda.synchronize()
+        return out
+
+    def checker_on(self, seqs, rope_mode, theta):
+        """The checker on the listed sequences: their pages are gathered into a compact host pool."""
+        pages = np.concatenate([self.indices[self.indptr[b]:self.indptr[b + 1]] for b in seqs])
+        sub = self.pool.view(self.pool_pages, self.stride_page)[torch.from_numpy(pages.astype(np.int64)).cuda()]
+        sub = to_host_bits(sub.contiguous()).reshape(-1)
+        counts = np.array([self.indptr[b + 1] - self.indptr[b] for b in seqs])
+        ip = np.concatenate([[0], np.cumsum(counts)]).astype(np.int32)
+        kv = oracle.PagedKV(sub, sub[self.stride_page // 2:], np.arange(len(pages), dtype=np.int32), ip,
+                            self.lpl[seqs].astype(np.int32), self.P, self.Hkv, self.D, self.stride_page, self.stride_n,
+                            self.stride_h, self.kv_dtype)
+        q = to_host_bits(self.q[torch.from_numpy(np.asarray(seqs, np.int64)).cuda()].contiguous())
+        return oracle.batch_decode(q, self.dtype, kv, self.Hq, rope_mode=rope_mode, rope_theta=theta, k_scale=self.k_scale,
+                                   v_scale=self.v_scale, parallel=True)
+
+    def v_hull(self):
+        """min / max over each sequence's cached V rows: [B, Hkv, D] each (torch, on the device)."""
+        lo = torch.empty((self.B, self.Hkv, self.D), dtype=torch.float32, device="cuda")
+        hi = torch.empty_like(lo)
+        pv = self.pool.view(self.pool_pages, 2, self.Hkv, self.P, self.D)
+        if self.kv_dtype == BZ_E4M3:
+            table = torch.from_numpy(wl.e4m3_bits_to_f32(np.arange(256, dtype=np.uint8))).cuda()
+        for b in range(self.B):
+            idx = torch.from_numpy(self.indices[self.indptr[b]:self.indptr[b + 1]].astype(np.int64)).cuda()
+            v = pv[idx, 1]  # [pages, Hkv, P, D]
+            v = table[v.long()] * self.v_scale_d[None, :, None, None] if self.kv_dtype == BZ_E4M3 else v.float()
+            v = v.permute(1, 0, 2, 3).reshape(self.Hkv, -1, self.D)[:, :int(self.ctx[b])]
+            lo[b], hi[b] = v.amin(dim=1), v.amax(dim=1)
+        return lo, hi
+
+    def check(self, rope_mode, theta, n_subset, base_tol):
+        pt = self.table(self.pool, self.indices)
+        out32 = self.decode(pt, BZ_F32, rope_mode, theta)
+        out = self.decode(pt, self.dtype, rope_mode, theta)
+        info = self.handler.info()
+        assert not torch.isnan(out32).any() and not torch.isnan(out.float()).any()
+        # (1) the checker on a seeded subset of sequences, all heads
+        seqs = np.sort(self.rng.choice(self.B, size=n_subset, replace=False))
+        ref = self.checker_on(seqs, rope_mode, theta)
+        sel = torch.from_numpy(seqs.astype(np.int64)).cuda()
+        got32, got = out32[sel].cpu().numpy(), out[sel].float().cpu().numpy()
+        err32 = float(np.abs(got32 - ref).max())
+        assert err32 <= (base_tol if self.kv_dtype == BZ_E4M3 else 1e-4), err32
+        assert (np.abs(got - ref) <= ulp_tol(ref, self.dtype, base_tol)).all(), float(np.abs(got - ref).max())
+        # (2) every row inside the convex hull of its sequence's V rows
+        lo, hi = self.v_hull()
+        G = self.Hq // self.Hkv
+        o = out32.view(self.B, self.Hkv, G, self.D)
+        eps = 2e-5
+        assert bool((o >= lo[:, :, None, :] - eps).all()) and bool((o <= hi[:, :, None, :] + eps).all())
+        # (3) every page moved to another place in the pool: bit-identical output
+        perm = torch.from_numpy(self.rng.permutation(self.pool_pages).astype(np.int64)).cuda()
+        pool2 = torch.empty_like(self.pool)
+        pool2.view(self.pool_pages, self.stride_page)[perm] = self.pool.view(self.pool_pages, self.stride_page)
+        indices2 = perm.cpu().numpy()[self.indices].astype(np.int32)
+        out2 = self.decode(self.table(pool2, indices2), BZ_F32, rope_mode, theta)
+        assert torch.equal(out2, out32)
+        return info
+
+
+def test_c2_full_batch():
+    """Llama-2-7B MHA decode at its full size: fp16, batch 64, 32/32 heads, contexts U[512,2048], q rotated
+    in the kernel (theta 1e4)."""
+    cfg = wl.CONFIGS["C2"]
+    ctx = wl.ctx_lens_for(cfg, np.random.default_rng(wl.DEFAULT_SEED))
+    assert len(ctx) == 64
+    fb = FullBatch(0xC2, ctx, cfg["Hq"], cfg["Hkv"], cfg["D"], cfg["P"], BZ_F16, BZ_F16)
+    info = fb.check(BZ_ROPE_Q_ONLY, 1e4, n_subset=8, base_tol=2e-3)
+    assert info["workgroups"] >= 2000  # the planner filled the chip's wave slots
+
+
+def test_c5_full_batch():
+    """Llama-3-70B GQA decode with an e4m3 KV pool at its full size: batch 256, 64/8 heads, context 4096,
+    per-kv-head scales amax/448, dequantisation inside the kernel."""
+    cfg = wl.CONFIGS["C5"]
+    ctx = wl.ctx_lens_for(cfg, np.random.default_rng(wl.DEFAULT_SEED))
+    assert len(ctx) == 256 and int(ctx.min()) == 4096
+    fb = FullBatch(0xC5, ctx, cfg["Hq"], cfg["Hkv"], cfg["D"], cfg["P"], BZ_BF16, BZ_E4M3)
+    info = fb.check(BZ_ROPE_NONE, 5e5, n_subset=6, base_tol=3e-2)
+    assert info["workgroups"] >= 2000

@@ -104,6 +104,23 @@ def test_c4_shape_sampled_rows(batch):
     assert np.abs(got[rows] - ref).max() <= 2e-3
 
 
+def test_c4_one_whole_request_of_full_length():
+    """BASELINE config 4 at full size (16 prompts, 40/40 heads): EVERY row of the longest request (all heads)
+    against the checker, i.e. every causal length from 1 to the request's end through every q tile and wave."""
+    cfg = wl.CONFIGS["C4"]
+    rng = np.random.default_rng(wl.DEFAULT_SEED)
+    lens = [int(x) for x in rng.integers(128, 4097, size=16)]
+    lens[5] = 4096  # one request at the maximum length
+    pf = Prefill(wl.DEFAULT_SEED + 1, lens, cfg["Hq"], cfg["Hkv"], cfg["D"], cfg["dtype"])
+    got = pf.run(causal=True)
+    rows = np.arange(pf.indptr[5], pf.indptr[6], dtype=np.int32)
+    assert len(rows) == 4096
+    ref = oracle.batch_prefill_ragged(pf.q, pf.k, pf.v, cfg["dtype"], pf.indptr, cfg["Hq"], cfg["Hkv"], cfg["D"],
+                                      causal=True, rows=rows, parallel=True)
+    assert not np.isnan(got).any()
+    assert np.abs(got[rows] - ref).max() <= 2e-3
+
+
 def test_prefill_error_codes():
     pf = Prefill(230, [5], 4, 4, 128, BZ_F16)
     qd = to_dev(pf.q, BZ_F16)
