@@ -47,6 +47,10 @@ def parse():
                          "(three launches) instead of the one-call decode step")
     ap.add_argument("--no-graph", action="store_true", help="decode workloads: skip the HIP-graph replay pass")
     ap.add_argument("--no-rope", action="store_true", help="decode workloads: leave RoPE out of the step (diagnostic)")
+    ap.add_argument("--q-rope", default="attention", choices=["attention", "store"],
+                    help="C4: where q is rotated. attention: in registers inside the attention kernel (q read once, "
+                         "never written; the page store rotates k only); store: in place by the page-store kernel "
+                         "(the attention kernel then takes q and k as they are)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also launch a few plain device copies of 1 GiB (reference point for rocprofv3 --pmc byte counters)")
     args = ap.parse_args()
@@ -342,7 +346,7 @@ def bench_prefill(args):
     import torch
 
     from blitz_scale_amd import kernel as K, workloads as wl
-    from blitz_scale_amd._lib import BZ_LAYOUT_HND, BZ_ROPE_NONE
+    from blitz_scale_amd._lib import BZ_LAYOUT_HND, BZ_ROPE_NONE, BZ_ROPE_Q_ONLY
 
     dev = "cuda"
     cfg = wl.CONFIGS["C4"]
@@ -382,12 +386,17 @@ def bench_prefill(args):
     plan_ms = (time.perf_counter() - t0) / 10 * 1e3
 
     def step(i, ev):
-        # fused RoPE (q, k in place) + page store, then attention on the rotated rows.  q and k are rotated
-        # again every step; rotations keep the N(0,1) statistics, so the work is the same each time.
-        K.store_prefill_kv_cache(pt, k, v, ip, num_tokens=N, q=q, num_qo_heads=Hq, rope=True, rope_theta=theta)
+        # page store with K rotated on the way (into the pages and in place), then attention, which rotates q in
+        # registers.  k is rotated again every step; rotations keep the N(0,1) statistics, so the work is
+        # the same each time.
+        if args.q_rope == "store":
+            K.store_prefill_kv_cache(pt, k, v, ip, num_tokens=N, q=q, num_qo_heads=Hq, rope=True, rope_theta=theta)
+        else:
+            K.store_prefill_kv_cache(pt, k, v, ip, num_tokens=N, rope=2, rope_theta=theta)
         if ev is not None:
             ev[0].record()
-        K.batch_prefill_attention(handler, q, ip, k, v, ip, out, B, Hq, Hkv, D, causal=True, rope_mode=BZ_ROPE_NONE)
+        K.batch_prefill_attention(handler, q, ip, k, v, ip, out, B, Hq, Hkv, D, causal=True, rope_theta=theta,
+                                  rope_mode=BZ_ROPE_NONE if args.q_rope == "store" else BZ_ROPE_Q_ONLY)
         if ev is not None:
             ev[1].record()
 
@@ -398,9 +407,10 @@ def bench_prefill(args):
         "metric": "ragged_causal_prefill_ms_per_step", "value": round(ms_per_step, 4), "unit": "ms/step",
         "n_gpus": 1, "steps": steps, "warmup": warmup, "ms_per_step": round(ms_per_step, 6),
         "higher_is_better": False, "scaling": "weak", "vs_baseline": None, "dtype": "f16", "data": "synthetic",
-        "config": {"workload": "C4: Llama-2-13B-shaped ragged causal prefill with fused RoPE + KV page store, one layer per step",
+        "config": {"workload": "C4: Llama-2-13B-shaped ragged causal prefill with RoPE + KV page store, one layer per step",
                    "batch": B, "num_qo_heads": Hq, "num_kv_heads": Hkv, "head_dim": D, "page_size": P,
                    "lens": "uniform[128,4096]", "tokens": N, "pool_pages": pool_pages, "rope_theta": theta,
+                   "q_rotated_by": args.q_rope,
                    "seed": hex(args.seed)},
         "tokens_per_s": round(N / (ms_per_step * 1e-3), 1),
         "plan_ms_per_model_step": round(plan_ms, 4),
@@ -418,7 +428,7 @@ def bench_prefill(args):
         qh, kh, vh = (t.view(torch.int16).cpu().numpy().view(np.uint16) for t in (q, k, v))
         K.batch_prefill_attention(handler, q, ip, k, v, ip, out, B, Hq, Hkv, D, causal=True, rope_mode=BZ_ROPE_NONE)
         torch.cuda.synchronize()
-        t0 = time.perf_counter()
+        t0 = time.perf_counter()  # (checked without RoPE on either side: the same q and k bits, used as they are)
         ref = oracle.batch_prefill_ragged(qh, kh, vh, oracle.F16, indptr, Hq, Hkv, D, causal=True, rows=rows, parallel=True)
         cpu_s = time.perf_counter() - t0
         res_json["max_abs_err_vs_cpu"] = float(np.abs(out[torch.from_numpy(rows.astype(np.int64)).to(dev)].float().cpu().numpy() - ref).max())

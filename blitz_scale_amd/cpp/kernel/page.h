@@ -82,7 +82,9 @@ struct PageTable {
 /// num_tokens: rows of k_data / v_data.  q_inout (optional, [N, num_qo_heads, D]): the fused RoPE of the
 /// prefill path -- K is rotated on its way into the pages and q and the caller's k rows are rotated in
 /// place by the same angles, so that batch_prefill_attention runs with BZ_ROPE_NONE afterwards.
-/// rotate: 1 / 0 force K rotation on / off, < 0 = on when q_inout is given, else opts().store_rotates_k.
+/// rotate: 1 / 0 force K rotation on / off, 2 = rotate K into the pages AND in place in the caller's rows
+/// (q is then left to batch_prefill_attention with BZ_ROPE_Q_ONLY), < 0 = on when q_inout is given, else
+/// opts().store_rotates_k.
 template<typename DType, typename IdType, typename SrcType = DType>
 void store_prefill_kv_cache(PageTable<DType, IdType>& page_table, SrcType* k_data, SrcType* v_data,
                             IdType* ragged_indptr, uint32_t num_tokens, SrcType* q_inout = nullptr,
@@ -91,10 +93,10 @@ void store_prefill_kv_cache(PageTable<DType, IdType>& page_table, SrcType* k_dat
     static_assert(sizeof(IdType) == 4, "page tables are int32");
     const AttentionOptions& o = page_table.opts();
     const bz_paged_kv_t kv = page_table.c_view();
-    const bool rot = rotate < 0 ? (q_inout != nullptr || o.store_rotates_k) : rotate != 0;
+    const int rot = rotate < 0 ? ((q_inout != nullptr || o.store_rotates_k) ? 1 : 0) : rotate;
     bz_throw(bz_store_prefill_kv(&kv, k_data, v_data, bz_dtype<SrcType>::value,
                                  reinterpret_cast<const int32_t*>(ragged_indptr), num_tokens, q_inout, num_qo_heads,
-                                 rot ? 1 : 0, o.rope_theta, k_scale, v_scale, o.stream),
+                                 rot, o.rope_theta, k_scale, v_scale, o.stream),
              "AppendPagedKVCache");
 }
 

@@ -3,7 +3,8 @@
 // attention-side work routed to the gfx950 kernels:
 //   decode : the one-call decode step (paged batch decode over the cached tokens, then a kernel that rotates
 //            and appends the new K/V rows, adds the new token's term and folds the split-K partials)
-//   prefill: fused RoPE(q, k) + KV page store, then ragged causal attention on the rotated rows
+//   prefill: KV page store with K rotated on the way (into the pages and in place), then ragged causal
+//            attention that rotates q in registers
 // K is cached rotated, so no kernel ever rotates cached K again.
 #pragma once
 
@@ -70,10 +71,12 @@ class Attention {
         gemm_->gemm(GemmOp::N, GemmOp::N, (int)N, (int)(Hkv_ * D_), (int)hidden_, input, wk_, k);
         gemm_->gemm(GemmOp::N, GemmOp::N, (int)N, (int)(Hkv_ * D_), (int)hidden_, input, wv_, v);
         if (qo_indptr_d) {
-            // fused RoPE(q, k) + page store, then attention on the rotated rows
-            kernel::store_prefill_kv_cache(page_table, k, v, qo_indptr_d, num_tokens, q, Hq_);
+            // K rotated once, into the pages and in place, while the pages are written; q is rotated in registers
+            // inside the attention kernel (read once, never written)
+            kernel::store_prefill_kv_cache(page_table, k, v, qo_indptr_d, num_tokens, static_cast<DType*>(nullptr), 0,
+                                           nullptr, nullptr, /*rotate=*/2);
             kernel::batch_prefill_attention(*prefill_, q, qo_indptr_d, k, v, qo_indptr_d, attn_state,
-                                            page_table.batch_size, Hq_, Hkv_, D_, BZ_ROPE_NONE);
+                                            page_table.batch_size, Hq_, Hkv_, D_, BZ_ROPE_Q_ONLY);
         } else {
             // append (new K rotated on its way in) + decode (q rotated inside the kernels) as one call
             kernel::decode_attention_step(*decode_, q, k, v, page_table, attn_state, Hq_);

@@ -103,7 +103,7 @@ __device__ __forceinline__ void page_write_rows(const PageWriteArgs& a, int64_t 
                 y[e] = yr;
             }
         }
-        if (PREFILL && rotate && Hq > 0) {
+        if (PREFILL && rotate && (Hq > 0 || a.rope == 2)) {
             // fused RoPE of the prefill path: the caller's k rows are rotated in place as well, so the
             // attention call that follows contracts rotated q with rotated k
             Vec8<ST> lr, hr;
@@ -330,7 +330,7 @@ static int fill_args(PageWriteArgs& a, const bz_paged_kv_t* kv, const void* k, c
     a.stride_page = kv->stride_page; a.stride_n = kv->stride_n; a.stride_h = kv->stride_h;
     a.batch_size = kv->batch_size; a.page_size = kv->page_size; a.num_kv_heads = kv->num_kv_heads;
     a.num_qo_heads = num_qo_heads; a.num_tokens = 0;
-    a.rope = rope ? 1 : 0;
+    a.rope = rope == 2 ? 2 : (rope ? 1 : 0);
     a.freqs = make_rope_freqs((int)kv->head_dim, rope_theta > 0.f ? rope_theta : 1e4f);
     return 0;
 }

@@ -71,8 +71,13 @@ struct PrefillItem { // one workgroup's job, in launch order
 struct PrefillPlan {
     bool planned = false;
     uint32_t batch_size = 0, num_qo_heads = 0, num_kv_heads = 0, head_dim = 0, num_items = 0;
-    uint32_t total_tokens = 0;
+    uint32_t total_tokens = 0, max_len = 0;
     const PrefillItem* items_d = nullptr;
+    // cos / sin of position * frequency for every position a request of this batch has (float workspace),
+    // filled by the first attention call that rotates q after a plan(), for the RoPE base of that call
+    float* rope_table = nullptr; // [max_len][64] pairs (cos, sin); nullptr: the float workspace has no room
+    float rope_table_theta = 0.f;
+    bool rope_table_valid = false;
     std::vector<PrefillItem> h_items; // host copy of the last job list (kept between calls)
     void* staging = nullptr;
     size_t staging_bytes = 0;
@@ -82,6 +87,8 @@ struct PrefillPlan {
 struct PrefillArgs {
     void* out;
     const PrefillItem* items;
+    const float2* rope_table; // ROPE_Q: [64 pairs][rope_pitch positions] x (cos, sin)
+    uint32_t rope_pitch;
     uint32_t num_qo_heads, num_kv_heads;
     int causal;
     float sm_scale_log2;
@@ -119,11 +126,14 @@ __device__ __forceinline__ uint32_t& pf_u4(uint4& v, int i) { return reinterpret
 // MFMAs), used for bf16 whose 8-bit significand alone would eat the error budget.
 // XOR applied to the 16-byte chunk index of V rows in LDS, by row % 4: 0, 4, 10, 14 (see the staging comment)
 #define BZ_VSWZ(r) (((r) << 2) ^ (((r) >> 1) << 1))
-template <bool BF16, bool SPLIT_P>
+// ROPE_Q: the q rows are rotated in registers on their way in (position = offset inside the request, angles
+// from a table), so q is read once and never written; k is expected rotated.
+template <bool BF16, bool SPLIT_P, bool ROPE_Q>
 __global__ __launch_bounds__(256, 2) void prefill_kernel(PrefillArgs a, const char* __restrict__ q_ptr,
                                                          const char* __restrict__ k_ptr,
                                                          const char* __restrict__ v_ptr) {
     using M = PfMma<BF16>;
+    constexpr bool QSCALED = !BF16 || ROPE_Q; // q carries sm_scale * log2(e) (see the prologue)
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
 
     const PrefillItem it = a.items[blockIdx.x];
@@ -145,12 +155,50 @@ __global__ __launch_bounds__(256, 2) void prefill_kernel(PrefillArgs a, const ch
         const char* qrow = q_ptr + (qtok * Hq + head) * 256;
 #pragma unroll
         for (int ks = 0; ks < 8; ++ks) qreg[ks] = *reinterpret_cast<const uint4*>(qrow + ks * 32 + h * 16);
+        if constexpr (ROPE_Q) {
+            // d = 16 ks + 8 h + e (ks < 4) pairs with d + 64, which this lane holds at step ks + 4.  The table is
+            // laid out pair by pair, so the 32 rows of a half-wave read 256 consecutive bytes per pair.
+            const float2* tab = a.rope_table + min(q_pos, L - 1);
+            float2 cs[32];
+#pragma unroll
+            for (int e = 0; e < 32; ++e) cs[e] = tab[(size_t)(16 * (e >> 3) + 8 * h + (e & 7)) * a.rope_pitch];
+#pragma unroll
+            for (int ks = 0; ks < 4; ++ks)
+#pragma unroll
+                for (int w = 0; w < 4; ++w) {
+                    const float2 c0 = cs[8 * ks + 2 * w], c1 = cs[8 * ks + 2 * w + 1]; // pairs i = 16 ks + 8 h + 2 w, i + 1
+                    const uint32_t xw = pf_u4(qreg[ks], w), yw = pf_u4(qreg[ks + 4], w);
+                    float x0, y0, x1, y1;
+                    rope_pair(M::lo(xw), M::lo(yw), c0.x, c0.y, x0, y0);
+                    rope_pair(M::hi(xw), M::hi(yw), c1.x, c1.y, x1, y1);
+                    // (the softmax scale rides on the one rounding of the rotated row, see below)
+                    pf_u4(qreg[ks], w) = M::pack2(x0 * a.sm_scale_log2, x1 * a.sm_scale_log2);
+                    pf_u4(qreg[ks + 4], w) = M::pack2(y0 * a.sm_scale_log2, y1 * a.sm_scale_log2);
+                }
+        } else if constexpr (QSCALED) {
+            // The q rows carry the softmax scale (times log2 e): the scores then come out of the matrix pipe as
+            // base-2 logits and go into exp2 as they are, one vector instruction less per score.  (Not for
+            // bf16 rows that arrive rotated: a second rounding to 8 significant bits would cost a factor of
+            // two in the error of every logit; there the scale is applied to the score instead.)
+#pragma unroll
+            for (int ks = 0; ks < 8; ++ks)
+#pragma unroll
+                for (int w = 0; w < 4; ++w) {
+                    const uint32_t xw = pf_u4(qreg[ks], w);
+                    pf_u4(qreg[ks], w) = M::pack2(M::lo(xw) * a.sm_scale_log2, M::hi(xw) * a.sm_scale_log2);
+                }
+        }
     }
 
     const int kv_limit = a.causal ? min(L, it.q0 + kBM) : L; // tokens any row of this workgroup can see
     const int n_tiles = (kv_limit + kBN - 1) / kBN;
-    // tiles this wave computes: under the causal mask its rows see nothing past token wave_q_hi
-    const int n_w = a.causal ? min(n_tiles, wave_q_hi / kBN + 1) : n_tiles;
+    // tiles this wave computes: under the causal mask its rows see nothing past token wave_q_hi; a wave whose
+    // rows all lie past the end of the request (last q tile of a request) computes nothing at all, it only
+    // takes part in the copies and barriers
+    const int n_w = wave_q_lo >= L ? 0 : (a.causal ? min(n_tiles, wave_q_hi / kBN + 1) : n_tiles);
+    // the last tile of a wave whose rows start on a tile boundary (causal): its second 32 tokens lie past
+    // every row of the wave, so only the first block is computed
+    const int t_half = (a.causal && (wave_q_lo % kBN) == 0) ? wave_q_lo / kBN : -1;
 
     // ---- global -> LDS staging of a K/V tile with LDS-direct loads (no registers, no LDS stores): a
     // wave instruction moves 64 x 16 B to 1 KiB of consecutive LDS, i.e. 4 unpadded 256-byte rows; wave w
@@ -200,7 +248,19 @@ __global__ __launch_bounds__(256, 2) void prefill_kernel(PrefillArgs a, const ch
         __syncthreads();
     };
 
-    float m_run = -INFINITY, l_run = 0.f;
+    // Online softmax without a maximum per tile.  The scores leave the matrix pipe already shifted by the
+    // reference maximum m_run of their row: the first score step of a block accumulates onto `cinit`, a block
+    // of registers that holds -m_run, so p = exp2(score) needs no further arithmetic.  m_run is set from the
+    // first tile (in the units of the scores: base-2 logits when q carries the scale) and moved only when it has to be: a tile's probabilities are computed on the assumption that
+    // no score exceeds m_run by 15 or more (p < 2^15 fits the 16-bit operand of the second contraction, and
+    // fp32 sums hold it easily); the row sums, which are needed anyway, tell whether the assumption held
+    // (every p < 2^15 if their sum is), and a wave for which it did not takes the tile's maximum, moves m_run,
+    // rescales its accumulators and computes the tile's probabilities again.  m_run never exceeds the true
+    // running maximum, so the largest probability of a row so far is always at least 1.
+    float m_run = 0.f, l_run = 0.f;
+    pf_f32x16 cinit;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) cinit[i] = 0.f;
     pf_f32x16 acc[4]; // O^T: block db covers d = 32*db .. +31; element 4b+r is d = 32*db + 8b + 4h + r
 #pragma unroll
     for (int db = 0; db < 4; ++db)
@@ -233,10 +293,13 @@ __global__ __launch_bounds__(256, 2) void prefill_kernel(PrefillArgs a, const ch
 
     // the arithmetic of tile t (K/V in LDS buffer BUF = t % 2, a compile-time constant so that the buffer
     // and step offsets fold into the immediate field of the LDS reads)
-    auto compute_tile = [&](int t, auto which) __attribute__((always_inline)) {
+    auto compute_tile = [&](int t, auto which, auto half_c) __attribute__((always_inline)) {
         constexpr int BUF = decltype(which)::value;
+        constexpr bool HALF = decltype(half_c)::value; // only the first 32 tokens of the tile (see t_half)
+        constexpr int NS = HALF ? 8 : 16;              // score steps, and steps of the second contraction
+        constexpr int NKB = HALF ? 1 : 2;              // 32-token blocks
         const int kv0 = t * kBN;
-        if (t < n_w) {
+        {
             // Both contractions are scheduled by hand.  An LDS read takes several times as long as a
             // matrix instruction, so the operand reads run kDK / kDV matrix instructions ahead of their
             // use (rings ka / va); scheduling barriers keep the steps in this order.
@@ -266,93 +329,97 @@ __global__ __launch_bounds__(256, 2) void prefill_kernel(PrefillArgs a, const ch
             for (int i = 0; i < kDK; ++i) ka[i] = k_read(i);
             __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-            for (int i = 0; i < 16; ++i) {
+            for (int i = 0; i < NS; ++i) {
                 if ((i & 7) == 0) {
-                    pf_f32x16 zero;
-#pragma unroll
-                    for (int e = 0; e < 16; ++e) zero[e] = 0.f;
-                    s[i >> 3] = M::run(ka[i % kDK], qreg[i & 7], zero);
+                    s[i >> 3] = M::run(ka[i % kDK], qreg[i & 7], cinit);
                 } else {
                     s[i >> 3] = M::run(ka[i % kDK], qreg[i & 7], s[i >> 3]);
                 }
-                if (i + kDK < 16) ka[i % kDK] = k_read(i + kDK);
-                else va[i + kDK - 16] = v_read(i + kDK - 16); // the first V operands arrive during the softmax
+                if (i + kDK < NS) ka[i % kDK] = k_read(i + kDK);
+                else va[i + kDK - NS] = v_read(i + kDK - NS); // the first V operands arrive during the softmax
                 __builtin_amdgcn_sched_barrier(0);
             }
             static_assert(kDV == kDK, "the tail of the score steps fills the whole V ring");
-            // ---- mask, maximum.  Element 4b+r of block kb is token kv0 + 32kb + 8b + 4h + r.
-            const bool need_mask = (a.causal && kv0 + kBN - 1 > wave_q_lo) || (kv0 + kBN > L);
-            float tmax = -INFINITY;
+            // ---- mask.  Element 4b+r of block kb is token kv0 + 32kb + 8b + 4h + r.
+            const bool need_mask = HALF || (a.causal && kv0 + kBN - 1 > wave_q_lo) || (kv0 + kBN > L);
             if (need_mask) { // wave-uniform; selects, not branches, per element
                 const int kv_max = a.causal ? min(q_pos, L - 1) : L - 1; // last token this row may see
 #pragma unroll
-                for (int kb = 0; kb < 2; ++kb)
+                for (int kb = 0; kb < NKB; ++kb)
 #pragma unroll
                     for (int i = 0; i < 16; ++i) {
                         const int kv = kv0 + 32 * kb + 8 * (i >> 2) + 4 * h + (i & 3);
-                        const float v = kv > kv_max ? -INFINITY : s[kb][i];
-                        s[kb][i] = v;
-                        tmax = fmaxf(tmax, v);
+                        s[kb][i] = kv > kv_max ? -INFINITY : s[kb][i];
                     }
-            } else {
+            }
+            float psum;
+            uint4 pa[4], pb[4]; // P^T operands of the four 16-token steps (head, and tail when SPLIT_P)
+            auto probabilities = [&](float shift) __attribute__((always_inline)) { // p = exp2(score - shift)
+                psum = 0.f;
 #pragma unroll
-                for (int kb = 0; kb < 2; ++kb)
+                for (int st = 0; st < 2 * NKB; ++st) {
+                    const int kb = st >> 1, b0 = 2 * (st & 1);
+#pragma unroll
+                    for (int w = 0; w < 4; ++w) { // elements e = 2w, 2w+1 of the operand: block b0 + e/4, r = e%4
+                        const int i0 = 4 * (b0 + (w >> 1)) + 2 * (w & 1);
+                        const float p0 = __builtin_amdgcn_exp2f(QSCALED ? s[kb][i0] - shift : (s[kb][i0] - shift) * a.sm_scale_log2);
+                        const float p1 = __builtin_amdgcn_exp2f(QSCALED ? s[kb][i0 + 1] - shift : (s[kb][i0 + 1] - shift) * a.sm_scale_log2);
+                        psum += p0 + p1;
+                        const uint32_t hw = M::pack2(p0, p1);
+                        pf_u4(pa[st], w) = hw;
+                        if (SPLIT_P) pf_u4(pb[st], w) = M::pack2(p0 - M::lo(hw), p1 - M::hi(hw));
+                    }
+                }
+            };
+            bool moved = t == 0; // the first tile sets the reference maximum (token 0 is visible to every row)
+            if (!moved) {
+                probabilities(0.f);
+                moved = __any(!(psum < 32768.0f)); // some score is 15 or more above m_run (or the sum is not finite)
+            }
+            if (moved) { // wave-uniform, rare after the first tile
+                float tmax = -INFINITY;
+#pragma unroll
+                for (int kb = 0; kb < NKB; ++kb)
 #pragma unroll
                     for (int i = 0; i < 16; ++i) tmax = fmaxf(tmax, s[kb][i]);
-            }
-            // the scores stay unscaled in registers: the (positive) softmax scale is applied to the maximum
-            // here and to every score inside the fused multiply-add that feeds exp2
-            tmax = lane_max_xor32(tmax) * a.sm_scale_log2;
-            // The reference maximum only moves when some row's maximum has grown by more than 2^8 since
-            // it was last set (wave-uniform decision): until then exp2(s - m_run) is at most 256, which
-            // fp32 sums and 16-bit operands hold without loss, and the accumulators need no rescaling.
-            // Token 0 is visible to every row, so the first tile always sets a finite maximum.
-            if (__any(tmax > m_run + 8.0f)) {
-                const float m_new = fmaxf(m_run, tmax);
-                const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
-                m_run = m_new;
+                tmax = lane_max_xor32(tmax); // relative to the present m_run; -inf for a row that sees nothing here
+                const float shift = t == 0 ? tmax : fmaxf(tmax, 0.f);
+                const float alpha = __builtin_amdgcn_exp2f(QSCALED ? -shift : -shift * a.sm_scale_log2);
+                m_run += shift;
                 l_run *= alpha;
 #pragma unroll
                 for (int db = 0; db < 4; ++db)
 #pragma unroll
                     for (int i = 0; i < 16; ++i) acc[db][i] *= alpha;
-            }
-            float psum = 0.f;
-            uint4 pa[4], pb[4]; // P^T operands of the four 16-token steps (head, and tail when SPLIT_P)
 #pragma unroll
-            for (int st = 0; st < 4; ++st) {
-                const int kb = st >> 1, b0 = 2 * (st & 1);
-#pragma unroll
-                for (int w = 0; w < 4; ++w) { // elements e = 2w, 2w+1 of the operand: block b0 + e/4, r = e%4
-                    const int i0 = 4 * (b0 + (w >> 1)) + 2 * (w & 1);
-                    const float p0 = __builtin_amdgcn_exp2f(fmaf(s[kb][i0], a.sm_scale_log2, -m_run));
-                    const float p1 = __builtin_amdgcn_exp2f(fmaf(s[kb][i0 + 1], a.sm_scale_log2, -m_run));
-                    psum += p0 + p1;
-                    const uint32_t hw = M::pack2(p0, p1);
-                    pf_u4(pa[st], w) = hw;
-                    if (SPLIT_P) pf_u4(pb[st], w) = M::pack2(p0 - M::lo(hw), p1 - M::hi(hw));
-                }
+                for (int i = 0; i < 16; ++i) cinit[i] = -m_run;
+                probabilities(shift);
             }
             psum = lane_sum_xor32(psum);
             l_run += psum;
             __builtin_amdgcn_sched_barrier(0);
             // ---- O^T += V^T P^T: step i takes tokens 16*(i/4) .. +15 and d block i%4
 #pragma unroll
-            for (int i = 0; i < 16; ++i) {
+            for (int i = 0; i < NS; ++i) {
                 acc[i & 3] = M::run(va[i % kDV], pa[i >> 2], acc[i & 3]);
                 if (SPLIT_P) acc[i & 3] = M::run(va[i % kDV], pb[i >> 2], acc[i & 3]);
-                if (i + kDV < 16) va[i % kDV] = v_read(i + kDV);
+                if (i + kDV < NS) va[i % kDV] = v_read(i + kDV);
                 __builtin_amdgcn_sched_barrier(0);
             }
         }
     };
+    auto tile = [&](int t, auto which) __attribute__((always_inline)) {
+        if (t >= n_w) return;
+        if (t == t_half) compute_tile(t, which, std::true_type{});
+        else compute_tile(t, which, std::false_type{});
+    };
     for (int t = 0; t < n_tiles; t += 2) {
         if (t + 1 < n_tiles) issue_tile(t + 1, 1); // buffer 1 was last read before the previous barrier
-        compute_tile(t, std::integral_constant<int, 0>{});
+        tile(t, std::integral_constant<int, 0>{});
         publish();
         if (t + 1 < n_tiles) {
             if (t + 2 < n_tiles) issue_tile(t + 2, 0);
-            compute_tile(t + 1, std::integral_constant<int, 1>{});
+            tile(t + 1, std::integral_constant<int, 1>{});
             publish();
         }
     }
@@ -417,11 +484,11 @@ __global__ __launch_bounds__(256) void rope_ragged_kernel(RopeRaggedArgs a) {
     }
     __syncthreads();
     const int lane8 = threadIdx.x & 7; // 8 lanes per row: 8 low-half and the 8 matching high-half elements each
-    const int rows = (int)(a.num_qo_heads + a.num_kv_heads);
+    const int nq = a.q ? (int)a.num_qo_heads : 0, nk = a.k ? (int)a.num_kv_heads : 0; // either may be left alone
+    const int rows = nq + nk;
     for (int r = threadIdx.x >> 3; r < rows; r += 32) {
-        T* row = (r < (int)a.num_qo_heads)
-                     ? reinterpret_cast<T*>(a.q) + ((size_t)tok * a.num_qo_heads + r) * 128
-                     : reinterpret_cast<T*>(a.k) + ((size_t)tok * a.num_kv_heads + (r - a.num_qo_heads)) * 128;
+        T* row = (r < nq) ? reinterpret_cast<T*>(a.q) + ((size_t)tok * a.num_qo_heads + r) * 128
+                          : reinterpret_cast<T*>(a.k) + ((size_t)tok * a.num_kv_heads + (r - nq)) * 128;
         Vec8<T> lo, hi;
         lo.load(row + lane8 * 8);
         hi.load(row + 64 + lane8 * 8);
@@ -441,6 +508,15 @@ __global__ __launch_bounds__(256) void rope_ragged_kernel(RopeRaggedArgs a) {
         lo.store(row + lane8 * 8);
         hi.store(row + 64 + lane8 * 8);
     }
+}
+
+// cos / sin table for the q rotation inside the attention kernel, pair by pair: table[i][pos]
+__global__ __launch_bounds__(256) void rope_table_kernel(float2* table, uint32_t positions, uint32_t pitch, RopeFreqs freqs) {
+    const uint32_t pos = blockIdx.x * 256 + threadIdx.x, i = blockIdx.y;
+    if (pos >= positions) return;
+    float s, c;
+    sincosf((float)pos * freqs.f[i], &s, &c);
+    table[(size_t)i * pitch + pos] = make_float2(c, s);
 }
 
 static inline size_t pf_align_up(size_t x, size_t a) { return (x + a - 1) / a * a; }
@@ -523,7 +599,11 @@ extern "C" int bz_prefill_plan_workspace(bz_prefill_plan_t* plan_, const int32_t
     PrefillPlan* p = reinterpret_cast<PrefillPlan*>(plan_);
     const int rc = build_prefill_items(p, qo_indptr_h, kv_indptr_h, batch_size, num_qo_heads, num_kv_heads, head_dim);
     if (rc) return rc;
-    if (float_buffer_bytes) *float_buffer_bytes = 0;
+    if (float_buffer_bytes) { // the angle table of the q rotation: 512 bytes per position of the longest request
+        int32_t longest = 0;
+        for (uint32_t b = 0; b < batch_size; ++b) longest = std::max(longest, qo_indptr_h[b + 1] - qo_indptr_h[b]);
+        *float_buffer_bytes = (size_t)longest * 512;
+    }
     if (int_buffer_bytes) *int_buffer_bytes = pf_align_up(p->h_items.size() * sizeof(PrefillItem), 256);
     return 0;
 }
@@ -542,7 +622,7 @@ extern "C" int bz_prefill_plan(bz_prefill_plan_t* plan_, void* float_buffer, siz
                                void* int_buffer, size_t int_buffer_bytes, const int32_t* qo_indptr_h,
                                const int32_t* kv_indptr_h, uint32_t batch_size, uint32_t num_qo_heads,
                                uint32_t num_kv_heads, uint32_t head_dim, uint32_t page_size, void* stream) {
-    (void)float_buffer; (void)float_buffer_bytes; (void)page_size;
+    (void)page_size;
     PrefillPlan* p = reinterpret_cast<PrefillPlan*>(plan_);
     if (!p || !int_buffer) return BZ_ERR_BAD_ARG;
     const int rc0 = build_prefill_items(p, qo_indptr_h, kv_indptr_h, batch_size, num_qo_heads, num_kv_heads, head_dim);
@@ -572,15 +652,22 @@ extern "C" int bz_prefill_plan(bz_prefill_plan_t* plan_, void* float_buffer, siz
     p->batch_size = batch_size; p->num_qo_heads = num_qo_heads; p->num_kv_heads = num_kv_heads;
     p->head_dim = head_dim;
     p->total_tokens = (uint32_t)qo_indptr_h[batch_size];
+    p->max_len = 0;
+    for (uint32_t b = 0; b < batch_size; ++b)
+        p->max_len = std::max<uint32_t>(p->max_len, (uint32_t)(qo_indptr_h[b + 1] - qo_indptr_h[b]));
+    // the float workspace holds the angle table of the q rotation when it has room for it (512 bytes per position)
+    p->rope_table = (float_buffer && (size_t)p->max_len * 512 <= float_buffer_bytes && (uintptr_t)float_buffer % 16 == 0)
+                        ? (float*)float_buffer : nullptr;
+    p->rope_table_valid = false;
     p->planned = true;
     return 0;
 }
 
-template <bool BF16, bool SPLIT_P>
+template <bool BF16, bool SPLIT_P, bool ROPE_Q>
 static int launch_prefill(const PrefillPlan* p, const PrefillArgs& a, const void* q, const void* k, const void* v,
                           hipStream_t s) {
     const size_t smem = 4 * (size_t)kTile;
-    auto kern = prefill_kernel<BF16, SPLIT_P>;
+    auto kern = prefill_kernel<BF16, SPLIT_P, ROPE_Q>;
     // raising the dynamic LDS limit: once per device (idempotent, so a race between two host threads is harmless)
     static std::atomic<uint64_t> attr_done{0};
     int dev = 0;
@@ -607,26 +694,49 @@ extern "C" int bz_batch_prefill_ragged(bz_prefill_plan_t* plan_, void* q, const 
         head_dim != p->head_dim)
         return BZ_ERR_BAD_ARG;
     if (dtype != BZ_F16 && dtype != BZ_BF16) return BZ_ERR_UNSUPPORTED;
-    if (rope_mode != BZ_ROPE_NONE && rope_mode != BZ_ROPE_FULL) return BZ_ERR_BAD_ARG;
+    if (rope_mode < BZ_ROPE_NONE || rope_mode > BZ_ROPE_FULL) return BZ_ERR_BAD_ARG;
     if (((uintptr_t)q | (uintptr_t)k | (uintptr_t)v | (uintptr_t)out) % 16) return BZ_ERR_BAD_ARG;
     hipStream_t s = (hipStream_t)stream;
     if (p->num_items == 0) return 0;
-    if (rope_mode == BZ_ROPE_FULL) {
+    // q is rotated in registers inside the attention kernel (angles from a table in the float workspace) and
+    // stays as it is in memory; k, which every q tile of a request reads, is rotated once, in place, first.
+    bool rope_q = rope_mode != BZ_ROPE_NONE;
+    if (rope_mode != BZ_ROPE_NONE) {
+        const float theta = rope_theta > 0.f ? rope_theta : 1e4f;
+        const RopeFreqs freqs = make_rope_freqs(128, theta);
+        if (p->rope_table && (!p->rope_table_valid || p->rope_table_theta != theta)) {
+            hipLaunchKernelGGL(rope_table_kernel, dim3((p->max_len + 255) / 256, 64), dim3(256), 0, s, (float2*)p->rope_table,
+                               p->max_len, p->max_len, freqs);
+            BZ_LAUNCH_CHECK();
+            p->rope_table_theta = theta;
+            p->rope_table_valid = true;
+        }
         RopeRaggedArgs ra;
-        ra.q = q; ra.k = k; ra.indptr = qo_indptr;
+        ra.q = p->rope_table ? nullptr : q; // no room for the table: q is rotated in place instead
+        ra.k = rope_mode == BZ_ROPE_FULL ? k : nullptr;
+        ra.indptr = qo_indptr;
         ra.batch_size = batch_size; ra.num_qo_heads = num_qo_heads; ra.num_kv_heads = num_kv_heads;
-        ra.freqs = make_rope_freqs(128, rope_theta > 0.f ? rope_theta : 1e4f);
-        if (dtype == BZ_F16) hipLaunchKernelGGL((rope_ragged_kernel<f16_t>), dim3(p->total_tokens), dim3(256), 0, s, ra);
-        else hipLaunchKernelGGL((rope_ragged_kernel<bf16_t>), dim3(p->total_tokens), dim3(256), 0, s, ra);
-        BZ_LAUNCH_CHECK();
+        ra.freqs = freqs;
+        if (ra.q || ra.k) {
+            if (dtype == BZ_F16) hipLaunchKernelGGL((rope_ragged_kernel<f16_t>), dim3(p->total_tokens), dim3(256), 0, s, ra);
+            else hipLaunchKernelGGL((rope_ragged_kernel<bf16_t>), dim3(p->total_tokens), dim3(256), 0, s, ra);
+            BZ_LAUNCH_CHECK();
+        }
+        rope_q = p->rope_table != nullptr;
     }
     PrefillArgs a;
     a.out = out;
     a.items = p->items_d;
+    a.rope_table = (const float2*)p->rope_table;
+    a.rope_pitch = p->max_len;
     a.num_qo_heads = num_qo_heads; a.num_kv_heads = num_kv_heads;
     a.causal = causal ? 1 : 0;
     if (!(sm_scale > 0.f)) sm_scale = 1.0f / sqrtf((float)head_dim);
     a.sm_scale_log2 = sm_scale * 1.4426950408889634f;
-    if (dtype == BZ_F16) return launch_prefill<false, false>(p, a, q, k, v, s);
-    return launch_prefill<true, true>(p, a, q, k, v, s);
+    if (rope_q) {
+        if (dtype == BZ_F16) return launch_prefill<false, false, true>(p, a, q, k, v, s);
+        return launch_prefill<true, true, true>(p, a, q, k, v, s);
+    }
+    if (dtype == BZ_F16) return launch_prefill<false, false, false>(p, a, q, k, v, s);
+    return launch_prefill<true, true, false>(p, a, q, k, v, s);
 }

@@ -219,9 +219,13 @@ int bz_prefill_plan_host_schedule(const bz_prefill_plan_t* plan, const int32_t**
  * batch_prefill_attention (src/kernel/attention.h:9-22, attention_prefill.cu:11-46): ragged
  * self-attention, q [N,Hq,D], k,v [N,Hkv,D], out [N,Hq,D], qo_indptr == kv_indptr (the only
  * way the reference calls it, src/layer/attn.h:175-187).  causal != 0 masks j > i.
- * rope_mode BZ_ROPE_NONE: q,k used as they are (rotate them first with bz_rope_store_prefill_kv);
- * BZ_ROPE_FULL: q and k rows are rotated IN PLACE by their offset inside the request before the
- * contraction (the caller's k buffer then holds rotated K for the page store that follows).
+ * rope_mode BZ_ROPE_NONE: q, k used as they are.  BZ_ROPE_Q_ONLY: q rows are rotated by their offset inside
+ * the request in registers (q in memory stays as it is), k is expected rotated (bz_store_prefill_kv with
+ * rope = 2 leaves it so).  BZ_ROPE_FULL, the reference's kRoPELlama: q as for BZ_ROPE_Q_ONLY, and the k rows
+ * are rotated IN PLACE first (the caller's k buffer then holds rotated K for the page store that follows,
+ * which must not rotate it again).  The angle table of the q rotation lives in the float workspace given to
+ * bz_prefill_plan (512 bytes per position of the longest request; bz_prefill_plan_workspace reports it);
+ * without room for it q is rotated in place by a separate launch instead.
  */
 int bz_batch_prefill_ragged(bz_prefill_plan_t* plan, void* q, const int32_t* qo_indptr, void* k, void* v,
                             const int32_t* kv_indptr, void* out, int dtype, uint32_t batch_size,
@@ -233,9 +237,11 @@ int bz_batch_prefill_ragged(bz_prefill_plan_t* plan, void* q, const int32_t* qo_
  * ------------------------------------------------------------------------------------- */
 /* store_prefill_kv_cache (src/kernel/page.h:66-67, page.cu:21-94): token t of request b goes to
  * page indices[indptr[b]+t/P], slot t%P.  k, v: [N, Hkv, D] of src_dtype.
- * rope != 0 rotates K at position t on the way in.  With q_inout (optional, [N, Hq, D],
- * num_qo_heads) given as well, q AND the caller's k rows are rotated in place by the same angles:
- * the fused RoPE of the prefill path, after which bz_batch_prefill_ragged runs with BZ_ROPE_NONE.
+ * rope != 0 rotates K at position t on the way in.  rope == 2 also rotates the caller's k rows in place
+ * (q is then left to bz_batch_prefill_ragged with BZ_ROPE_Q_ONLY, which rotates it in registers: the
+ * fused RoPE of the prefill path).  With q_inout (optional, [N, Hq, D], num_qo_heads) given, q AND the
+ * caller's k rows are rotated in place by the same angles, after which bz_batch_prefill_ragged runs
+ * with BZ_ROPE_NONE.
  * k_scale / v_scale: device fp32 [Hkv]; for an e4m3 pool the value stored is quant(x / scale).
  * num_tokens: N, or BZ_NUM_TOKENS_FROM_INDPTR when the host does not know it (the reference's call has no
  * such argument and shapes its launch from page size and batch, page.cu:84-89).  Tokens of a request beyond

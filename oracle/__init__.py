@@ -152,7 +152,8 @@ def batch_decode(q_bits, q_dtype, kv, num_qo_heads, rope_mode=ROPE_NONE, rope_th
 
 def batch_prefill_ragged(q_bits, k_bits, v_bits, dtype, indptr, Hq, Hkv, D, causal=True, rope=False,
                          rope_theta=1e4, sm_scale=None, rows=None, parallel=False):
-    """fp32 [N or len(rows), Hq, D]."""
+    """fp32 [N or len(rows), Hq, D].  rope: False / True rotate neither / both of q and k at their offsets inside
+    the request (in fp32, nothing is rounded); "q" rotates q only (k rows hold rotated K already)."""
     q_bits, k_bits, v_bits = (_c(a, storage_np(dtype)) for a in (q_bits, k_bits, v_bits))
     indptr = _c(indptr, np.int32)
     B = len(indptr) - 1
@@ -162,7 +163,8 @@ def batch_prefill_ragged(q_bits, k_bits, v_bits, dtype, indptr, Hq, Hkv, D, caus
     n = int(indptr[-1]) if rows is None else len(rows)
     out = np.empty((n, Hq, D), np.float32)
     lib(parallel).bzo_batch_prefill_ragged(_p(q_bits), _p(k_bits), _p(v_bits), dtype, _p(indptr), B, Hq, Hkv, D,
-                                           int(causal), int(rope), C.c_float(rope_theta), C.c_float(sm_scale),
+                                           int(causal), 2 if rope == "q" else int(bool(rope)), C.c_float(rope_theta),
+                                           C.c_float(sm_scale),
                                            _p(rows), 0 if rows is None else len(rows), _p(out))
     return out
 

@@ -311,7 +311,7 @@ void bzo_batch_prefill_ragged(const void* q, const void* k, const void* v, int d
             float m = -INFINITY;
             for (int j = beg; j < end; ++j) {
                 for (int d = 0; d < D; ++d) kr[d] = load_as_f32(k, dtype, ((size_t)j * Hkv + kvh) * D + d);
-                if (rope) bzo_rope_llama(kr, D, j - beg, rope_theta);
+                if (rope == 1) bzo_rope_llama(kr, D, j - beg, rope_theta); /* rope == 2: k rows are rotated already */
                 float acc = 0.0f;
                 for (int d = 0; d < D; ++d) acc += qv[d] * kr[d];
                 s[j - beg] = acc * sm_scale;

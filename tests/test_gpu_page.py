@@ -174,3 +174,31 @@ def test_store_prefill_drops_tokens_beyond_the_listed_pages():
     K.store_prefill_kv_cache(dev.pt, to_dev(k, dtype), to_dev(v, dtype), to_dev(ri.view(np.float32), 3).view(torch.int32))
     torch.cuda.synchronize()
     assert np.array_equal(to_host_bits(dev.pool), want)
+
+
+def test_store_prefill_rotates_k_in_place_without_q():
+    """rope = 2: K is rotated into the pages AND in the caller's rows (q is left to the attention call, which
+    rotates it in registers); same bits in both places."""
+    rng = np.random.default_rng(64)
+    lens, Hkv, D, P, dtype, theta = [3, 64, 130], 4, 128, 16, BZ_F16, 1e4
+    p, fill = _setup(65, lens, 8, Hkv, D, P, dtype, BZ_LAYOUT_HND)
+    ri = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+    k, v = wl.randn_bits(rng, (ri[-1], Hkv, D), dtype), wl.randn_bits(rng, (ri[-1], Hkv, D), dtype)
+    want = p.pool.copy()
+    oracle.store_prefill_kv(p.oracle_kv(want), k, v, dtype, ri, rope=True, rope_theta=theta)
+    want_k = oracle.rope_ragged(k, dtype, ri, Hkv, D, theta)
+    dev = DeviceDecode(p)
+    kd, vd = to_dev(k, dtype), to_dev(v, dtype)
+    K.store_prefill_kv_cache(dev.pt, kd, vd, to_dev(ri.view(np.float32), 3).view(torch.int32), rope=2, rope_theta=theta)
+    torch.cuda.synchronize()
+    got_pool, got_k = to_host_bits(dev.pool), to_host_bits(kd)
+    for g, w in ((got_pool, want), (got_k, want_k)):
+        assert np.abs(wl.to_f32(g, dtype) - wl.to_f32(w, dtype)).max() <= 2.0 ** -8
+        assert (g != w).mean() < 2e-3
+    assert np.array_equal(to_host_bits(vd), v)
+    # the caller's rows and the cached rows are the same bits
+    kv = p.oracle_kv(got_pool)
+    K0, _ = DecodeProblem.gather_kv.__get__(type("X", (), dict(ctx=np.array(lens), pool=got_pool, kv_dtype=dtype, P=P, Hkv=Hkv, D=D,
+                                                               indices=p.indices, indptr=p.indptr, stride_page=p.stride_page,
+                                                               stride_n=p.stride_n, stride_h=p.stride_h))())(2)
+    assert np.array_equal(K0, wl.to_f32(got_k, dtype).reshape(-1, Hkv, D)[ri[2]:ri[3]])

@@ -7,7 +7,7 @@ import torch
 import oracle
 from blitz_scale_amd import kernel as K
 from blitz_scale_amd import workloads as wl
-from blitz_scale_amd._lib import BZ_BF16, BZ_F16, BZ_LAYOUT_HND, BZ_ROPE_FULL, BZ_ROPE_NONE
+from blitz_scale_amd._lib import BZ_BF16, BZ_F16, BZ_LAYOUT_HND, BZ_ROPE_FULL, BZ_ROPE_NONE, BZ_ROPE_Q_ONLY
 
 from _gpu import DeviceDecode, to_dev, to_host_bits
 from _util import DecodeProblem, ulp_tol
@@ -55,18 +55,52 @@ def test_small_ragged_full_check(dtype, causal, Hq, Hkv):
         assert np.abs(got - ref).max() <= 2e-3
 
 
-def test_rope_inside_the_call_rotates_q_and_k_in_place():
-    theta, dtype = 1e4, BZ_F16
-    pf = Prefill(210, [5, 200, 131], 8, 4, 128, dtype)
+@pytest.mark.parametrize("dtype", [BZ_F16, BZ_BF16])
+@pytest.mark.parametrize("float_ws_bytes", [1 << 20, 1 << 10])
+def test_rope_inside_the_call(dtype, float_ws_bytes):
+    """BZ_ROPE_FULL, the reference's kRoPELlama: k rows are rotated in place (the page store that follows
+    copies them), q is rotated in registers from the angle table in the float workspace and stays untouched in
+    memory -- unless the workspace has no room for the table (second case), then q is rotated in place too.
+    BZ_ROPE_Q_ONLY on the rotated k gives the same output and touches nothing."""
+    theta = 1e4
+    pf = Prefill(210, [5, 200, 131, 1, 64], 8, 4, 128, dtype)
+    pf.float_ws = torch.empty(float_ws_bytes, dtype=torch.uint8, device="cuda")
     got = pf.run(causal=True, rope_mode=BZ_ROPE_FULL, theta=theta)
     q_rot = oracle.rope_ragged(pf.q, dtype, pf.indptr, 8, 128, theta)
     k_rot = oracle.rope_ragged(pf.k, dtype, pf.indptr, 4, 128, theta)
-    for g, w in ((pf.q_after, q_rot), (pf.k_after, k_rot)):
-        assert np.abs(wl.to_f32(g, dtype) - wl.to_f32(w, dtype)).max() <= 2.0 ** -8
-        assert (g != w).mean() < 2e-3
-    # attention over exactly the bits the device left behind
-    ref = oracle.batch_prefill_ragged(pf.q_after, pf.k_after, pf.v, dtype, pf.indptr, 8, 4, 128, causal=True, parallel=True)
-    assert np.abs(got - ref).max() <= 2e-3
+    step = 2.0 ** -8 if dtype == BZ_F16 else 2.0 ** -5
+    assert np.abs(wl.to_f32(pf.k_after, dtype) - wl.to_f32(k_rot, dtype)).max() <= step
+    assert (pf.k_after != k_rot).mean() < 2e-3
+    if float_ws_bytes >= 200 * 512:
+        assert np.array_equal(pf.q_after, pf.q)  # q is read only
+    else:
+        assert np.abs(wl.to_f32(pf.q_after, dtype) - wl.to_f32(q_rot, dtype)).max() <= step
+        assert (pf.q_after != q_rot).mean() < 2e-3
+    if float_ws_bytes >= 200 * 512:
+        # q rotated in registers (fp32, rounded once together with the softmax scale): the checker rotates q in
+        # fp32 as well and reads the k bits the device left behind
+        ref = oracle.batch_prefill_ragged(pf.q, pf.k_after, pf.v, dtype, pf.indptr, 8, 4, 128, causal=True, rope="q",
+                                          rope_theta=theta, parallel=True)
+        # (for bf16 the one rounding of the rotated, scaled q row to 8 significant bits moves the logits by up
+        # to ~1e-2; the same holds for any kernel that feeds bf16 operands to the matrix cores)
+        assert np.abs(got - ref).max() <= (2e-3 if dtype == BZ_F16 else 2e-2), np.abs(got - ref).max()
+    else:
+        # attention over the rotated rows as the device left them in memory
+        ref = oracle.batch_prefill_ragged(pf.q_after, pf.k_after, pf.v, dtype, pf.indptr, 8, 4, 128, causal=True, parallel=True)
+        assert (np.abs(got - ref) <= ulp_tol(ref, dtype)).all(), np.abs(got - ref).max()
+    # and against kRoPELlama on the raw rows (rotation in fp32, no rounding of q and k).  For f16 the same bar;
+    # for bf16 the rounding of the rotated rows to 8 significant bits alone moves the logits by ~1e-2, which is
+    # why K is compared on the bits as cached above (the bound here only catches a wrong angle or pairing)
+    ref_raw = oracle.batch_prefill_ragged(pf.q, pf.k, pf.v, dtype, pf.indptr, 8, 4, 128, causal=True, rope=True,
+                                          rope_theta=theta, parallel=True)
+    assert np.abs(got - ref_raw).max() <= (2e-3 if dtype == BZ_F16 else 3e-2), np.abs(got - ref_raw).max()
+    if float_ws_bytes >= 200 * 512:
+        # q only: k as the first call left it
+        pf2 = Prefill(210, [5, 200, 131, 1, 64], 8, 4, 128, dtype)
+        pf2.k = pf.k_after
+        got2 = pf2.run(causal=True, rope_mode=BZ_ROPE_Q_ONLY, theta=theta)
+        assert np.array_equal(got2, got)
+        assert np.array_equal(pf2.q_after, pf2.q) and np.array_equal(pf2.k_after, pf2.k)
 
 
 def test_prefill_then_store_then_decode_is_consistent():

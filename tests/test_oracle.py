@@ -423,3 +423,24 @@ def test_gemm_rounding_and_defaults():
     step = 2.0 ** (np.floor(np.log2(np.maximum(np.abs(want), 2.0 ** -14))) - 10)
     assert (np.abs(got.reshape(2, m, n) - want16) <= step).all()
     assert (got.reshape(2, m, n) == want16).mean() > 0.99
+
+
+def test_prefill_rope_q_only_mode():
+    """rope="q" (q rotated, k rows hold rotated K already) is pinned by the full mode: with fp32 storage nothing
+    is rounded in between, so rotating k beforehand with rope_llama and asking for q only must give the very
+    same numbers as rotating both inside the call."""
+    rng = np.random.default_rng(3)
+    lens = [5, 17, 1]
+    ip = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+    N = int(ip[-1])
+    q = rng.standard_normal((N, 4, 128)).astype(np.float32)
+    k = rng.standard_normal((N, 2, 128)).astype(np.float32)
+    v = rng.standard_normal((N, 2, 128)).astype(np.float32)
+    both = oracle.batch_prefill_ragged(q, k, v, oracle.F32, ip, 4, 2, 128, rope=True, rope_theta=5e5)
+    kr = k.copy()
+    for r, L in enumerate(lens):
+        for t in range(L):
+            for h in range(2):
+                kr[ip[r] + t, h] = oracle.rope_llama(k[ip[r] + t, h], t, 5e5)
+    assert np.array_equal(oracle.batch_prefill_ragged(q, kr, v, oracle.F32, ip, 4, 2, 128, rope="q", rope_theta=5e5), both)
+    assert not np.array_equal(oracle.batch_prefill_ragged(q, kr, v, oracle.F32, ip, 4, 2, 128, rope=False), both)
