@@ -597,9 +597,12 @@ def bench_layers(args):
 
     def step_layers(stream=None):
         for l in range(layers):
-            K.append_decode_kv_cache(pts[l], k[l], v[l], q=q[l], num_qo_heads=Hq, rope=True, rope_theta=5e5,
-                                     stream=stream)
-            K.batch_decode_attention(handler, q[l], pts[l], out[l], Hq, rope_mode=BZ_ROPE_NONE, stream=stream)
+            if args.two_call:  # the reference's two calls: append (rotates q and k in place), then attention
+                K.append_decode_kv_cache(pts[l], k[l], v[l], q=q[l], num_qo_heads=Hq, rope=True, rope_theta=5e5,
+                                         stream=stream)
+                K.batch_decode_attention(handler, q[l], pts[l], out[l], Hq, rope_mode=BZ_ROPE_NONE, stream=stream)
+            else:              # both as one call (two launches; q is rotated inside the kernels and left as it is)
+                K.decode_step(handler, q[l], k[l], v[l], pts[l], out[l], Hq, rope=True, rope_theta=5e5, stream=stream)
 
     steps = args.steps or 50
     warmup = args.warmup if args.warmup is not None else 5
@@ -673,7 +676,8 @@ def bench_layers(args):
             "n_gpus": 1, "steps": steps, "warmup": warmup, "ms_per_step": round(graph_ms, 6),
             "higher_is_better": False, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
             "config": {"workload": "LAYERS: attention part (fused RoPE + append, paged decode) of 32 Llama-3-8B "
-                                   f"layers, batch {B}, context {ctx}, one plan per step; value = HIP-graph replay"},
+                                   f"layers, batch {B}, context {ctx}, one plan per step; value = HIP-graph replay",
+                       "calls_per_layer": "append + attention" if args.two_call else "decode_step"},
             "eager_us_per_step": round(eager_ms * 1e3, 2), "graph_us_per_step": round(graph_ms * 1e3, 2),
             "us_per_layer": {"eager": round(eager_ms * 1e3 / layers, 2), "graph": round(graph_ms * 1e3 / layers, 2)},
             "graph_replay_bit_exact_vs_eager": same,

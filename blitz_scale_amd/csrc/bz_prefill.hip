@@ -386,11 +386,13 @@ __global__ __launch_bounds__(256, 2) void prefill_kernel(PrefillArgs a, const ch
                 const float shift = t == 0 ? tmax : fmaxf(tmax, 0.f);
                 const float alpha = __builtin_amdgcn_exp2f(QSCALED ? -shift : -shift * a.sm_scale_log2);
                 m_run += shift;
-                l_run *= alpha;
+                if (t != 0) { // (nothing has been accumulated before the first tile)
+                    l_run *= alpha;
 #pragma unroll
-                for (int db = 0; db < 4; ++db)
+                    for (int db = 0; db < 4; ++db)
 #pragma unroll
-                    for (int i = 0; i < 16; ++i) acc[db][i] *= alpha;
+                        for (int i = 0; i < 16; ++i) acc[db][i] *= alpha;
+                }
 #pragma unroll
                 for (int i = 0; i < 16; ++i) cinit[i] = -m_run;
                 probabilities(shift);
