@@ -304,7 +304,10 @@ __global__ __launch_bounds__(64, 2) void decode_mfma_kernel(MfmaDecodeArgs a, co
 
     // The records of the first 32 tiles are requested first and the first tile's q, K and V right behind
     // them (its description came with the slot head), so parking the records in LDS waits for them only.
-    const Desc d0 = fetch_info(g_begin);
+    // (a slot with a single tile -- small batches -- needs no records at all, and fetching them would put two more
+    // dependent round trips in front of its K/V loads)
+    Desc d0 = {};
+    if (g_end - g_begin > 1) d0 = fetch_info(g_begin);
     TileUni un; // description of the tile whose loads are issued next
     un.pid0 = indices[first.idx0];
     un.pid1 = indices[first.idx1];
@@ -315,8 +318,10 @@ __global__ __launch_bounds__(64, 2) void decode_mfma_kernel(MfmaDecodeArgs a, co
     un.tok_end = min(first.tile_end * kTileTok, un.seq_len);
     issue_q(un);
     issue_loads(tile_base(un));
-    stash_info(d0, 0);
-    wave_lds_sync();
+    if (g_end - g_begin > 1) {
+        stash_info(d0, 0);
+        wave_lds_sync();
+    }
     int chunk_base = g_begin, buf = 0;
     Desc dnext;
 

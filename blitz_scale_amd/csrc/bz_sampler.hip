@@ -41,71 +41,92 @@ template <typename T> __device__ __forceinline__ float elem_f32(uint16_t bits);
 template <> __device__ __forceinline__ float elem_f32<f16_t>(uint16_t bits) { return __half2float(__ushort_as_half(bits)); }
 template <> __device__ __forceinline__ float elem_f32<bf16_t>(uint16_t bits) { return __uint_as_float((uint32_t)bits << 16); }
 
-// (value, index) order of the argmax: larger value first, then smaller index; NaN never wins
-__device__ __forceinline__ bool better(float v, uint32_t i, float bv, uint32_t bi) {
-    return v > bv || (v == bv && i < bi);
+// Order of the argmax: a non-NaN value maps to an integer key that sorts like the value (-0 and +0 share
+// a key, as they compare equal), NaN to the smallest integer, which never beats the starting key.
+constexpr int kNoKey = (int)0x80000000;
+constexpr uint32_t kNoIndex = 0xFFFFFFFFu; // "nothing seen": loses every tie
+__device__ __forceinline__ int order_key(float v) {
+    int b = __float_as_int(v);
+    if ((b & 0x7fffffff) > 0x7f800000) return kNoKey; // NaN
+    if (b == kNoKey) b = 0;                           // -0
+    return b ^ ((b >> 31) & 0x7fffffff);
+}
+__device__ __forceinline__ bool better(int key, uint32_t i, int bkey, uint32_t bi) {
+    return key > bkey || (key == bkey && i < bi);
 }
 
-// grid (batch), block 1024: 16-byte loads where the row start allows it, scalar head and tail
+// grid (batch), block 1024: 16-byte loads where the row start allows it, scalar head and tail.  The scan is
+// bound by vector instructions, not by memory, when every element is compared on its own (seven
+// instructions each); so a lane takes the maximum of the eight values of a load first (v_max3, NaN operands
+// drop out), compares once per load, remembers only which load held its best value, and fetches that one load
+// again at the end to find the element.
 template <typename T>
 __global__ __launch_bounds__(1024) void batch_find_max_kernel(uint32_t* __restrict__ out, const uint16_t* __restrict__ in,
                                                                uint32_t length) {
-    __shared__ float s_val[16];
+    __shared__ int s_key[16];
     __shared__ uint32_t s_idx[16];
     const uint16_t* row = in + (size_t)blockIdx.x * length;
-    float best = -INFINITY;
-    uint32_t best_i = 0xFFFFFFFFu; // "nothing seen": loses every tie
     // elements before the first 16-byte boundary of the row, then whole vectors, then the tail
     const uint32_t head = min(length, (uint32_t)(((16 - ((uintptr_t)row & 15)) & 15) / 2));
     const uint32_t nvec = (length - head) / 8;
-    for (uint32_t i = threadIdx.x; i < head; i += blockDim.x) {
-        const float v = elem_f32<T>(row[i]);
-        if (better(v, i, best, best_i)) { best = v; best_i = i; }
-    }
     const uint4* vrow = reinterpret_cast<const uint4*>(row + head);
-    auto take = [&](const uint4& w, uint32_t k) {
+    int best = kNoKey;
+    uint32_t best_vec = kNoIndex;
+    auto take = [&](const uint4& w, uint32_t k) { // k ascends within a lane: the first of equal maxima stays
+        const uint32_t ws[4] = {w.x, w.y, w.z, w.w};
+        float m = elem_f32<T>((uint16_t)ws[0]);
+#pragma unroll
+        for (int e = 1; e < 8; ++e) m = fmaxf(m, elem_f32<T>((uint16_t)(ws[e >> 1] >> (16 * (e & 1))))); // NaN only if all are
+        const int key = order_key(m);
+        if (key > best) { best = key; best_vec = k; }
+    };
+    // One workgroup (one CU) per row: what a CU streams is bounded by the bytes it has in flight, so every lane
+    // keeps eight 16-byte loads outstanding (128 KiB per CU).
+    uint32_t k = threadIdx.x;
+    const uint32_t nt = blockDim.x;
+    for (; k < nvec; k += 8 * nt) { // (the last round re-reads the row's last load where it runs past the end)
+        uint4 w[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) w[u] = vrow[min(k + u * nt, nvec - 1)];
+#pragma unroll
+        for (int u = 0; u < 8; ++u)
+            if (k + u * nt < nvec) take(w[u], k + u * nt);
+    }
+    uint32_t best_i = kNoIndex;
+    if (best_vec != kNoIndex) { // the first element of that load with the lane's best key
+        const uint4 w = vrow[best_vec];
         const uint32_t ws[4] = {w.x, w.y, w.z, w.w};
 #pragma unroll
-        for (int e = 0; e < 8; ++e) {
-            const float v = elem_f32<T>((uint16_t)(ws[e >> 1] >> (16 * (e & 1))));
-            const uint32_t i = head + 8 * k + e;
-            if (better(v, i, best, best_i)) { best = v; best_i = i; }
-        }
+        for (int e = 7; e >= 0; --e)
+            if (order_key(elem_f32<T>((uint16_t)(ws[e >> 1] >> (16 * (e & 1))))) == best) best_i = head + 8 * best_vec + e;
+    }
+    auto take_one = [&](uint32_t i) {
+        const int key = order_key(elem_f32<T>(row[i]));
+        if (key != kNoKey && better(key, i, best, best_i)) { best = key; best_i = i; }
     };
-    uint32_t k = threadIdx.x;
-    for (; k + 3 * blockDim.x < nvec; k += 4 * blockDim.x) { // four loads in flight per lane
-        const uint4 w0 = vrow[k], w1 = vrow[k + blockDim.x], w2 = vrow[k + 2 * blockDim.x], w3 = vrow[k + 3 * blockDim.x];
-        take(w0, k);
-        take(w1, k + blockDim.x);
-        take(w2, k + 2 * blockDim.x);
-        take(w3, k + 3 * blockDim.x);
-    }
-    for (; k < nvec; k += blockDim.x) take(vrow[k], k);
-    for (uint32_t i = head + 8 * nvec + threadIdx.x; i < length; i += blockDim.x) {
-        const float v = elem_f32<T>(row[i]);
-        if (better(v, i, best, best_i)) { best = v; best_i = i; }
-    }
+    for (uint32_t i = threadIdx.x; i < head; i += blockDim.x) take_one(i);
+    for (uint32_t i = head + 8 * nvec + threadIdx.x; i < length; i += blockDim.x) take_one(i);
     // wave64 reduction, then one value per wave through LDS
 #pragma unroll
     for (int off = 32; off > 0; off >>= 1) {
-        const float ov = __shfl_xor(best, off, 64);
+        const int ok = __shfl_xor(best, off, 64);
         const uint32_t oi = __shfl_xor(best_i, off, 64);
-        if (better(ov, oi, best, best_i)) { best = ov; best_i = oi; }
+        if (better(ok, oi, best, best_i)) { best = ok; best_i = oi; }
     }
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-    if (lane == 0) { s_val[wave] = best; s_idx[wave] = best_i; }
+    if (lane == 0) { s_key[wave] = best; s_idx[wave] = best_i; }
     __syncthreads();
     if (wave == 0) {
         const int nw = blockDim.x >> 6;
-        best = lane < nw ? s_val[lane] : -INFINITY;
-        best_i = lane < nw ? s_idx[lane] : 0xFFFFFFFFu;
+        best = lane < nw ? s_key[lane] : kNoKey;
+        best_i = lane < nw ? s_idx[lane] : kNoIndex;
 #pragma unroll
         for (int off = 8; off > 0; off >>= 1) {
-            const float ov = __shfl_xor(best, off, 64);
+            const int ok = __shfl_xor(best, off, 64);
             const uint32_t oi = __shfl_xor(best_i, off, 64);
-            if (better(ov, oi, best, best_i)) { best = ov; best_i = oi; }
+            if (better(ok, oi, best, best_i)) { best = ok; best_i = oi; }
         }
-        if (lane == 0) out[blockIdx.x] = best_i == 0xFFFFFFFFu ? 0u : best_i; // no non-NaN element: 0
+        if (lane == 0) out[blockIdx.x] = best_i == kNoIndex ? 0u : best_i; // no non-NaN element: 0
     }
 }
 

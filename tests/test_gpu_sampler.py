@@ -74,3 +74,40 @@ def test_argmax_of_all_nan_row_is_zero():
     K.batch_find_max(out, to_dev(x, BZ_F16), 2, 100)
     torch.cuda.synchronize()
     assert out.cpu().tolist() == [0, 0]
+
+
+@pytest.mark.parametrize("dtype", [BZ_F16, BZ_BF16])
+@pytest.mark.parametrize("length", [8, 40, 9000, 128256])
+def test_argmax_special_values_anywhere_in_the_row(dtype, length):
+    """Ties (also between -0 and +0, and between values met by different lanes, loads and waves), -inf, NaN of both
+    signs, subnormals and rows without a finite value: the smallest index of the largest non-NaN value."""
+    rng = np.random.default_rng(length)
+    enc = (lambda v: wl.to_bits(np.asarray(v, np.float32), dtype))
+    ninf, nan = np.float32(-np.inf), np.float32(np.nan)
+    neg_nan = np.uint16(0xFE00 if dtype == BZ_F16 else 0xFFC0)
+    sub = np.uint16(0x0001)  # smallest positive subnormal of either format
+
+    def fill(v):
+        return np.full(length, enc([v])[0], np.uint16)
+
+    def at(n):
+        return np.sort(rng.choice(length, size=min(n, length), replace=False))
+
+    rows = []
+    r = fill(1.0); r[at(5)] = enc([5.0])[0]; rows.append(r)                     # ties of the maximum
+    rows.append(fill(ninf))                                                       # all -inf: index 0
+    r = fill(ninf); r[at(1)] = enc([-65504.0])[0]; rows.append(r)                 # one finite value, very negative
+    r = fill(nan); p = at(3); r[p] = enc([7.0])[0]; r[p[0]] = enc([3.0])[0]; rows.append(r)  # NaN never wins
+    rows.append(fill(nan))                                                        # no non-NaN element: 0
+    r = fill(-1.0); p = at(4); r[p] = enc([0.0])[0]; r[p[::2]] = enc([-0.0])[0]; rows.append(r)  # -0 == +0: the first
+    r = fill(ninf); r[:] = neg_nan; r[at(2)] = enc([ninf])[0]; rows.append(r)     # negative NaN against -inf
+    r = fill(0.0); r[at(2)] = sub; rows.append(r)                                 # a subnormal above zero
+    r = fill(-0.0); r[0] = enc([nan])[0]; rows.append(r)                          # NaN first, then zeros
+    x = np.stack(rows)
+    out = torch.full((len(rows),), -1, dtype=torch.int32, device="cuda")
+    K.batch_find_max(out, to_dev(x, dtype), len(rows), length)
+    torch.cuda.synchronize()
+    want = oracle.batch_find_max(x, dtype)
+    f = wl.to_f32(x, dtype)
+    assert want[4] == 0 and (length < 2 or want[8] == 1) and f[0, want[0]] == 5.0  # (the checker itself, on these rows)
+    assert np.array_equal(out.cpu().numpy().view(np.uint32), want)
