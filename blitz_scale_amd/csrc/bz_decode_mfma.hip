@@ -12,6 +12,7 @@
 //   softmax  : online, 8 scores per lane, row max / sum over the 4 lane groups with two shuffles
 // The loads of tile t+1 are issued before the arithmetic of tile t.
 #include <cmath>
+#include <type_traits>
 
 #include "bz_common.hpp"
 #include "bz_decode_plan.hpp"
@@ -172,7 +173,9 @@ __global__ __launch_bounds__(64, 2) void decode_mfma_kernel(MfmaDecodeArgs a, co
                                                             const int32_t* __restrict__ indices,
                                                             const MfmaPiece* __restrict__ pieces,
                                                             const MfmaTile* __restrict__ tiles,
-                                                            const MfmaSlotHead* __restrict__ heads) {
+                                                            const MfmaSlotHead* __restrict__ heads,
+                                                            const float* __restrict__ k_scale,
+                                                            const float* __restrict__ v_scale) {
     using M = Mma<BF16>;
     __shared__ __attribute__((aligned(16))) unsigned char v_lds[kTileTok * kVRowBytes];
     __shared__ __attribute__((aligned(16))) int info_lds[2][kInfoChunk][kInfoInts];
@@ -265,30 +268,38 @@ __global__ __launch_bounds__(64, 2) void decode_mfma_kernel(MfmaDecodeArgs a, co
         }
         return r;
     };
+    // One-byte pools: a tile is 8 KiB and lands in half of the registers a 16-bit tile needs, so the two halves
+    // are two sets (SET 0 / 1: kreg[u][2 SET + p], vreg[4 SET + w]) and two tiles are in flight per wave.
+    // `live` false: the set has no tile to fetch; the loads are issued all the same, every lane at the tile's first
+    // bytes (one cache line), so that the number of loads behind a set's own does not depend on the path taken
+    // and the waits the compiler derives for the sets stay apart.
+    auto issue_loads_kv8 = [&](const TileBase& tb, auto set_c, bool live) __attribute__((always_inline)) {
+        constexpr int SET = decltype(set_c)::value;
+        const size_t base[2] = {tb.b[0], tb.b[1]};
+        const size_t koff = live ? (size_t)n * row_bytes + (size_t)(j * 16) : 0;
+#pragma unroll
+        for (int p = 0; p < 2; ++p) { // 16 bytes feed MFMA steps 2p and 2p+1
+            kreg[0][2 * SET + p] = ld_kv16(k_data + base[0] + koff + (live ? p * 64 : 0), NT && kNtK8);
+            kreg[1][2 * SET + p] = ld_kv16(k_data + base[1] + koff + (live ? p * 64 : 0), NT && kNtK8);
+        }
+#pragma unroll
+        for (int w = 0; w < 4; ++w) { // rows 8w..8w+7 of the tile, 8 lanes x 16 B per 128-byte row
+            const int row = 8 * w + (lane >> 3);
+            const size_t voff = live ? (size_t)(row & 15) * row_bytes + (size_t)((lane & 7) * 16) : 0;
+            vreg[4 * SET + w] = ld_kv16(v_data + base[live ? (row >> 4) : 0] + voff, NT && kNtV8);
+        }
+    };
     auto issue_loads = [&](const TileBase& tb) {
         const size_t base[2] = {tb.b[0], tb.b[1]};
-        if constexpr (KV8) {
 #pragma unroll
-            for (int p = 0; p < 2; ++p) { // 16 bytes feed MFMA steps 2p and 2p+1
-                kreg[0][p] = ld_kv16(k_data + base[0] + (size_t)n * row_bytes + p * 64 + j * 16, NT && kNtK8);
-                kreg[1][p] = ld_kv16(k_data + base[1] + (size_t)n * row_bytes + p * 64 + j * 16, NT && kNtK8);
-            }
+        for (int ks = 0; ks < 4; ++ks) {
+            kreg[0][ks] = ld_kv16(k_data + base[0] + (size_t)n * row_bytes + ks * 64 + j * 16, NT && kNtK16);
+            kreg[1][ks] = ld_kv16(k_data + base[1] + (size_t)n * row_bytes + ks * 64 + j * 16, NT && kNtK16);
+        }
 #pragma unroll
-            for (int w = 0; w < 4; ++w) { // rows 8w..8w+7 of the tile, 8 lanes x 16 B per 128-byte row
-                const int row = 8 * w + (lane >> 3);
-                vreg[w] = ld_kv16(v_data + base[row >> 4] + (size_t)(row & 15) * row_bytes + (lane & 7) * 16, NT && kNtV8);
-            }
-        } else {
-#pragma unroll
-            for (int ks = 0; ks < 4; ++ks) {
-                kreg[0][ks] = ld_kv16(k_data + base[0] + (size_t)n * row_bytes + ks * 64 + j * 16, NT && kNtK16);
-                kreg[1][ks] = ld_kv16(k_data + base[1] + (size_t)n * row_bytes + ks * 64 + j * 16, NT && kNtK16);
-            }
-#pragma unroll
-            for (int w = 0; w < 8; ++w) { // rows 4w..4w+3 of the tile, 16 lanes x 16 B per row
-                const int row = 4 * w + j;
-                vreg[w] = ld_kv16(v_data + base[row >> 4] + (size_t)(row & 15) * row_bytes + n * 16, NT && kNtV16);
-            }
+        for (int w = 0; w < 8; ++w) { // rows 4w..4w+3 of the tile, 16 lanes x 16 B per row
+            const int row = 4 * w + j;
+            vreg[w] = ld_kv16(v_data + base[row >> 4] + (size_t)(row & 15) * row_bytes + n * 16, NT && kNtV16);
         }
     };
     // q rows of a piece as MFMA B operand: lane (head n, group j) holds q[head][32*ks + 8*j .. +7]
@@ -302,7 +313,7 @@ __global__ __launch_bounds__(64, 2) void decode_mfma_kernel(MfmaDecodeArgs a, co
         }
     };
 
-    // The records of the first 32 tiles are requested first and the first tile's q, K and V right behind
+    // The records of the first tiles are requested first and the first tile's q, K and V right behind
     // them (its description came with the slot head), so parking the records in LDS waits for them only.
     // (a slot with a single tile -- small batches -- needs no records at all, and fetching them would put two more
     // dependent round trips in front of its K/V loads)
@@ -317,7 +328,8 @@ __global__ __launch_bounds__(64, 2) void decode_mfma_kernel(MfmaDecodeArgs a, co
     un.seq_len = max(first.seq_len - ahead - a.step_mode, 0);
     un.tok_end = min(first.tile_end * kTileTok, un.seq_len);
     issue_q(un);
-    issue_loads(tile_base(un));
+    if constexpr (KV8) issue_loads_kv8(tile_base(un), std::integral_constant<int, 0>{}, true);
+    else issue_loads(tile_base(un));
     if (g_end - g_begin > 1) {
         stash_info(d0, 0);
         wave_lds_sync();
@@ -329,143 +341,74 @@ __global__ __launch_bounds__(64, 2) void decode_mfma_kernel(MfmaDecodeArgs a, co
     float m_run = -INFINITY, l_run = 0.f;
     f32x4_t acc[8];
 
-    for (int g = g_begin; g < g_end; ++g) {
-        const TileUni uc = un; // the tile computed in this iteration (its loads are in flight or done)
-        const int i = g - chunk_base;
-        // The description and the addresses of the next tile come first, while this tile's data is
-        // still on its way: the time between its arrival and the next loads is time in which this
-        // wave has nothing in flight.
-        TileBase nb;
-        if (g + 1 < g_end) {
-            const int nbuf = (i + 1 == kInfoChunk) ? buf ^ 1 : buf;
-            un = read_info(nbuf, (i + 1) & (kInfoChunk - 1));
-            nb = tile_base(un);
-        }
-        __builtin_amdgcn_sched_barrier(0);
-        // descriptions of the next chunk of tiles: fetched a quarter into this chunk, parked in the other LDS
-        // buffer at three quarters
+    // descriptions of the next chunk of tiles: fetched a quarter into this chunk, parked in the other LDS
+    // buffer at three quarters
+    auto info_traffic = [&](int i) __attribute__((always_inline)) {
         if (i == kInfoChunk / 4 && chunk_base + kInfoChunk < g_end) dnext = fetch_info(chunk_base + kInfoChunk);
         if (i == 3 * kInfoChunk / 4 && chunk_base + kInfoChunk < g_end) { stash_info(dnext, buf ^ 1); wave_lds_sync(); }
-        const int t = uc.t, tok_end = uc.tok_end, seq_len = uc.seq_len;
-        // (positive; the floor keeps masked scores at -inf instead of NaN should a head's K scale be zero)
-        const float score_scale = fmaxf(a.sm_scale_log2 * ((KV8 && a.k_scale) ? a.k_scale[uc.kvr] : 1.0f), 1e-30f);
-
-        if (uc.flags & 1) { // ================= first tile of a piece =================
+    };
+    // (positive; the floor keeps masked scores at -inf instead of NaN should a head's K scale be zero)
+    auto score_scale_of = [&](const TileUni& uc) __attribute__((always_inline)) {
+        return fmaxf(a.sm_scale_log2 * ((KV8 && k_scale) ? k_scale[uc.kvr] : 1.0f), 1e-30f);
+    };
+    // ================= first tile of a piece =================
+    auto open_piece = [&](const TileUni& uc) __attribute__((always_inline)) {
 #pragma unroll
-            for (int ks = 0; ks < 4; ++ks) { qhi[ks] = qnext[ks]; qlo[ks] = make_uint4(0, 0, 0, 0); }
-            if (ROPE_Q) {
-                float sn1, cs1;
-                sincosf((float)(seq_len - 1 + a.step_mode) * a.freqs.f[lane], &sn1, &cs1); // q sits at the last token
-                wave_lds_sync(); // the previous piece's reads of the table are done
-                rope_cs[0][lane] = cs1;
-                rope_cs[ROPE_Q ? 1 : 0][lane] = sn1; // (the index keeps the one-row dummy of the other instantiations in bounds)
-                wave_lds_sync();
-            }
-            if (ROPE_Q && n < G) {
-                // the rotated q is split into a storage-precision head and tail (q = hi + lo) and both are
-                // contracted, so rotating inside the kernel costs no precision
-#pragma unroll
-                for (int ks = 0; ks < 2; ++ks) { // dims d = 32ks+8j+e pair with d+64, held at ks+2
-#pragma unroll
-                    for (int w = 0; w < 4; ++w) {
-                        float x[2] = {M::unpack_lo(u4(qhi[ks], w)), M::unpack_hi(u4(qhi[ks], w))};
-                        float y[2] = {M::unpack_lo(u4(qhi[ks + 2], w)), M::unpack_hi(u4(qhi[ks + 2], w))};
-                        float xr[2], yr[2];
-#pragma unroll
-                        for (int e = 0; e < 2; ++e) {
-                            const float c = rope_cs[0][d_of(ks) + 2 * w + e], s = rope_cs[ROPE_Q ? 1 : 0][d_of(ks) + 2 * w + e];
-                            rope_pair(x[e], y[e], c, s, xr[e], yr[e]);
-                        }
-                        const uint32_t xh = M::pack2(xr[0], xr[1]), yh = M::pack2(yr[0], yr[1]);
-                        u4(qhi[ks], w) = xh;
-                        u4(qhi[ks + 2], w) = yh;
-                        u4(qlo[ks], w) = M::pack2(xr[0] - M::unpack_lo(xh), xr[1] - M::unpack_hi(xh));
-                        u4(qlo[ks + 2], w) = M::pack2(yr[0] - M::unpack_lo(yh), yr[1] - M::unpack_hi(yh));
-                    }
-                }
-            }
-            m_run = -INFINITY;
-            l_run = 0.f;
-#pragma unroll
-            for (int d = 0; d < 8; ++d) acc[d] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+        for (int ks = 0; ks < 4; ++ks) { qhi[ks] = qnext[ks]; qlo[ks] = make_uint4(0, 0, 0, 0); }
+        if (ROPE_Q) {
+            float sn1, cs1;
+            sincosf((float)(uc.seq_len - 1 + a.step_mode) * a.freqs.f[lane], &sn1, &cs1); // q sits at the last token
+            wave_lds_sync(); // the previous piece's reads of the table are done
+            rope_cs[0][lane] = cs1;
+            rope_cs[ROPE_Q ? 1 : 0][lane] = sn1; // (the index keeps the one-row dummy of the other instantiations in bounds)
+            wave_lds_sync();
         }
-
-        // ================= one tile =================
-        const int tile_tok0 = t * kTileTok;
-        const bool ragged = tile_tok0 + kTileTok > tok_end; // wave-uniform
-        wave_lds_sync(); // transposed reads of the previous tile come before V is overwritten
-        // (the masked variant sits behind a wave-uniform branch: written as one predicated sequence it costs
-        // eight register moves and an exec-mask round trip per row on every tile, between the arrival of a
-        // tile and the next loads)
-        if constexpr (KV8) {
-            if (!ragged) {
+        if (ROPE_Q && n < G) {
+            // the rotated q is split into a storage-precision head and tail (q = hi + lo) and both are
+            // contracted, so rotating inside the kernel costs no precision
 #pragma unroll
-                for (int w = 0; w < 4; ++w) { // 16 e4m3 bytes -> 16 operand-type values -> 32 B of the LDS row
-                    unsigned char* dst = v_lds + (8 * w + (lane >> 3)) * kVRowBytes + (lane & 7) * 32;
-                    *reinterpret_cast<uint4*>(dst) = fp8x8_to_op<BF16>(vreg[w], 0);
-                    *reinterpret_cast<uint4*>(dst + 16) = fp8x8_to_op<BF16>(vreg[w], 1);
-                }
-            } else {
+            for (int ks = 0; ks < 2; ++ks) { // dims d = 32ks+8j+e pair with d+64, held at ks+2
 #pragma unroll
                 for (int w = 0; w < 4; ++w) {
-                    uint4 v = vreg[w];
-                    const int row = 8 * w + (lane >> 3);
-                    if (tile_tok0 + row >= tok_end) v = make_uint4(0, 0, 0, 0); // 0 * garbage must be 0
-                    unsigned char* dst = v_lds + row * kVRowBytes + (lane & 7) * 32;
-                    *reinterpret_cast<uint4*>(dst) = fp8x8_to_op<BF16>(v, 0);
-                    *reinterpret_cast<uint4*>(dst + 16) = fp8x8_to_op<BF16>(v, 1);
-                }
-            }
-        } else {
-            if (!ragged) {
+                    float x[2] = {M::unpack_lo(u4(qhi[ks], w)), M::unpack_hi(u4(qhi[ks], w))};
+                    float y[2] = {M::unpack_lo(u4(qhi[ks + 2], w)), M::unpack_hi(u4(qhi[ks + 2], w))};
+                    float xr[2], yr[2];
 #pragma unroll
-                for (int w = 0; w < 8; ++w)
-                    *reinterpret_cast<uint4*>(v_lds + (4 * w + j) * kVRowBytes + n * 16) = vreg[w];
-            } else {
-#pragma unroll
-                for (int w = 0; w < 8; ++w) {
-                    uint4 v = vreg[w];
-                    if (tile_tok0 + 4 * w + j >= tok_end) v = make_uint4(0, 0, 0, 0); // 0 * garbage must be 0
-                    *reinterpret_cast<uint4*>(v_lds + (4 * w + j) * kVRowBytes + n * 16) = v;
+                    for (int e = 0; e < 2; ++e) {
+                        const float c = rope_cs[0][d_of(ks) + 2 * w + e], s = rope_cs[ROPE_Q ? 1 : 0][d_of(ks) + 2 * w + e];
+                        rope_pair(x[e], y[e], c, s, xr[e], yr[e]);
+                    }
+                    const uint32_t xh = M::pack2(xr[0], xr[1]), yh = M::pack2(yr[0], yr[1]);
+                    u4(qhi[ks], w) = xh;
+                    u4(qhi[ks + 2], w) = yh;
+                    u4(qlo[ks], w) = M::pack2(xr[0] - M::unpack_lo(xh), xr[1] - M::unpack_hi(xh));
+                    u4(qlo[ks + 2], w) = M::pack2(yr[0] - M::unpack_lo(yh), yr[1] - M::unpack_hi(yh));
                 }
             }
         }
-        // 16-bit pools: the K rows are contracted straight out of their landing registers and the next
-        // tile's loads go out right behind the eight score instructions (which have read their operands
-        // by then); e4m3 pools: the rows are widened into operand registers first, which frees the landing
-        // registers, so the loads go out before the contraction.
-        auto issue_next = [&]() {
-            if (g + 1 < g_end) {
-                if (i + 1 == kInfoChunk) { chunk_base += kInfoChunk; buf ^= 1; }
-                if (un.flags & 1) issue_q(un); // next tile opens a new piece
-                issue_loads(nb);
-            }
-        };
-        uint4 kcur[2][4];
-        if constexpr (KV8) {
+        m_run = -INFINITY;
+        l_run = 0.f;
 #pragma unroll
-            for (int u = 0; u < 2; ++u)
-#pragma unroll
-                for (int ks = 0; ks < 4; ++ks) kcur[u][ks] = fp8x8_to_op<BF16>(kreg[u][ks >> 1], ks & 1);
-            issue_next();
-        }
-        // ---- scores: S^T[token][head], lane (head n, group j) gets tokens 16u + 4j + r
-        f32x4_t s[2];
+        for (int d = 0; d < 8; ++d) acc[d] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+    };
+    // ---- scores: S^T[token][head], lane (head n, group j) gets tokens 16u + 4j + r
+    auto scores = [&](const uint4 (&kop)[2][4], f32x4_t (&s)[2]) __attribute__((always_inline)) {
 #pragma unroll
         for (int u = 0; u < 2; ++u) {
             s[u] = f32x4_t{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-            for (int ks = 0; ks < 4; ++ks) s[u] = M::run(KV8 ? kcur[u][ks] : kreg[u][ks], qhi[ks], s[u]);
+            for (int ks = 0; ks < 4; ++ks) s[u] = M::run(kop[u][ks], qhi[ks], s[u]);
             if (ROPE_Q) {
 #pragma unroll
-                for (int ks = 0; ks < 4; ++ks) s[u] = M::run(KV8 ? kcur[u][ks] : kreg[u][ks], qlo[ks], s[u]);
+                for (int ks = 0; ks < 4; ++ks) s[u] = M::run(kop[u][ks], qlo[ks], s[u]);
             }
         }
-        if constexpr (!KV8) {
-            __builtin_amdgcn_sched_barrier(0); // the loads below overwrite the operands of the instructions above
-            issue_next();
-        }
-        if (ragged) { // wave-uniform
+    };
+    // ---- mask, online softmax, O += P V (V of the tile is in LDS), and the rows of a finished piece
+    auto softmax_pv = [&](const TileUni& uc, f32x4_t (&s)[2], float score_scale) __attribute__((always_inline)) {
+        const int tile_tok0 = uc.t * kTileTok, tok_end = uc.tok_end;
+        const bool ragged = tile_tok0 + kTileTok > tok_end; // wave-uniform
+        if (ragged) {
 #pragma unroll
             for (int u = 0; u < 2; ++u)
 #pragma unroll
@@ -535,7 +478,7 @@ __global__ __launch_bounds__(64, 2) void decode_mfma_kernel(MfmaDecodeArgs a, co
 
         if (uc.flags & 2) { // ================= last tile of a piece: final rows, or the split-K partial
             const int b = uc.seq, kvh = uc.kvh, partial = uc.partial;
-            const float inv_l = (l_run > 0.f ? 1.0f / l_run : 0.f) * ((KV8 && a.v_scale) ? a.v_scale[uc.kvr] : 1.0f);
+            const float inv_l = (l_run > 0.f ? 1.0f / l_run : 0.f) * ((KV8 && v_scale) ? v_scale[uc.kvr] : 1.0f);
             const float lse2 = l_run > 0.f ? m_run + log2f(l_run) : -INFINITY;
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
@@ -560,6 +503,127 @@ __global__ __launch_bounds__(64, 2) void decode_mfma_kernel(MfmaDecodeArgs a, co
                     a.part_lse[(size_t)partial * 16 + n] = lse2;
                 }
             }
+        }
+    };
+
+    if constexpr (KV8) {
+        // ---- one-byte pools: two tiles in flight.  Tile g lives in set (g - g_begin) % 2; its set is refilled with
+        // tile g + 2 as soon as its bytes have been widened into operand registers (K) and parked in LDS (V).
+        TileUni dA = un, dB = un; // descriptions of the tiles in sets 0 and 1
+        {
+            const bool second = g_begin + 1 < g_end;
+            if (second) dB = read_info(0, 1);
+            issue_loads_kv8(tile_base(dB), std::integral_constant<int, 1>{}, second);
+        }
+        auto body = [&](int g, auto set_c) __attribute__((always_inline)) {
+            constexpr int SET = decltype(set_c)::value;
+            const TileUni uc = SET ? dB : dA;
+            const int i = g - chunk_base;
+            // the tile after next, which takes over this set
+            const bool more = g + 2 < g_end;
+            TileUni u2 = uc;
+            if (more) u2 = read_info(i + 2 >= kInfoChunk ? buf ^ 1 : buf, (i + 2) & (kInfoChunk - 1));
+            const TileBase nb = tile_base(u2);
+            __builtin_amdgcn_sched_barrier(0);
+            info_traffic(i);
+            const float score_scale = score_scale_of(uc);
+            if (uc.flags & 1) open_piece(uc);
+
+            const int tile_tok0 = uc.t * kTileTok;
+            const bool ragged = tile_tok0 + kTileTok > uc.tok_end; // wave-uniform
+            wave_lds_sync(); // transposed reads of the previous tile come before V is overwritten
+            if (!ragged) {
+#pragma unroll
+                for (int w = 0; w < 4; ++w) { // 16 e4m3 bytes -> 16 operand-type values -> 32 B of the LDS row
+                    unsigned char* dst = v_lds + (8 * w + (lane >> 3)) * kVRowBytes + (lane & 7) * 32;
+                    *reinterpret_cast<uint4*>(dst) = fp8x8_to_op<BF16>(vreg[4 * SET + w], 0);
+                    *reinterpret_cast<uint4*>(dst + 16) = fp8x8_to_op<BF16>(vreg[4 * SET + w], 1);
+                }
+            } else {
+#pragma unroll
+                for (int w = 0; w < 4; ++w) {
+                    uint4 v = vreg[4 * SET + w];
+                    const int row = 8 * w + (lane >> 3);
+                    if (tile_tok0 + row >= uc.tok_end) v = make_uint4(0, 0, 0, 0); // 0 * garbage must be 0
+                    unsigned char* dst = v_lds + row * kVRowBytes + (lane & 7) * 32;
+                    *reinterpret_cast<uint4*>(dst) = fp8x8_to_op<BF16>(v, 0);
+                    *reinterpret_cast<uint4*>(dst + 16) = fp8x8_to_op<BF16>(v, 1);
+                }
+            }
+            uint4 kcur[2][4];
+#pragma unroll
+            for (int u = 0; u < 2; ++u)
+#pragma unroll
+                for (int ks = 0; ks < 4; ++ks) kcur[u][ks] = fp8x8_to_op<BF16>(kreg[u][2 * SET + (ks >> 1)], ks & 1);
+            // the set is free: q rows of the next tile's piece (one tile ahead), K/V of the tile after next
+            if (g + 1 < g_end) {
+                const TileUni& u1 = SET ? dA : dB;
+                if (u1.flags & 1) issue_q(u1);
+            }
+            issue_loads_kv8(nb, set_c, more);
+            if (SET) dB = u2; else dA = u2;
+            if (i + 1 == kInfoChunk) { chunk_base += kInfoChunk; buf ^= 1; }
+            f32x4_t s[2];
+            scores(kcur, s);
+            softmax_pv(uc, s, score_scale);
+        };
+        // (The loop has no exit between its halves, so that the only way into one set's half is through the
+        // other set's half: the waits the compiler places for a set's registers then leave the other set's loads
+        // in flight.  An odd last tile gets a copy of the body of its own.)
+        int g = g_begin;
+        for (; g + 1 < g_end; g += 2) {
+            body(g, std::integral_constant<int, 0>{});
+            body(g + 1, std::integral_constant<int, 1>{});
+        }
+        if (g < g_end) body(g, std::integral_constant<int, 0>{});
+    } else {
+        for (int g = g_begin; g < g_end; ++g) {
+            const TileUni uc = un; // the tile computed in this iteration (its loads are in flight or done)
+            const int i = g - chunk_base;
+            // The description and the addresses of the next tile come first, while this tile's data is
+            // still on its way: the time between its arrival and the next loads is time in which this
+            // wave has nothing in flight.
+            TileBase nb;
+            if (g + 1 < g_end) {
+                const int nbuf = (i + 1 == kInfoChunk) ? buf ^ 1 : buf;
+                un = read_info(nbuf, (i + 1) & (kInfoChunk - 1));
+                nb = tile_base(un);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+            info_traffic(i);
+            const float score_scale = score_scale_of(uc);
+            if (uc.flags & 1) open_piece(uc);
+
+            // ================= one tile =================
+            const int tile_tok0 = uc.t * kTileTok;
+            const bool ragged = tile_tok0 + kTileTok > uc.tok_end; // wave-uniform
+            wave_lds_sync(); // transposed reads of the previous tile come before V is overwritten
+            // (the masked variant sits behind a wave-uniform branch: written as one predicated sequence it costs
+            // eight register moves and an exec-mask round trip per row on every tile, between the arrival of a
+            // tile and the next loads)
+            if (!ragged) {
+#pragma unroll
+                for (int w = 0; w < 8; ++w)
+                    *reinterpret_cast<uint4*>(v_lds + (4 * w + j) * kVRowBytes + n * 16) = vreg[w];
+            } else {
+#pragma unroll
+                for (int w = 0; w < 8; ++w) {
+                    uint4 v = vreg[w];
+                    if (tile_tok0 + 4 * w + j >= uc.tok_end) v = make_uint4(0, 0, 0, 0); // 0 * garbage must be 0
+                    *reinterpret_cast<uint4*>(v_lds + (4 * w + j) * kVRowBytes + n * 16) = v;
+                }
+            }
+            // The K rows are contracted straight out of their landing registers and the next tile's loads go
+            // out right behind the eight score instructions (which have read their operands by then).
+            f32x4_t s[2];
+            scores(kreg, s);
+            __builtin_amdgcn_sched_barrier(0); // the loads below overwrite the operands of the instructions above
+            if (g + 1 < g_end) {
+                if (i + 1 == kInfoChunk) { chunk_base += kInfoChunk; buf ^= 1; }
+                if (un.flags & 1) issue_q(un); // next tile opens a new piece
+                issue_loads(nb);
+            }
+            softmax_pv(uc, s, score_scale);
         }
     }
 }
@@ -868,10 +932,12 @@ template <bool BF16, typename OT, bool ROPE_Q, bool KV8>
 static void launch_mfma_k(const DecodePlan* p, const MfmaDecodeArgs& a, hipStream_t s) {
     if (p->mfma_streaming)
         hipLaunchKernelGGL((decode_mfma_kernel<BF16, OT, ROPE_Q, KV8, true>), dim3(p->mfma_slots), dim3(64), 0, s, a,
-                           (const char*)a.q, a.k_data, a.v_data, a.indices, a.pieces, a.tiles, a.heads);
+                           (const char*)a.q, a.k_data, a.v_data, a.indices, a.pieces, a.tiles, a.heads, a.k_scale,
+                           a.v_scale);
     else
         hipLaunchKernelGGL((decode_mfma_kernel<BF16, OT, ROPE_Q, KV8, false>), dim3(p->mfma_slots), dim3(64), 0, s, a,
-                           (const char*)a.q, a.k_data, a.v_data, a.indices, a.pieces, a.tiles, a.heads);
+                           (const char*)a.q, a.k_data, a.v_data, a.indices, a.pieces, a.tiles, a.heads, a.k_scale,
+                           a.v_scale);
 }
 
 template <bool BF16, typename OT>
