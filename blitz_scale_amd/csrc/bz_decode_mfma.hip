@@ -515,17 +515,18 @@ __global__ __launch_bounds__(64, 2) void decode_mfma_kernel(MfmaDecodeArgs a, co
             if (second) dB = read_info(0, 1);
             issue_loads_kv8(tile_base(dB), std::integral_constant<int, 1>{}, second);
         }
-        auto body = [&](int g, auto set_c) __attribute__((always_inline)) {
+        auto body = [&](int g, auto set_c, auto last_c) __attribute__((always_inline)) {
             constexpr int SET = decltype(set_c)::value;
+            constexpr bool LAST = decltype(last_c)::value; // the copy behind the loop: nothing left to fetch
             const TileUni uc = SET ? dB : dA;
             const int i = g - chunk_base;
             // the tile after next, which takes over this set
-            const bool more = g + 2 < g_end;
+            const bool more = !LAST && g + 2 < g_end;
             TileUni u2 = uc;
             if (more) u2 = read_info(i + 2 >= kInfoChunk ? buf ^ 1 : buf, (i + 2) & (kInfoChunk - 1));
             const TileBase nb = tile_base(u2);
             __builtin_amdgcn_sched_barrier(0);
-            info_traffic(i);
+            if (!LAST) info_traffic(i);
             const float score_scale = score_scale_of(uc);
             if (uc.flags & 1) open_piece(uc);
 
@@ -556,13 +557,15 @@ __global__ __launch_bounds__(64, 2) void decode_mfma_kernel(MfmaDecodeArgs a, co
 #pragma unroll
                 for (int ks = 0; ks < 4; ++ks) kcur[u][ks] = fp8x8_to_op<BF16>(kreg[u][2 * SET + (ks >> 1)], ks & 1);
             // the set is free: q rows of the next tile's piece (one tile ahead), K/V of the tile after next
-            if (g + 1 < g_end) {
-                const TileUni& u1 = SET ? dA : dB;
-                if (u1.flags & 1) issue_q(u1);
+            if constexpr (!LAST) {
+                if (g + 1 < g_end) {
+                    const TileUni& u1 = SET ? dA : dB;
+                    if (u1.flags & 1) issue_q(u1);
+                }
+                issue_loads_kv8(nb, set_c, more);
+                if (SET) dB = u2; else dA = u2;
+                if (i + 1 == kInfoChunk) { chunk_base += kInfoChunk; buf ^= 1; }
             }
-            issue_loads_kv8(nb, set_c, more);
-            if (SET) dB = u2; else dA = u2;
-            if (i + 1 == kInfoChunk) { chunk_base += kInfoChunk; buf ^= 1; }
             f32x4_t s[2];
             scores(kcur, s);
             softmax_pv(uc, s, score_scale);
@@ -572,10 +575,10 @@ __global__ __launch_bounds__(64, 2) void decode_mfma_kernel(MfmaDecodeArgs a, co
         // in flight.  An odd last tile gets a copy of the body of its own.)
         int g = g_begin;
         for (; g + 1 < g_end; g += 2) {
-            body(g, std::integral_constant<int, 0>{});
-            body(g + 1, std::integral_constant<int, 1>{});
+            body(g, std::integral_constant<int, 0>{}, std::false_type{});
+            body(g + 1, std::integral_constant<int, 1>{}, std::false_type{});
         }
-        if (g < g_end) body(g, std::integral_constant<int, 0>{});
+        if (g < g_end) body(g, std::integral_constant<int, 0>{}, std::true_type{});
     } else {
         for (int g = g_begin; g < g_end; ++g) {
             const TileUni uc = un; // the tile computed in this iteration (its loads are in flight or done)
