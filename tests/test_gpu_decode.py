@@ -240,3 +240,31 @@ def test_more_than_sixteen_q_heads_per_kv_head(Hq, Hkv, kv_dtype):
     if kv_dtype is None:
         got32 = dev.decode(BZ_F32, BZ_ROPE_NONE)
         assert np.abs(got32 - ref).max() <= 2e-5
+
+
+@pytest.mark.parametrize("case", ["short_pieces", "chunk_crossing"])
+@pytest.mark.parametrize("rope_mode", [BZ_ROPE_NONE, BZ_ROPE_Q_ONLY])
+def test_e4m3_pool_with_several_tiles_per_wave_slot(case, rope_mode):
+    """The one-byte-pool kernel keeps two tiles in flight per wave (two register sets taking turns).  Regimes of
+    that pipeline on 256 compute units (2 048 wave slots):
+      short_pieces    700 sequences of 1..200 tokens on 4 kv heads: ~4 or 5 tiles per slot (odd and even counts),
+                      pieces of one to seven tiles, so consecutive tiles open new pieces and the q rows of a
+                      piece are fetched one tile ahead several times in a row;
+      chunk_crossing  150 sequences of 100..3 000 tokens on 8 kv heads: ~29 tiles per slot, i.e. the tile
+                      descriptions come in more than one batch of 16 and ragged last tiles sit anywhere."""
+    rng = np.random.default_rng(77 if case == "short_pieces" else 78)
+    if case == "short_pieces":
+        ctx, Hq, Hkv = rng.integers(1, 201, size=700).tolist(), 16, 4
+    else:
+        ctx, Hq, Hkv = rng.integers(100, 3001, size=150).tolist(), 32, 8
+    p = DecodeProblem(500 + len(ctx), ctx, Hq, Hkv, 128, 16, BZ_BF16, kv_dtype=BZ_E4M3)
+    ref = oracle.batch_decode(p.q, p.dtype, p.oracle_kv(), p.Hq, rope_mode=rope_mode, rope_theta=5e5, k_scale=p.k_scale,
+                              v_scale=p.v_scale, parallel=True)
+    dev = DeviceDecode(p)
+    info = dev.plan(0)
+    tiles = sum((c + 31) // 32 for c in ctx) * Hkv
+    assert info["workgroups"] >= 2000 and tiles / info["workgroups"] > (3 if case == "short_pieces" else 20)
+    got32 = dev.decode(BZ_F32, rope_mode, 5e5)
+    assert np.abs(got32 - ref).max() <= (2e-5 if rope_mode == BZ_ROPE_NONE else 1e-4)
+    got = dev.decode(None, rope_mode, 5e5)
+    assert (np.abs(got - ref) <= ulp_tol(ref, p.dtype, 3e-2)).all()

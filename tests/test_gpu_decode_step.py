@@ -109,6 +109,14 @@ def test_step_e4m3_pool():
     run_step(p, split_tokens=1024)
 
 
+def test_step_e4m3_pool_with_several_tiles_per_wave_slot():
+    """700 short sequences on 4 kv heads: four or five tiles per wave slot, pieces of one to seven tiles, so the
+    two-tiles-in-flight pipeline of the one-byte-pool kernel runs with odd and even counts and opens pieces on
+    consecutive tiles, in step mode (every piece leaves a partial, the newest token is left to the second kernel)."""
+    ctx = np.random.default_rng(79).integers(1, 201, size=700).tolist()
+    run_step(DecodeProblem(305, ctx, 16, 4, 128, 16, BZ_BF16, kv_dtype=BZ_E4M3), split_tokens=2048)
+
+
 def test_step_without_rope_and_with_many_partials():
     run_step(DecodeProblem(303, [20000, 77], 32, 8, 128, 16, BZ_BF16), split_tokens=2048, rope=False)
 
