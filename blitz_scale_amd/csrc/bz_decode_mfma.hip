@@ -1014,9 +1014,10 @@ static int launch_step_finish(const DecodePlan* p, const StepFinishArgs& a, hipS
             hipLaunchKernelGGL((decode_step_finish_kernel<QT, PT, OT, 1, 2>), dim3(p->mfma_units, (G + 1) / 2), dim3(32, 2, 1), 0, s, a);
         else
             hipLaunchKernelGGL((decode_step_finish_kernel<QT, PT, OT, 1, 1>), dim3(p->mfma_units, G), dim3(32, 1, 1), 0, s, a);
-    } else if (p->mfma_unit_max_count <= 64) {
+    } else if (p->mfma_unit_max_count > 32 && p->mfma_unit_max_count <= 64) {
         hipLaunchKernelGGL((decode_step_finish_kernel<QT, PT, OT, 4, 2>), dim3(p->mfma_units, (G + 1) / 2), dim3(32, 2, 4), 0, s, a);
-    } else {
+    } else { // 17..32 partials: one batch of four per slice, a single round of loads; more than 64: eight slices as well
+
         hipLaunchKernelGGL((decode_step_finish_kernel<QT, PT, OT, 8, 2>), dim3(p->mfma_units, (G + 1) / 2), dim3(32, 2, 8), 0, s, a);
     }
     BZ_LAUNCH_CHECK();
