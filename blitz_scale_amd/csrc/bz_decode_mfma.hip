@@ -10,7 +10,8 @@
 //   V rows   : global -> VGPR -> LDS (row stride 288 B), read back with the transposing LDS load
 //              (ds_read_b64_tr_b16) as MFMA B operands (contraction over tokens)
 //   softmax  : online, 8 scores per lane, row max / sum over the 4 lane groups with two shuffles
-// The loads of tile t+1 are issued before the arithmetic of tile t.
+// The loads of tile t+1 are issued before the arithmetic of tile t; with one-byte pools, whose tiles need half
+// the landing registers, two tiles are in flight per wave.
 #include <cmath>
 #include <type_traits>
 
@@ -140,7 +141,7 @@ template <bool BF16> __device__ __forceinline__ uint4 fp8x8_to_op(const uint4& r
 //
 // Under load a dependent memory round trip costs several microseconds, so the kernel has none in its
 // steady state: the planner lists every tile of a wave slot as a 16-byte record, and the wave fetches
-// the records, the page ids they point at and the metadata of their pieces for 32 tiles at a time
+// the records, the page ids they point at and the metadata of their pieces for 16 tiles at a time
 // (one lane per tile) well before they are needed; inside the tile loop everything wave-uniform comes
 // out of those registers with v_readlane.  The K/V loads of tile g+1 and the q rows of the next piece
 // are issued before the arithmetic of tile g.
