@@ -81,6 +81,71 @@ def test_prefill_random_shapes(case):
     assert (np.abs(got - ref) <= ulp_tol(ref, dtype)).all(), (case, float(np.abs(got - ref).max()))
 
 
+@pytest.mark.parametrize("case", range(12))
+def test_prefill_random_shapes_q_rotated_in_registers(case):
+    """BZ_ROPE_Q_ONLY of the prefill call: q is rotated on its way into the operand registers (angle table in the
+    float workspace), k is taken as it is; the checker does the same in fp32.  Float workspaces with and without
+    room for the table (without: q is rotated in place by a separate kernel first)."""
+    rng = np.random.default_rng(9700 + case)
+    B = int(rng.integers(1, 7))
+    Hkv = int(rng.choice([1, 2, 4]))
+    G = int(rng.choice([1, 2, 3, 4, 7, 8]))
+    dtype = int(rng.choice([BZ_F16, BZ_F16, BZ_BF16]))
+    causal = bool(rng.random() < 0.75)
+    theta = float(rng.choice([1e4, 5e5]))
+    lens = [max(1, x) for x in draw_lens(rng, B, 900)]
+    pf = Prefill(9750 + case, lens, Hkv * G, Hkv, 128, dtype)
+    roomy = bool(rng.random() < 0.75)
+    pf.float_ws = torch.empty((1 << 20) if roomy else 256, dtype=torch.uint8, device="cuda")
+    got = pf.run(causal=causal, rope_mode=BZ_ROPE_Q_ONLY, theta=theta)
+    assert np.array_equal(pf.k_after, pf.k)
+    assert not np.isnan(got).any()
+    if roomy:
+        assert np.array_equal(pf.q_after, pf.q)
+        ref = oracle.batch_prefill_ragged(pf.q, pf.k, pf.v, dtype, pf.indptr, Hkv * G, Hkv, 128, causal=causal, rope="q",
+                                          rope_theta=theta, parallel=True)
+        # (bf16: the one rounding of the rotated, scaled q row to 8 significant bits moves the logits by ~1e-2)
+        tol = ulp_tol(ref, dtype) if dtype == BZ_F16 else np.maximum(ulp_tol(ref, dtype), 2e-2)
+    else:
+        ref = oracle.batch_prefill_ragged(pf.q_after, pf.k, pf.v, dtype, pf.indptr, Hkv * G, Hkv, 128, causal=causal,
+                                          parallel=True)
+        tol = ulp_tol(ref, dtype)
+    assert (np.abs(got - ref) <= tol).all(), (case, float(np.abs(got - ref).max()))
+
+
+@pytest.mark.parametrize("case", range(16))
+def test_decode_step_random_shapes(case):
+    """The one-call decode step (append + attention) on random shapes: matrix-core path and the fallback, e4m3
+    pools, both layouts, with and without RoPE; checked against the two-call sequence and the checker."""
+    from test_gpu_decode_step import run_step
+    rng = np.random.default_rng(9300 + case)
+    B = int(rng.integers(1, 41))
+    Hkv = int(rng.choice([1, 2, 4, 8]))
+    G = int(rng.choice([1, 2, 3, 4, 6, 8, 12, 16, 32]))
+    D = int(rng.choice([64, 128, 128, 128, 128]))
+    P = int(rng.choice([8, 16, 16, 32, 64]))
+    dtype = int(rng.choice([BZ_F16, BZ_BF16]))
+    kv_dtype = BZ_E4M3 if rng.random() < 0.3 else dtype
+    layout = int(rng.choice([BZ_LAYOUT_HND, BZ_LAYOUT_NHD]))
+    split_tokens = int(rng.choice([0, 64, 256, 2048]))
+    ctx = [max(1, x) for x in draw_lens(rng, B, 2500)]  # the newest token included
+    if rng.random() < 0.3:
+        ctx[int(rng.integers(0, B))] = 0               # a sequence without pages
+    if not any(ctx):
+        ctx[0] = 40
+    p = DecodeProblem(9400 + case, ctx, Hkv * G, Hkv, D, P, dtype, kv_dtype=kv_dtype, layout=layout)
+    parts = (G + 15) // 16
+    while parts < G and G % parts:
+        parts += 1
+    mfma = D == 128 and P % 16 == 0 and parts <= 8
+    if mfma:
+        dev = DeviceDecode(p)
+        dev.plan(split_tokens)
+        assert len(dev.handler.host_schedule(7)) == int((p.ctx > 0).sum()) * Hkv * parts
+    run_step(p, split_tokens=split_tokens, rope=bool(rng.random() < 0.7), theta=float(rng.choice([1e4, 5e5])),
+             expect_units=False)
+
+
 @pytest.mark.parametrize("case", range(6))
 def test_store_and_append_random_shapes(case):
     """Prefill store followed by a decode append into the same table: page placement bit-exact."""
