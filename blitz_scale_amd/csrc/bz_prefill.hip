@@ -133,7 +133,7 @@ __global__ __launch_bounds__(256, 2) void prefill_kernel(PrefillArgs a, const ch
                                                          const char* __restrict__ k_ptr,
                                                          const char* __restrict__ v_ptr) {
     using M = PfMma<BF16>;
-    constexpr bool QSCALED = !BF16 || ROPE_Q; // q carries sm_scale * log2(e) (see the prologue)
+    constexpr bool QSCALED = ROPE_Q; // q carries sm_scale * log2(e) (see the prologue)
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
 
     const PrefillItem it = a.items[blockIdx.x];
@@ -175,19 +175,12 @@ __global__ __launch_bounds__(256, 2) void prefill_kernel(PrefillArgs a, const ch
                     pf_u4(qreg[ks], w) = M::pack2(x0 * a.sm_scale_log2, x1 * a.sm_scale_log2);
                     pf_u4(qreg[ks + 4], w) = M::pack2(y0 * a.sm_scale_log2, y1 * a.sm_scale_log2);
                 }
-        } else if constexpr (QSCALED) {
-            // The q rows carry the softmax scale (times log2 e): the scores then come out of the matrix pipe as
-            // base-2 logits and go into exp2 as they are, one vector instruction less per score.  (Not for
-            // bf16 rows that arrive rotated: a second rounding to 8 significant bits would cost a factor of
-            // two in the error of every logit; there the scale is applied to the score instead.)
-#pragma unroll
-            for (int ks = 0; ks < 8; ++ks)
-#pragma unroll
-                for (int w = 0; w < 4; ++w) {
-                    const uint32_t xw = pf_u4(qreg[ks], w);
-                    pf_u4(qreg[ks], w) = M::pack2(M::lo(xw) * a.sm_scale_log2, M::hi(xw) * a.sm_scale_log2);
-                }
         }
+        // Rows rotated here carry the softmax scale (times log2 e) in their one rounding: the scores then come
+        // out of the matrix pipe as base-2 logits and go into exp2 as they are, one vector instruction less per
+        // score.  Rows that arrive as they are keep their bits -- a second rounding would move a logit of
+        // magnitude 30 by 30 * 2^-12 (f16) or 30 * 2^-9 (bf16), visibly more than the stated tolerance -- and the
+        // scale is applied to the score instead.
     }
 
     const int kv_limit = a.causal ? min(L, it.q0 + kBM) : L; // tokens any row of this workgroup can see

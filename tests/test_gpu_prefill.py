@@ -103,6 +103,48 @@ def test_rope_inside_the_call(dtype, float_ws_bytes):
         assert np.array_equal(pf2.q_after, pf2.q) and np.array_equal(pf2.k_after, pf2.k)
 
 
+@pytest.mark.parametrize("dtype", [BZ_F16, BZ_BF16])
+@pytest.mark.parametrize("pattern", ["rising", "falling", "spikes"])
+@pytest.mark.parametrize("rope_mode", [BZ_ROPE_NONE, BZ_ROPE_Q_ONLY])
+def test_logits_with_a_large_dynamic_range(dtype, pattern, rope_mode):
+    """The kernel keeps one reference maximum per row and moves it only when a score exceeds it by 2^15 or more
+    (probabilities are computed on that assumption first and again if it did not hold).  Here the K rows are
+    scaled along the sequence so that the row maxima climb by far more than that from tile to tile (rising), sit
+    in the first tile with everything after it far below (falling), or jump at a few isolated tokens (spikes);
+    the logits span about +-40 in base-2 units."""
+    lens = [700, 130, 64, 1000]
+    pf = Prefill(220, lens, 8, 2, 128, dtype)
+    rng = np.random.default_rng(221)
+    k = wl.to_f32(pf.k, dtype)
+    for b in range(len(lens)):
+        lo, hi = int(pf.indptr[b]), int(pf.indptr[b + 1])
+        pos = np.arange(hi - lo, dtype=np.float32) / max(1, hi - lo - 1)
+        if pattern == "rising":
+            scale = 0.5 + 7.5 * pos
+        elif pattern == "falling":
+            scale = 8.0 - 7.5 * pos
+        else:
+            scale = np.where(rng.random(hi - lo) < 0.02, 9.0, 0.7).astype(np.float32)
+        k[lo:hi] *= scale[:, None, None]
+    pf.k = wl.to_bits(k, dtype)
+    got = pf.run(causal=True, rope_mode=rope_mode, theta=1e4)
+    ref = oracle.batch_prefill_ragged(pf.q, pf.k, pf.v, dtype, pf.indptr, 8, 2, 128, causal=True,
+                                      rope="q" if rope_mode == BZ_ROPE_Q_ONLY else False, rope_theta=1e4, parallel=True)
+    assert not np.isnan(got).any()
+    err = np.abs(got - ref)
+    if rope_mode == BZ_ROPE_NONE:
+        # q and k enter the matrix cores with the bits the checker reads: the stated bar.  Rows that attend to a
+        # single token reach |o| > 4 here, where half an f16 step is 1.95e-3 by itself; the probabilities enter
+        # the second contraction rounded to f16 (relative 2^-12), which is allowed for on top.
+        assert (err <= ulp_tol(ref, dtype) + 2.0 ** -12 * np.abs(ref)).all(), float(err.max())
+    else:
+        # the rotated q row is rounded to the storage type on its way into the matrix cores (the checker keeps it
+        # in fp32): a logit of magnitude 30 moves by 30 * 2^-12 (f16) or 30 * 2^-9 (bf16), and the output with
+        # it; the bounds catch a wrong maximum or a lost tile, which show up as errors of order one or NaN
+        big, med = (2e-2, 2e-3) if dtype == BZ_F16 else (0.35, 2e-2)
+        assert err.max() <= big and np.median(err) <= med, (float(err.max()), float(np.median(err)))
+
+
 def test_prefill_then_store_then_decode_is_consistent():
     """Row i of the prefill output equals a decode over the first i+1 cached tokens (GPU against GPU and
     against the checker): ties the three kernels of the path together."""
