@@ -268,3 +268,15 @@ def test_e4m3_pool_with_several_tiles_per_wave_slot(case, rope_mode):
     assert np.abs(got32 - ref).max() <= (2e-5 if rope_mode == BZ_ROPE_NONE else 1e-4)
     got = dev.decode(None, rope_mode, 5e5)
     assert (np.abs(got - ref) <= ulp_tol(ref, p.dtype, 3e-2)).all()
+
+
+@pytest.mark.parametrize("dtype,kv_dtype", [(BZ_F16, None), (BZ_BF16, None), (BZ_BF16, BZ_E4M3)])
+def test_logits_with_a_large_dynamic_range(dtype, kv_dtype):
+    """q rows eight times the usual size: logits of +-40 base-2 units, rows that attend to one or two tokens, and
+    split-K partials whose log-sum-exps differ by tens of units (two-call path with the combine kernel, and the
+    one-call step with its finishing kernel)."""
+    from test_gpu_decode_step import run_step
+    p = DecodeProblem(60, [3000, 40, 700, 1, 5000, 129], 32, 8, 128, 16, dtype, kv_dtype=kv_dtype)
+    p.q = wl.to_bits(wl.to_f32(p.q, dtype) * np.float32(8.0), dtype)
+    check(p, split_tokens=512, f32_tol=2e-5, parallel=True)  # matrix-core kernel and general kernel
+    run_step(p, split_tokens=512, rope=False)
