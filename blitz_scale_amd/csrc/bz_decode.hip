@@ -8,6 +8,8 @@
 #include <vector>
 #include <new>
 
+#include <type_traits>
+
 #include "bz_common.hpp"
 #include "bz_decode_plan.hpp"
 
@@ -45,10 +47,24 @@ struct DecodeArgs {
     uint32_t group_div; // workgroups per kv head: a group that is no instantiated size is split into equal parts
     int rope_mode;
     float sm_scale_log2; // sm_scale * log2(e)
+    const float2* rope_table; // BZ_ROPE_FULL: (cos, sin) per [position][pair] or nullptr (angles computed on the fly)
     RopeFreqs freqs;
 };
 
-template <typename QT, typename KVT, typename OT, int D, int G>
+// (cos, sin) of position * frequency i for positions [0, positions): the expression the kernels evaluate on the
+// fly, evaluated once per plan instead of once per cached token, kv head and step.
+__global__ __launch_bounds__(256) void decode_rope_table_kernel(float2* table, uint32_t positions, uint32_t pairs,
+                                                                RopeFreqs freqs) {
+    const uint32_t i = blockIdx.x * 256 + threadIdx.x;
+    if (i >= positions * pairs) return;
+    float s, c;
+    sincosf((float)(i / pairs) * freqs.f[i % pairs], &s, &c);
+    table[i] = make_float2(c, s);
+}
+
+// TABLE: BZ_ROPE_FULL with the angles of the cached K rows taken from a.rope_table (an instantiation of its own,
+// so that the registers the table rows travel through do not cost the other modes their occupancy).
+template <typename QT, typename KVT, typename OT, int D, int G, bool TABLE = false>
 __global__ __launch_bounds__(256) void decode_general_kernel(DecodeArgs a) {
     using Geo = RowGeom<KVT, D>;
     constexpr int LANES = Geo::kLanes;
@@ -111,6 +127,15 @@ __global__ __launch_bounds__(256) void decode_general_kernel(DecodeArgs a) {
     const size_t esz = sizeof(KVT);
     const size_t head_off = ((size_t)kvh * a.stride_h + (size_t)lane_in_row * 8) * esz;
 
+    // BZ_ROPE_FULL rotates every cached K row at its own position.  Evaluating sincosf per element makes the
+    // kernel compute-bound several times over, so the angles come from a table when the plan has room for one
+    // (64 bytes per lane and token, fetched TU tokens ahead; the groups of eight q heads have no registers left
+    // for that and keep the on-the-fly evaluation).
+    constexpr int TU = G <= 2 ? 4 : 2;
+    static_assert(!TABLE || G <= 4, "no registers for the table rows beside eight q heads");
+    constexpr bool table_rope = TABLE;
+    const float4* cs_lane = reinterpret_cast<const float4*>(a.rope_table) + (lane_in_row % (LANES / 2)) * 4;
+
     for (int base = tok_begin; base < tok_end; base += TOK * UNROLL) {
         Vec8<KVT> kv[UNROLL], vv[UNROLL];
         bool valid[UNROLL];
@@ -127,6 +152,17 @@ __global__ __launch_bounds__(256) void decode_general_kernel(DecodeArgs a) {
             kv[u].load_nt(a.k_data + off); // read once per launch (+2 to 3 % over plain loads)
             vv[u].load_nt(a.v_data + off);
         }
+        float4 cs[TABLE ? TU : 1][4]; // (cos, sin) of this lane's eight pairs at the positions of TU tokens
+        auto fetch_cs = [&](int u) {
+            const int jc = valid[u] ? jj[u] : tok_begin;
+            const float4* row = cs_lane + (size_t)jc * (D / 4); // D/2 pairs of 8 bytes = D/4 float4 per position
+#pragma unroll
+            for (int i = 0; i < 4; ++i) cs[u % TU][i] = row[i];
+        };
+        if constexpr (TABLE) {
+#pragma unroll
+            for (int u = 0; u < TU; ++u) fetch_cs(u);
+        }
 #pragma unroll
         for (int u = 0; u < UNROLL; ++u) {
             float kf[8], vf[8];
@@ -134,12 +170,22 @@ __global__ __launch_bounds__(256) void decode_general_kernel(DecodeArgs a) {
             vv[u].to_float(vf);
             if (a.rope_mode == BZ_ROPE_FULL) {
                 const bool upper = lane_in_row >= LANES / 2;
+                float cv[8], sv[8];
+                if constexpr (TABLE) {
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) {
+                        const float4 t = cs[u % TU][i];
+                        cv[2 * i] = t.x; sv[2 * i] = t.y; cv[2 * i + 1] = t.z; sv[2 * i + 1] = t.w;
+                    }
+                    if (u + TU < UNROLL) fetch_cs(u + TU);
+                }
 #pragma unroll
                 for (int e = 0; e < 8; ++e) {
                     const float other = __shfl_xor(kf[e], LANES / 2, 64);
                     const int fi = (lane_in_row % (LANES / 2)) * 8 + e;
                     float s, c;
-                    sincosf((float)jj[u] * a.freqs.f[fi], &s, &c);
+                    if constexpr (TABLE) { c = cv[e]; s = sv[e]; }
+                    else sincosf((float)jj[u] * a.freqs.f[fi], &s, &c);
                     float lo_r, hi_r;
                     rope_pair(upper ? other : kf[e], upper ? kf[e] : other, c, s, lo_r, hi_r);
                     kf[e] = upper ? hi_r : lo_r;
@@ -260,6 +306,17 @@ __global__ void decode_zero_rows_kernel(const int32_t* empty_seqs, void* out, ui
 // ------------------------------------------------------------------------------------------
 template <typename QT, typename KVT, typename OT, int D>
 static int launch_general_g(const DecodeArgs& a, int G, dim3 grid, hipStream_t s) {
+    if constexpr (std::is_same<QT, KVT>::value) {
+        if (a.rope_mode == BZ_ROPE_FULL && a.rope_table && G <= 4) { // angles from the table
+            switch (G) {
+                case 1: hipLaunchKernelGGL((decode_general_kernel<QT, KVT, OT, D, 1, true>), grid, dim3(256), 0, s, a); break;
+                case 2: hipLaunchKernelGGL((decode_general_kernel<QT, KVT, OT, D, 2, true>), grid, dim3(256), 0, s, a); break;
+                default: hipLaunchKernelGGL((decode_general_kernel<QT, KVT, OT, D, 4, true>), grid, dim3(256), 0, s, a); break;
+            }
+            BZ_LAUNCH_CHECK();
+            return 0;
+        }
+    }
     switch (G) {
         case 1: hipLaunchKernelGGL((decode_general_kernel<QT, KVT, OT, D, 1>), grid, dim3(256), 0, s, a); break;
         case 2: hipLaunchKernelGGL((decode_general_kernel<QT, KVT, OT, D, 2>), grid, dim3(256), 0, s, a); break;
@@ -351,6 +408,7 @@ static int batch_decode_impl(DecodePlan* p, const void* q, int q_dtype, const bz
     a.page_size = kv->page_size; a.num_qo_heads = num_qo_heads; a.num_kv_heads = kv->num_kv_heads;
     a.group_div = 1;
     a.rope_mode = rope_mode;
+    a.rope_table = nullptr;
     if (!(sm_scale > 0.f)) sm_scale = 1.0f / sqrtf((float)D);
     a.sm_scale_log2 = sm_scale * 1.4426950408889634f;
     a.freqs = make_rope_freqs(D, rope_theta > 0.f ? rope_theta : 1e4f);
@@ -361,6 +419,7 @@ static int batch_decode_impl(DecodePlan* p, const void* q, int q_dtype, const bz
             rc = decode_fast_path(p, q, out, lse, q_dtype, out_dtype, rope_mode, a.sm_scale_log2, a.freqs, kv,
                                   num_qo_heads, k_scale, v_scale, bufs.mfma_part_o, bufs.mfma_part_lse, false, s);
         if (rc == 0) {
+            if (!bufs_or_null) p->rope_table_valid = false; // its partials share the workspace with the angle table
             // the MFMA path brings its own combine; only empty sequences are left to do
             if (p->num_empty > 0) {
                 const uint32_t row = num_qo_heads * D;
@@ -377,6 +436,25 @@ static int batch_decode_impl(DecodePlan* p, const void* q, int q_dtype, const bz
             int Gk = 8;
             while (G % Gk) Gk >>= 1;
             a.group_div = (uint32_t)(G / Gk);
+            // kRoPELlama on a raw-K cache: the angle table behind the general partials of the plan's own float
+            // workspace, when it fits (512 bytes per position at head_dim 128)
+            if (rope_mode == BZ_ROPE_FULL && !bufs_or_null && p->max_seq_len > 0) {
+                const size_t off = (p->general_part_bytes + 255) / 256 * 256;
+                const size_t tbytes = (size_t)p->max_seq_len * (size_t)(D / 2) * sizeof(float2);
+                if (off + tbytes <= p->float_buffer_bytes) {
+                    float2* table = reinterpret_cast<float2*>(reinterpret_cast<char*>(p->part_o) + off);
+                    const float theta = rope_theta > 0.f ? rope_theta : 1e4f;
+                    if (!p->rope_table_valid || p->rope_table_theta != theta) {
+                        const uint32_t n = p->max_seq_len * (uint32_t)(D / 2);
+                        hipLaunchKernelGGL(decode_rope_table_kernel, dim3((n + 255) / 256), dim3(256), 0, s, table,
+                                           p->max_seq_len, (uint32_t)(D / 2), a.freqs);
+                        BZ_LAUNCH_CHECK();
+                        p->rope_table_valid = true;
+                        p->rope_table_theta = theta;
+                    }
+                    a.rope_table = table;
+                }
+            }
             dim3 grid(p->num_segments, kv->num_kv_heads * a.group_div);
             if (p->time_start) BZ_CHECK_HIP(hipEventRecord(p->time_start, s));
             if (q_dtype == BZ_F16)
@@ -474,6 +552,7 @@ extern "C" int bz_decode_step(bz_decode_plan_t* plan_, const void* q, int q_dtyp
         const RopeFreqs freqs = make_rope_freqs(D, rope_theta > 0.f ? rope_theta : 1e4f);
         rc = decode_step_fast_path(p, q, k_new, v_new, out, lse, q_dtype, out_dtype, rope, scale * 1.4426950408889634f,
                                    freqs, kv, num_qo_heads, k_scale, v_scale, s);
+        if (rc == 0) p->rope_table_valid = false; // the step's partials share the workspace with the angle table
         if (rc == 0 && p->num_empty > 0) { // sequences without pages: nothing to append, zero rows
             const uint32_t row = num_qo_heads * D;
             if (out_dtype == BZ_F32) launch_zero<float>(p, out, row, s);

@@ -351,6 +351,13 @@ extern "C" int bz_decode_plan(bz_decode_plan_t* plan_, void* float_buffer, size_
     p->combos_d = (const DecodeCombine*)((char*)int_buffer + seg_bytes);
     p->empty_d = (const int32_t*)((char*)int_buffer + seg_bytes + combo_bytes);
     p->float_buffer_bytes = float_buffer_bytes;
+    p->general_part_bytes = part_o_bytes + part_lse_bytes;
+    p->rope_table_valid = false;
+    p->max_seq_len = 0;
+    for (uint32_t b = 0; b < batch_size; ++b) {
+        const int32_t np = indptr_h[b + 1] - indptr_h[b];
+        if (np > 0) p->max_seq_len = std::max<uint32_t>(p->max_seq_len, (uint32_t)(np - 1) * page_size + (uint32_t)last_page_len_h[b]);
+    }
     p->part_o = (float*)float_buffer;
     p->part_lse = (float*)((char*)float_buffer + part_o_bytes);
     p->batch_size = batch_size; p->num_qo_heads = num_qo_heads; p->num_kv_heads = num_kv_heads;

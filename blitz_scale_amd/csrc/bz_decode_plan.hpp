@@ -123,6 +123,13 @@ struct DecodePlan {
     size_t float_buffer_bytes = 0;              // size of the float workspace given to plan()
     float* mfma_part_o = nullptr;
     float* mfma_part_lse = nullptr;
+    // general kernel, BZ_ROPE_FULL: (cos, sin) of position * frequency for every position of the planned table,
+    // kept in the float workspace behind the general kernel's partials and filled by the first such call after
+    // a plan() (any call that puts matrix-core partials into the workspace invalidates it)
+    uint32_t max_seq_len = 0;       // longest sequence of the planned table
+    size_t general_part_bytes = 0;  // bytes of the general kernel's partials at the start of the float workspace
+    bool rope_table_valid = false;
+    float rope_table_theta = 0.f;
     // host scratch of plan(), kept between calls so that a step's plan neither allocates nor faults in
     // fresh pages (the schedule of a large batch is around a megabyte)
     std::vector<DecodeSegment> h_segs;

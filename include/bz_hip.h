@@ -150,6 +150,9 @@ int bz_decode_plan_set_timing_events(bz_decode_plan_t* plan, void* start_event, 
  * sm_scale <= 0 selects 1/sqrt(head_dim) (the default the reference never overrides).
  * k_scale / v_scale: device fp32 [num_kv_heads] dequantisation factors for an e4m3 pool
  * (NULL = 1).  lse: optional device fp32 [batch, num_qo_heads] (reference passes nullptr).
+ * BZ_ROPE_FULL (raw K in the cache, the reference's kRoPELlama): the first such call after a plan builds a table
+ * of angles, 4 * head_dim bytes per position of the longest sequence, in the plan's float workspace behind the
+ * split-K partials when there is room (it is only faster with it).
  */
 int bz_batch_decode(bz_decode_plan_t* plan, const void* q, int q_dtype, const bz_paged_kv_t* kv, void* out,
                     int out_dtype, uint32_t num_qo_heads, int rope_mode, float rope_theta, float sm_scale,

@@ -12,6 +12,7 @@ import pytest
 import torch
 
 import oracle
+from blitz_scale_amd import kernel as K
 from blitz_scale_amd import workloads as wl
 from blitz_scale_amd._lib import (BZ_BF16, BZ_E4M3, BZ_F16, BZ_F32, BZ_LAYOUT_HND, BZ_LAYOUT_NHD, BZ_ROPE_FULL,
                                   BZ_ROPE_NONE, BZ_ROPE_Q_ONLY)
@@ -280,3 +281,28 @@ def test_logits_with_a_large_dynamic_range(dtype, kv_dtype):
     p.q = wl.to_bits(wl.to_f32(p.q, dtype) * np.float32(8.0), dtype)
     check(p, split_tokens=512, f32_tol=2e-5, parallel=True)  # matrix-core kernel and general kernel
     run_step(p, split_tokens=512, rope=False)
+
+
+@pytest.mark.parametrize("Hq,Hkv,D", [(8, 2, 128), (4, 4, 64), (16, 2, 128)])
+def test_rope_full_with_and_without_the_angle_table(Hq, Hkv, D):
+    """kRoPELlama on a raw-K cache takes the angles of the cached rows from a table in the plan's float workspace
+    when there is room behind the partials (groups of one, two and four q heads per workgroup), and evaluates
+    them on the fly otherwise (no room; groups of eight).  Same results either way, also after a call in another
+    mode has used the workspace in between."""
+    p = DecodeProblem(70 + Hq, [3, 77, 500, 2100, 64], Hq, Hkv, D, 16, BZ_F16)
+    ref = oracle.batch_decode(p.q, p.dtype, p.oracle_kv(), p.Hq, rope_mode=BZ_ROPE_FULL, rope_theta=5e5, parallel=True)
+    roomy = DeviceDecode(p)                       # 32 MiB: partials + 2100 positions x D/2 x 8 bytes fit
+    roomy.plan(256)
+    a = roomy.decode(BZ_F32, BZ_ROPE_FULL, 5e5)
+    assert np.abs(a - ref).max() <= 1e-4
+    roomy.decode(BZ_F32, BZ_ROPE_Q_ONLY, 5e5)     # matrix-core path where it applies: its partials overwrite the table
+    b = roomy.decode(BZ_F32, BZ_ROPE_FULL, 5e5)   # rebuilt
+    assert np.array_equal(a, b)
+    c = roomy.decode(BZ_F32, BZ_ROPE_FULL, 1e4)   # another base: rebuilt as well
+    ref2 = oracle.batch_decode(p.q, p.dtype, p.oracle_kv(), p.Hq, rope_mode=BZ_ROPE_FULL, rope_theta=1e4, parallel=True)
+    assert np.abs(c - ref2).max() <= 1e-4
+    need = K.BlitzBatchDecodeHandler().workspace(p.indptr, p.last_page_len, p.B, Hq, Hkv, D, 16, split_tokens=256)[0]
+    tight = DeviceDecode(p, float_ws_bytes=max(int(need), 4096))  # room for the partials only
+    tight.plan(256)
+    d = tight.decode(BZ_F32, BZ_ROPE_FULL, 5e5)
+    assert np.abs(d - ref).max() <= 1e-4 and np.abs(d - a).max() <= 2e-6
