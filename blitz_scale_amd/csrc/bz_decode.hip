@@ -62,6 +62,26 @@ __global__ __launch_bounds__(256) void decode_rope_table_kernel(float2* table, u
     table[i] = make_float2(c, s);
 }
 
+// Sum over the N (8 or 16) consecutive lanes that share a token row, left in every one of them.  Row rotations
+// and quad permutes of the DPP path (one full-rate instruction per step) where the lanes of a row are the 16
+// lanes of a DPP row; an 8-lane row needs one cross-lane read for its upper and lower half.
+template <int N> __device__ __forceinline__ float row_sum(float v) {
+    auto dpp_add = [](float x, auto ctrl) {
+        constexpr int C = decltype(ctrl)::value;
+        return x + __uint_as_float(__builtin_amdgcn_update_dpp(0u, __float_as_uint(x), C, 0xF, 0xF, false));
+    };
+    if constexpr (N == 16) {
+        v = dpp_add(v, std::integral_constant<int, 0x128>{}); // row_ror:8
+        v = dpp_add(v, std::integral_constant<int, 0x124>{}); // row_ror:4
+    } else {
+        static_assert(N == 8, "rows of 8 or 16 lanes");
+        v += __shfl_xor(v, 4, 64);
+    }
+    v = dpp_add(v, std::integral_constant<int, 0x4E>{}); // quad_perm [2,3,0,1]
+    v = dpp_add(v, std::integral_constant<int, 0xB1>{}); // quad_perm [1,0,3,2]
+    return v;
+}
+
 // TABLE: BZ_ROPE_FULL with the angles of the cached K rows taken from a.rope_table (an instantiation of its own,
 // so that the registers the table rows travel through do not cost the other modes their occupancy).
 template <typename QT, typename KVT, typename OT, int D, int G, bool TABLE = false>
@@ -163,11 +183,14 @@ __global__ __launch_bounds__(256) void decode_general_kernel(DecodeArgs a) {
 #pragma unroll
             for (int u = 0; u < TU; ++u) fetch_cs(u);
         }
+        // Scores of the UNROLL tokens first (a token's row is spread over LANES lanes: products, then a sum across
+        // the lanes of the row with DPP row rotations), then one softmax update per q head for all of them: one
+        // maximum, one rescale of the accumulators per batch instead of per token, raw v_exp_f32.
+        float sc_tok[UNROLL][G];
 #pragma unroll
         for (int u = 0; u < UNROLL; ++u) {
-            float kf[8], vf[8];
+            float kf[8];
             kv[u].to_float(kf);
-            vv[u].to_float(vf);
             if (a.rope_mode == BZ_ROPE_FULL) {
                 const bool upper = lane_in_row >= LANES / 2;
                 float cv[8], sv[8];
@@ -196,19 +219,35 @@ __global__ __launch_bounds__(256) void decode_general_kernel(DecodeArgs a) {
                 float s = 0.f;
 #pragma unroll
                 for (int e = 0; e < 8; ++e) s += q[g][e] * kf[e];
-#pragma unroll
-                for (int o = LANES / 2; o > 0; o >>= 1) s += __shfl_xor(s, o, 64);
-                s *= kscale;
-                if (valid[u]) {
-                    const float mn = fmaxf(m[g], s);
-                    const float sc = exp2f(m[g] - mn); // m = -inf on the first token gives 0
-                    const float p = exp2f(s - mn);
-                    l[g] = l[g] * sc + p;
-#pragma unroll
-                    for (int e = 0; e < 8; ++e) acc[g][e] = acc[g][e] * sc + p * vf[e];
-                    m[g] = mn;
-                }
+                s = row_sum<LANES>(s);
+                sc_tok[u][g] = valid[u] ? s * kscale : -INFINITY;
             }
+        }
+        float vf[UNROLL][8];
+#pragma unroll
+        for (int u = 0; u < UNROLL; ++u) vv[u].to_float(vf[u]);
+#pragma unroll
+        for (int g = 0; g < G; ++g) {
+            float mx = m[g];
+#pragma unroll
+            for (int u = 0; u < UNROLL; ++u) mx = fmaxf(mx, sc_tok[u][g]);
+            const float mref = fmaxf(mx, -1e30f); // finite also while nothing live has been seen: weights come out 0
+            const float sc = __builtin_amdgcn_exp2f(m[g] - mref); // m = -inf before the first live token gives 0
+            float p[UNROLL], psum = 0.f;
+#pragma unroll
+            for (int u = 0; u < UNROLL; ++u) {
+                p[u] = __builtin_amdgcn_exp2f(sc_tok[u][g] - mref); // -inf (no such token) gives 0
+                psum += p[u];
+            }
+            l[g] = l[g] * sc + psum;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                float t = acc[g][e] * sc;
+#pragma unroll
+                for (int u = 0; u < UNROLL; ++u) t += p[u] * vf[u][e];
+                acc[g][e] = t;
+            }
+            m[g] = mx;
         }
     }
 
