@@ -89,7 +89,7 @@ __global__ __launch_bounds__(256) void decode_general_kernel(DecodeArgs a) {
     using Geo = RowGeom<KVT, D>;
     constexpr int LANES = Geo::kLanes;
     constexpr int TOK = Geo::kTok;
-    constexpr int UNROLL = 4;
+    constexpr int UNROLL = G == 8 ? 2 : 4; // tokens per lane slot and register set
 
     const DecodeSegment seg = a.segments[blockIdx.x];
     const int unit = blockIdx.y;                   // G consecutive q heads, all of one kv head
@@ -156,22 +156,35 @@ __global__ __launch_bounds__(256) void decode_general_kernel(DecodeArgs a) {
     constexpr bool table_rope = TABLE;
     const float4* cs_lane = reinterpret_cast<const float4*>(a.rope_table) + (lane_in_row % (LANES / 2)) * 4;
 
-    for (int base = tok_begin; base < tok_end; base += TOK * UNROLL) {
+    // Two register sets of UNROLL tokens per lane slot take turns: the loads of the next set go out before the
+    // arithmetic of the present one.  They are issued whether or not the set has a live token (addresses are
+    // clamped to a token of the segment): with the same number of loads behind a set on every path, the waits the
+    // compiler derives for a set leave the other set's loads in flight.  (Not for single heads per workgroup,
+    // whose occupancy the second set would cost.)
+    struct TokSet {
         Vec8<KVT> kv[UNROLL], vv[UNROLL];
         bool valid[UNROLL];
         int jj[UNROLL];
+    };
+    auto issue = [&](int base, TokSet& S) __attribute__((always_inline)) {
 #pragma unroll
         for (int u = 0; u < UNROLL; ++u) {
             const int j = base + u * TOK + slot;
-            jj[u] = j;
-            valid[u] = j < tok_end;
-            const int jc = valid[u] ? j : tok_begin; // any in-range token: keeps the load legal
+            S.jj[u] = j;
+            S.valid[u] = j < tok_end;
+            const int jc = S.valid[u] ? j : tok_begin; // any in-range token: keeps the load legal
             const int64_t page = a.indices[ip0 + jc / (int)a.page_size];
             const size_t off =
                 ((size_t)page * a.stride_page + (size_t)(jc % (int)a.page_size) * a.stride_n) * esz + head_off;
-            kv[u].load_nt(a.k_data + off); // read once per launch (+2 to 3 % over plain loads)
-            vv[u].load_nt(a.v_data + off);
+            S.kv[u].load_nt(a.k_data + off); // read once per launch (+2 to 3 % over plain loads)
+            S.vv[u].load_nt(a.v_data + off);
         }
+    };
+    auto compute = [&](TokSet& S) __attribute__((always_inline)) {
+        Vec8<KVT>(&kv)[UNROLL] = S.kv;
+        Vec8<KVT>(&vv)[UNROLL] = S.vv;
+        bool(&valid)[UNROLL] = S.valid;
+        int(&jj)[UNROLL] = S.jj;
         float4 cs[TABLE ? TU : 1][4]; // (cos, sin) of this lane's eight pairs at the positions of TU tokens
         auto fetch_cs = [&](int u) {
             const int jc = valid[u] ? jj[u] : tok_begin;
@@ -248,6 +261,23 @@ __global__ __launch_bounds__(256) void decode_general_kernel(DecodeArgs a) {
                 acc[g][e] = t;
             }
             m[g] = mx;
+        }
+    };
+    constexpr int STEP = TOK * UNROLL;
+    if constexpr (G >= 2) {
+        TokSet A, B;
+        if (tok_begin < tok_end) issue(tok_begin, A);
+        for (int base = tok_begin; base < tok_end; base += 2 * STEP) {
+            issue(base + STEP, B);
+            compute(A);
+            issue(base + 2 * STEP, A);
+            if (base + STEP < tok_end) compute(B);
+        }
+    } else {
+        for (int base = tok_begin; base < tok_end; base += STEP) {
+            TokSet A;
+            issue(base, A);
+            compute(A);
         }
     }
 
