@@ -291,7 +291,9 @@ def bench_decode(args, name):
         "plan_ms_per_model_step": round(plan_ms, 4),
         "step_launch": graph_note,
         "step_calls": "append_decode_kv_cache + batch_decode_attention (3 launches)" if args.two_call
-                      else "bz_decode_step (2 launches: decode kernel, then append + new-token term + split-K fold)",
+                      else "bz_decode_step (2 launches: decode kernel, then append + new-token term + split-K fold)"
+                      if handler.step_form() == "one_call"
+                      else "bz_decode_step (its choice for this plan: append, decode kernel, split-K combine)",
         "eager_us_per_step": round(eager_ms * 1e3, 3),
         "decode_call_us": pct(dec_ms),
         "decode_kernel_us": pct(kern_ms),

@@ -55,6 +55,7 @@ SIGNATURES = {
                                         C.POINTER(_sz)]),
     "bz_decode_plan_host_schedule": (_i32, [_vp, _i32, C.POINTER(_vp), C.POINTER(_sz), C.POINTER(_u32)]),
     "bz_decode_plan_info": (_i32, [_vp, C.POINTER(_u32), C.POINTER(_u32), C.POINTER(_u32)]),
+    "bz_decode_plan_step_form": (_i32, [_vp]),
     "bz_decode_plan_set_timing_events": (_i32, [_vp, _vp, _vp]),
     "bz_batch_decode": (_i32, [_vp, _vp, _i32, _kvp, _vp, _i32, _u32, _i32, _f32, _f32, _vp, _vp, _vp, _vp]),
     "bz_decode_step": (_i32, [_vp, _vp, _i32, _vp, _vp, _kvp, _vp, _i32, _u32, _i32, _f32, _f32, _vp, _vp, _vp, _vp]),

@@ -615,7 +615,7 @@ extern "C" int bz_decode_step(bz_decode_plan_t* plan_, const void* q, int q_dtyp
     hipStream_t s = (hipStream_t)stream;
     if (p->batch_size == 0) return 0;
     int rc = BZ_ERR_UNSUPPORTED;
-    if (!p->force_general && p->num_segments > 0) {
+    if (p->step_one_call && p->num_segments > 0) {
         const int D = (int)kv->head_dim;
         const float scale = sm_scale > 0.f ? sm_scale : 1.0f / sqrtf((float)D);
         const RopeFreqs freqs = make_rope_freqs(D, rope_theta > 0.f ? rope_theta : 1e4f);

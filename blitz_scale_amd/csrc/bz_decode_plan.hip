@@ -390,9 +390,26 @@ extern "C" int bz_decode_plan(bz_decode_plan_t* plan_, void* float_buffer, size_
         }
     }
     // BZ_DECODE_PATH=general keeps the MFMA kernel out (used to test the general kernel on shapes
-    // both kernels cover)
+    // both kernels cover); BZ_DECODE_PATH=one_call makes the decode step take its one-call form wherever
+    // it applies, also where the two calls are the faster choice (used to test it on such batches)
     const char* path = getenv("BZ_DECODE_PATH");
     p->force_general = path && !strcmp(path, "general");
+    const bool force_one_call = path && !strcmp(path, "one_call");
+
+    // Form of the decode step.  In its one-call form every piece goes through a partial row that the
+    // finishing kernel reads back; in the two calls a (sequence, kv head) that one wave slot holds whole
+    // writes its final rows at once.  So the one call pays where most of them are split over wave slots
+    // anyway (batches with fewer of them than the launch has slots), and the two calls are taken where most
+    // are whole (1024 sequences of 64 tokens: 63 us against 77 us).  The one call also needs room for one
+    // partial per piece in the float workspace.
+    {
+        const size_t part_o_bytes = ((size_t)p->mfma_pieces * 16 * 128 * sizeof(float) + 255) / 256 * 256;
+        const size_t part_lse_bytes = ((size_t)p->mfma_pieces * 16 * sizeof(float) + 255) / 256 * 256;
+        const bool applies = p->mfma_ok && !p->force_general && p->mfma_slots > 0 && p->mfma_units_d &&
+                             p->mfma_units > 0 && part_o_bytes + part_lse_bytes <= p->float_buffer_bytes;
+        const bool mostly_split = 2 * (uint64_t)p->mfma_combos >= p->mfma_units;
+        p->step_one_call = applies && (force_one_call || mostly_split);
+    }
 
     p->planned = true;
     return 0;
@@ -451,6 +468,12 @@ extern "C" int bz_decode_plan_info(const bz_decode_plan_t* plan_, uint32_t* num_
     if (num_split_seqs) *num_split_seqs = mfma ? p->mfma_split_seqs : p->num_combos;
     if (num_workgroups) *num_workgroups = mfma ? p->mfma_slots : p->num_workgroups;
     return 0;
+}
+
+extern "C" int bz_decode_plan_step_form(const bz_decode_plan_t* plan_) {
+    const DecodePlan* p = reinterpret_cast<const DecodePlan*>(plan_);
+    if (!p || !p->planned) return BZ_ERR_NOT_PLANNED;
+    return p->step_one_call ? 1 : 0;
 }
 
 extern "C" int bz_decode_plan_set_timing_events(bz_decode_plan_t* plan_, void* start_event, void* stop_event) {

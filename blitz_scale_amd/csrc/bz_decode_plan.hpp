@@ -109,6 +109,7 @@ struct DecodePlan {
     // MFMA path schedule (valid when mfma_ok)
     bool mfma_ok = false;
     bool force_general = false; // tests: run the general kernel even where the MFMA path applies
+    bool step_one_call = false;  // bz_decode_step runs its two-launch form (else the append and the decode calls)
     uint32_t mfma_slots = 0, mfma_combos = 0, mfma_partials = 0, mfma_pieces = 0, mfma_split_seqs = 0;
     uint32_t mfma_max_count = 0; // most partials any split (sequence, kv head) has
     bool mfma_streaming = false; // every wave slot has two tiles or more (bandwidth-bound launch)

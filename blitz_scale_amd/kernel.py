@@ -161,6 +161,13 @@ class BlitzBatchDecodeHandler:
         check(_lib.load().bz_decode_plan_info(self._h, C.byref(a), C.byref(b), C.byref(c)), "Handler info")
         return {"segments": a.value, "split_seqs": b.value, "workgroups": c.value}
 
+    def step_form(self):
+        """'one_call': decode_step on this plan runs its two-launch form; 'two_calls': it runs the append and
+        the decode one after the other (the faster order where most (sequence, kv head)s are not split)."""
+        rc = _lib.load().bz_decode_plan_step_form(self._h)
+        check(min(rc, 0), "Handler step form")
+        return "one_call" if rc == 1 else "two_calls"
+
     def __del__(self):
         try:
             if self._h:

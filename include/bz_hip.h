@@ -137,6 +137,9 @@ int bz_decode_plan_host_schedule(const bz_decode_plan_t* plan, int which, const 
 /* introspection for tests and the bench: number of segments / of sequences that were split */
 int bz_decode_plan_info(const bz_decode_plan_t* plan, uint32_t* num_segments, uint32_t* num_split_seqs,
                         uint32_t* num_workgroups);
+/* introspection: 1 when bz_decode_step on this plan runs its two-launch form, 0 when it runs the append and the
+ * decode calls one after the other (see bz_decode_step); negative on error.  No counterpart in the reference. */
+int bz_decode_plan_step_form(const bz_decode_plan_t* plan);
 
 /* Profiling aid (no counterpart in the reference): when both handles are non-NULL hipEvent_t values,
  * the next bz_batch_decode calls on this plan record them on the launch stream immediately before
@@ -168,7 +171,10 @@ int bz_batch_decode(bz_decode_plan_t* plan, const void* q, int q_dtype, const bz
  * only (q is rotated in registers); the pool receives the same bits bz_append_decode_kv writes; `out` agrees
  * with the two-call sequence to rounding (the summation order differs).  Needs a float workspace with room
  * for one partial per piece (bz_decode_plan_workspace reports it); where the matrix-core kernel does not
- * apply, or the workspace is too small, the call runs the two-call sequence itself.  Launch only.
+ * apply, or the workspace is too small, the call runs the two-call sequence itself.  It also does so where
+ * that is the faster order: batches in which most (sequence, kv head)s fit one wave slot whole write their
+ * final rows directly in the two calls, while the two-launch form would send each through a partial row
+ * (bz_decode_plan_step_form tells which form a plan takes).  Launch only.
  */
 int bz_decode_step(bz_decode_plan_t* plan, const void* q, int q_dtype, const void* k_new, const void* v_new,
                    const bz_paged_kv_t* kv, void* out, int out_dtype, uint32_t num_qo_heads, int rope,

@@ -24,7 +24,10 @@ from _util import DecodeProblem, ulp_tol
 pytestmark = pytest.mark.gpu
 
 
-def run_step(p, split_tokens=0, rope=True, theta=5e5, expect_units=True):
+def run_step(p, split_tokens=0, rope=True, theta=5e5, expect_units=True, form="one_call"):
+    """form "one_call": the two-launch form wherever it applies, also on batches where the library would choose
+    the two calls (BZ_DECODE_PATH=one_call at plan time); "library": the library's own choice.  Returns the form
+    that ran beside the results."""
     rng = np.random.default_rng(999)
     k = wl.randn_bits(rng, (p.B, p.Hkv, p.D), p.dtype)
     v = wl.randn_bits(rng, (p.B, p.Hkv, p.D), p.dtype)
@@ -39,8 +42,17 @@ def run_step(p, split_tokens=0, rope=True, theta=5e5, expect_units=True):
     pool_two = to_host_bits(two.pool)
 
     # ---- the one call
-    dev = DeviceDecode(p)
-    dev.plan(split_tokens)
+    dev = DeviceDecode(p, float_ws_bytes=128 << 20)  # the reference's size (src/model/llama.h:111): one partial per piece fits
+    if form == "one_call":
+        os.environ["BZ_DECODE_PATH"] = "one_call"
+    try:
+        dev.plan(split_tokens)
+    finally:
+        if form == "one_call":
+            del os.environ["BZ_DECODE_PATH"]
+    dev.form = dev.handler.step_form()
+    if form == "one_call" and expect_units:
+        assert dev.form == "one_call"
     if expect_units:
         assert len(dev.handler.host_schedule(7)) == int((p.ctx > 0).sum()) * p.Hkv * max(1, (p.Hq // p.Hkv + 15) // 16)
     kd, vd = to_dev(k, p.dtype), to_dev(v, p.dtype)
@@ -117,6 +129,16 @@ def test_step_e4m3_pool_with_several_tiles_per_wave_slot():
     run_step(DecodeProblem(305, ctx, 16, 4, 128, 16, BZ_BF16, kv_dtype=BZ_E4M3), split_tokens=2048)
 
 
+def test_step_takes_the_faster_form():
+    """Left to itself the call takes its two-launch form where most (sequence, kv head)s are split over wave slots
+    (few long sequences) and the two calls where most are whole (many short ones); same results either way."""
+    dev, _, _ = run_step(DecodeProblem(308, [3000, 4100, 2500, 3300], 32, 8, 128, 16, BZ_BF16), form="library")
+    assert dev.form == "one_call"
+    ctx = np.random.default_rng(80).integers(1, 120, size=1100).tolist()
+    dev, _, _ = run_step(DecodeProblem(309, ctx, 16, 4, 128, 16, BZ_BF16), form="library")
+    assert dev.form == "two_calls"
+
+
 def test_step_without_rope_and_with_many_partials():
     run_step(DecodeProblem(303, [20000, 77], 32, 8, 128, 16, BZ_BF16), split_tokens=2048, rope=False)
 
@@ -139,7 +161,7 @@ def test_step_falls_back_where_the_matrix_core_kernel_does_not_apply():
     run_step(DecodeProblem(305, [17, 64, 130, 255, 1], 4, 4, 64, 16, BZ_F16), expect_units=False, theta=1e4)
     os.environ["BZ_DECODE_PATH"] = "general"
     try:
-        run_step(DecodeProblem(306, [700, 3000], 32, 8, 128, 16, BZ_BF16), split_tokens=512)
+        run_step(DecodeProblem(306, [700, 3000], 32, 8, 128, 16, BZ_BF16), split_tokens=512, form="library")
     finally:
         del os.environ["BZ_DECODE_PATH"]
 
