@@ -806,6 +806,10 @@ __global__ __launch_bounds__(32 * HB * S) void decode_step_finish_kernel(StepFin
     load_batch(NB * (int)sl, li0, oi0);
 
     const int seq_len = u.seq_len - max(ahead_raw, 0);
+    // (the page of the newest token is asked for here, with the loads above, not where it is used: one
+    // dependent round trip less between the unit record and the append)
+    const bool appends = g_raw == 0 && sl == 0 && u.unit % (int)a.parts == 0; // one head's lanes per (sequence, kv head)
+    const int64_t page = appends ? a.indices[u.ip0 + max(seq_len - 1, 0) / (int)a.page_size] : 0;
     OT* orow = reinterpret_cast<OT*>(a.out) + ((size_t)b * a.num_qo_heads + hq) * 128;
     if (seq_len <= 0) { // no token at present: nothing to append, a zero row
         const OT z[4] = {StoreCvt<OT>::from(0.f), StoreCvt<OT>::from(0.f), StoreCvt<OT>::from(0.f), StoreCvt<OT>::from(0.f)};
@@ -850,8 +854,7 @@ __global__ __launch_bounds__(32 * HB * S) void decode_step_finish_kernel(StepFin
             dot += qd[e] * pool_to_f32(k_st[e]);
             v_term[e] = pool_to_f32(v_st[e]) * vsc;
         }
-        if (g_raw == 0 && sl == 0 && u.unit % (int)a.parts == 0) { // the append: one head's lanes per (sequence, kv head)
-            const int64_t page = a.indices[u.ip0 + pos / (int)a.page_size];
+        if (appends) { // the append
             const size_t off = (size_t)page * a.stride_page + (size_t)(pos % (int)a.page_size) * a.stride_n +
                                (size_t)kvr * a.stride_h + d0;
             store4(reinterpret_cast<PT*>(a.k_data) + off, k_st);

@@ -84,7 +84,7 @@ __global__ __launch_bounds__(1024) void batch_find_max_kernel(uint32_t* __restri
     // keeps eight 16-byte loads outstanding (128 KiB per CU).
     uint32_t k = threadIdx.x;
     const uint32_t nt = blockDim.x;
-    for (; k < nvec; k += 8 * nt) { // (the last round re-reads the row's last load where it runs past the end)
+    for (; k < nvec; k += 8 * nt) { // (the last pass re-reads the row's last load where it runs past the end)
         uint4 w[8];
 #pragma unroll
         for (int u = 0; u < 8; ++u) w[u] = vrow[min(k + u * nt, nvec - 1)];
