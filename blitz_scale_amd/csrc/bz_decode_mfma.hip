@@ -188,6 +188,14 @@ __global__ __launch_bounds__(64, 2) void decode_mfma_kernel(MfmaDecodeArgs a, co
     const int lane = threadIdx.x;
     const int n = lane & 15; // query head (scores) / d column (output) / token row (K operand)
     const int j = lane >> 4; // lane group: which 8-wide slice of the MFMA contraction
+    // This lane's rotation frequency, fetched once and before anything else: read where a piece is opened, the
+    // load would sit behind the tile's K/V loads in the (in-order) queue, and the angles and the rotation of q
+    // -- some 400 instructions -- would start only after the tile has arrived instead of running while it travels.
+    float lane_freq = 0.f;
+    if (ROPE_Q) {
+        lane_freq = a.freqs.f[lane];
+        asm volatile("" : "+v"(lane_freq)); // (kept in its register: not fetched again at the point of use)
+    }
     const int P = (int)a.page_size;
     constexpr int ES = KV8 ? 1 : 2; // bytes per pool element
     const size_t row_bytes = (size_t)a.stride_n * ES;
@@ -358,7 +366,7 @@ __global__ __launch_bounds__(64, 2) void decode_mfma_kernel(MfmaDecodeArgs a, co
         for (int ks = 0; ks < 4; ++ks) { qhi[ks] = qnext[ks]; qlo[ks] = make_uint4(0, 0, 0, 0); }
         if (ROPE_Q) {
             float sn1, cs1;
-            sincosf((float)(uc.seq_len - 1 + a.step_mode) * a.freqs.f[lane], &sn1, &cs1); // q sits at the last token
+            sincosf((float)(uc.seq_len - 1 + a.step_mode) * lane_freq, &sn1, &cs1); // q sits at the last token
             wave_lds_sync(); // the previous piece's reads of the table are done
             rope_cs[0][lane] = cs1;
             rope_cs[ROPE_Q ? 1 : 0][lane] = sn1; // (the index keeps the one-row dummy of the other instantiations in bounds)
