@@ -627,6 +627,12 @@ __global__ __launch_bounds__(64, 2) void decode_mfma_kernel(MfmaDecodeArgs a, co
             }
             // The K rows are contracted straight out of their landing registers and the next tile's loads go
             // out right behind the eight score instructions (which have read their operands by then).
+            // Every load of this wave has arrived by now (the V rows just parked were the youngest).  Said
+            // explicitly, because the compiler's bookkeeping merges paths on which it cannot tell: without this
+            // it guards the landing registers it reuses as address temporaries further down with waits that
+            // count loads from the wrong end -- no-ops on most tiles, but where a new piece's q rows have just
+            // been requested they held the next tile's V loads back until q had arrived.
+            __builtin_amdgcn_s_waitcnt(0x0F70); // vmcnt(0)
             f32x4_t s[2];
             scores(kreg, s);
             __builtin_amdgcn_sched_barrier(0); // the loads below overwrite the operands of the instructions above
