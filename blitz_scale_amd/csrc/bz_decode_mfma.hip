@@ -148,6 +148,13 @@ template <bool BF16> __device__ __forceinline__ uint4 fp8x8_to_op(const uint4& r
 // wave-level ordering of LDS traffic: LDS instructions of one wave execute in order, so making the
 // compiler keep the order is all that is needed (a workgroup barrier would also drain the global loads
 // that are in flight for the next tile)
+// 16 bytes to global memory through a pointer whose address space the compiler cannot see (it came out of LDS):
+// said explicitly, so that the store is a global one and not a flat one, which would also count as an LDS access.
+__device__ __forceinline__ void store_global_16(void* p, float a, float b, float c, float d) {
+    typedef float vec4 __attribute__((ext_vector_type(4)));
+    *(__attribute__((address_space(1))) vec4*)p = vec4{a, b, c, d};
+}
+
 __device__ __forceinline__ void wave_lds_sync() {
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
     __builtin_amdgcn_wave_barrier();
@@ -180,6 +187,13 @@ __global__ __launch_bounds__(64, 2) void decode_mfma_kernel(MfmaDecodeArgs a, co
     using M = Mma<BF16>;
     __shared__ __attribute__((aligned(16))) unsigned char v_lds[kTileTok * kVRowBytes];
     __shared__ __attribute__((aligned(16))) int info_lds[2][kInfoChunk][kInfoInts];
+    // Normalised rows of finished pieces, kept here until the slot's last tile is done (or the space runs out):
+    // 16 rows of 128 floats (+ 4 per row, so that the four lane groups fall on different banks), one log-sum-exp
+    // per row, and for each parked piece where its rows go.
+    constexpr int kStageRow = 132, kStageRows = 16, kStagePieces = 8;
+    struct StagedPiece { char* dst; float* lse; int row0, rows, f32, pad; };
+    __shared__ __attribute__((aligned(16))) float stage_lds[kStageRows * kStageRow + kStageRows];
+    __shared__ StagedPiece stage_desc[kStagePieces];
 
     // cos / sin of position * frequency i for the piece being opened: one sincosf per lane instead of
     // sixteen (each lane needs the angles of its own 16 contraction indices)
@@ -413,8 +427,52 @@ __global__ __launch_bounds__(64, 2) void decode_mfma_kernel(MfmaDecodeArgs a, co
             }
         }
     };
+    // Rows of finished pieces leave in one go at the end of the slot.  A store in the middle of the stream is
+    // expensive out of proportion on this target: loads and stores share one in-order counter, so the data of
+    // every load issued after a store is held back until the store has been acknowledged, and under a full read
+    // stream that takes longer than a tile -- measured 2.3 us per piece, wherever in the tile loop the stores
+    // were placed, non-temporal or not.
+    int pend_rows = 0, pend_n = 0;
+    // rows [row0, row0 + rows) of the parked rows to dst, their log-sum-exps to lse_p (all arguments wave-uniform)
+    auto store_piece = [&](char* dst_c, float* lse_p, int row0, int rows, bool f32) __attribute__((always_inline)) {
+        const float* src = stage_lds + row0 * kStageRow;
+        if (f32) { // fp32 rows, four elements per lane; the rows lie side by side at the destination
+            float* dst = reinterpret_cast<float*>(dst_c);
+            for (int c = lane; c < rows * 32; c += 64) {
+                const int row = c >> 5, w = c & 31;
+                const float4 v = *reinterpret_cast<const float4*>(src + row * kStageRow + 4 * w);
+                store_global_16(dst + row * 128 + 4 * w, v.x, v.y, v.z, v.w);
+            }
+        } else if constexpr (!std::is_same<OT, float>::value) { // 16-bit rows, eight elements per lane
+            OT* dst = reinterpret_cast<OT*>(dst_c);
+            for (int c = lane; c < rows * 16; c += 64) {
+                const int row = c >> 4, w = c & 15;
+                const float4 x = *reinterpret_cast<const float4*>(src + row * kStageRow + 8 * w);
+                const float4 y = *reinterpret_cast<const float4*>(src + row * kStageRow + 8 * w + 4);
+                uint4 o;
+                o.x = (uint32_t)StoreCvt<OT>::from(x.x).bits | ((uint32_t)StoreCvt<OT>::from(x.y).bits << 16);
+                o.y = (uint32_t)StoreCvt<OT>::from(x.z).bits | ((uint32_t)StoreCvt<OT>::from(x.w).bits << 16);
+                o.z = (uint32_t)StoreCvt<OT>::from(y.x).bits | ((uint32_t)StoreCvt<OT>::from(y.y).bits << 16);
+                o.w = (uint32_t)StoreCvt<OT>::from(y.z).bits | ((uint32_t)StoreCvt<OT>::from(y.w).bits << 16);
+                store_global_16(dst + row * 128 + 8 * w, __uint_as_float(o.x), __uint_as_float(o.y), __uint_as_float(o.z),
+                                __uint_as_float(o.w));
+            }
+        }
+        if (lse_p && lane < rows)
+            *(__attribute__((address_space(1))) float*)(lse_p + lane) = stage_lds[kStageRows * kStageRow + row0 + lane];
+    };
+    auto store_rows = [&]() __attribute__((always_inline)) {
+        for (int pc = 0; pc < pend_n; ++pc) {
+            const StagedPiece sp = stage_desc[pc]; // (the same in every lane)
+            store_piece(sp.dst, sp.lse, __builtin_amdgcn_readfirstlane(sp.row0), __builtin_amdgcn_readfirstlane(sp.rows),
+                        __builtin_amdgcn_readfirstlane(sp.f32) != 0);
+        }
+        wave_lds_sync(); // everything parked has been read before anything new is parked
+        pend_rows = 0;
+        pend_n = 0;
+    };
     // ---- mask, online softmax, O += P V (V of the tile is in LDS), and the rows of a finished piece
-    auto softmax_pv = [&](const TileUni& uc, f32x4_t (&s)[2], float score_scale) __attribute__((always_inline)) {
+    auto softmax_pv = [&](const TileUni& uc, f32x4_t (&s)[2], float score_scale, bool last_of_slot) __attribute__((always_inline)) {
         const int tile_tok0 = uc.t * kTileTok, tok_end = uc.tok_end;
         const bool ragged = tile_tok0 + kTileTok > tok_end; // wave-uniform
         if (ragged) {
@@ -489,28 +547,44 @@ __global__ __launch_bounds__(64, 2) void decode_mfma_kernel(MfmaDecodeArgs a, co
             const int b = uc.seq, kvh = uc.kvh, partial = uc.partial;
             const float inv_l = (l_run > 0.f ? 1.0f / l_run : 0.f) * ((KV8 && v_scale) ? v_scale[uc.kvr] : 1.0f);
             const float lse2 = l_run > 0.f ? m_run + log2f(l_run) : -INFINITY;
+            // the normalised rows are parked in LDS, head-major (store_rows above says why)
+            if (pend_rows + G > kStageRows || pend_n == kStagePieces) store_rows();
+            float* rows = stage_lds + pend_rows * kStageRow;
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
                 const int head = 4 * j + i;
                 const float il = __shfl(inv_l, head, 64);
                 if (head < G) {
-                    if (partial < 0) {
-                        OT* orow = reinterpret_cast<OT*>(a.out) + ((size_t)b * a.num_qo_heads + kvh * G + head) * 128;
 #pragma unroll
-                        for (int d = 0; d < 8; ++d) orow[d * 16 + n] = StoreCvt<OT>::from(acc[d][i] * il);
-                    } else {
-                        float* prow = a.part_o + ((size_t)partial * 16 + head) * 128;
-#pragma unroll
-                        for (int d = 0; d < 8; ++d) prow[d * 16 + n] = acc[d][i] * il;
-                    }
+                    for (int d = 0; d < 8; ++d) rows[head * kStageRow + d * 16 + n] = acc[d][i] * il;
                 }
             }
-            if (j == 0 && n < G) {
-                if (partial < 0) {
-                    if (a.lse) a.lse[(size_t)b * a.num_qo_heads + kvh * G + n] = lse2 * 0.6931471805599453f;
-                } else {
-                    a.part_lse[(size_t)partial * 16 + n] = lse2;
+            if (j == 0 && n < G) stage_lds[kStageRows * kStageRow + pend_rows + n] = partial < 0 ? lse2 * 0.6931471805599453f : lse2;
+            const bool f32_rows = partial >= 0 || std::is_same<OT, float>::value;
+            char* dst_c;
+            float* lse_p;
+            if (partial >= 0) {
+                dst_c = reinterpret_cast<char*>(a.part_o + (size_t)partial * 16 * 128);
+                lse_p = a.part_lse + (size_t)partial * 16;
+            } else {
+                dst_c = reinterpret_cast<char*>(reinterpret_cast<OT*>(a.out) + ((size_t)b * a.num_qo_heads + kvh * G) * 128);
+                lse_p = a.lse ? a.lse + (size_t)b * a.num_qo_heads + kvh * G : nullptr;
+            }
+            if (last_of_slot) { // nothing comes after these stores: out they go, behind whatever is still parked
+                wave_lds_sync();
+                const int row0 = pend_rows;
+                store_rows();
+                store_piece(dst_c, lse_p, row0, G, f32_rows);
+            } else {
+                if (lane == 0) {
+                    StagedPiece sp;
+                    sp.dst = dst_c; sp.lse = lse_p;
+                    sp.row0 = pend_rows; sp.rows = G; sp.f32 = f32_rows ? 1 : 0; sp.pad = 0;
+                    stage_desc[pend_n] = sp;
                 }
+                wave_lds_sync();
+                pend_rows += G;
+                ++pend_n;
             }
         }
     };
@@ -577,7 +651,7 @@ __global__ __launch_bounds__(64, 2) void decode_mfma_kernel(MfmaDecodeArgs a, co
             }
             f32x4_t s[2];
             scores(kcur, s);
-            softmax_pv(uc, s, score_scale);
+            softmax_pv(uc, s, score_scale, g + 1 == g_end);
         };
         // (The loop has no exit between its halves, so that the only way into one set's half is through the
         // other set's half: the waits the compiler places for a set's registers then leave the other set's loads
@@ -641,9 +715,10 @@ __global__ __launch_bounds__(64, 2) void decode_mfma_kernel(MfmaDecodeArgs a, co
                 if (un.flags & 1) issue_q(un); // next tile opens a new piece
                 issue_loads(nb);
             }
-            softmax_pv(uc, s, score_scale);
+            softmax_pv(uc, s, score_scale, g + 1 == g_end);
         }
     }
+    store_rows(); // every piece the slot has finished since the last time
 }
 
 // Combine the partials of one split (sequence, kv head): o = sum_i o_i 2^(lse_i - M) / sum_i 2^(lse_i - M).
@@ -1000,7 +1075,7 @@ int decode_fast_path(const DecodePlan* p, const void* q, void* out, float* lse, 
     if (!kv8 && (k_scale || v_scale)) return BZ_ERR_UNSUPPORTED;
     const uint64_t es = kv8 ? 1 : 2;
     if ((kv->stride_n * es) % 16 || (kv->stride_h * es) % 16 || (kv->stride_page * es) % 16) return BZ_ERR_UNSUPPORTED;
-    if (((uintptr_t)kv->k_data | (uintptr_t)kv->v_data | (uintptr_t)q) % 16) return BZ_ERR_UNSUPPORTED;
+    if (((uintptr_t)kv->k_data | (uintptr_t)kv->v_data | (uintptr_t)q | (uintptr_t)out) % 16) return BZ_ERR_UNSUPPORTED;
     MfmaDecodeArgs a;
     a.q = q; a.out = out; a.lse = lse;
     a.k_data = (const char*)kv->k_data; a.v_data = (const char*)kv->v_data;
