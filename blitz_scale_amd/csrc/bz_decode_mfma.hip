@@ -573,7 +573,7 @@ __global__ __launch_bounds__(64, 2) void decode_mfma_kernel(MfmaDecodeArgs a, co
             if (last_of_slot) { // nothing comes after these stores: out they go, behind whatever is still parked
                 wave_lds_sync();
                 const int row0 = pend_rows;
-                store_rows();
+                if (pend_n) store_rows();
                 store_piece(dst_c, lse_p, row0, G, f32_rows);
             } else {
                 if (lane == 0) {
