@@ -202,14 +202,6 @@ __global__ __launch_bounds__(64, 2) void decode_mfma_kernel(MfmaDecodeArgs a, co
     const int lane = threadIdx.x;
     const int n = lane & 15; // query head (scores) / d column (output) / token row (K operand)
     const int j = lane >> 4; // lane group: which 8-wide slice of the MFMA contraction
-    // This lane's rotation frequency, fetched once and before anything else: read where a piece is opened, the
-    // load would sit behind the tile's K/V loads in the (in-order) queue, and the angles and the rotation of q
-    // -- some 400 instructions -- would start only after the tile has arrived instead of running while it travels.
-    float lane_freq = 0.f;
-    if (ROPE_Q) {
-        lane_freq = a.freqs.f[lane];
-        asm volatile("" : "+v"(lane_freq)); // (kept in its register: not fetched again at the point of use)
-    }
     const int P = (int)a.page_size;
     constexpr int ES = KV8 ? 1 : 2; // bytes per pool element
     const size_t row_bytes = (size_t)a.stride_n * ES;
@@ -226,6 +218,15 @@ __global__ __launch_bounds__(64, 2) void decode_mfma_kernel(MfmaDecodeArgs a, co
     const MfmaSlotHead* __restrict__ head = heads + blockIdx.x;
     const int g_begin = head->begin, g_end = head->end;
     const MfmaSlotHead first = *head;
+    // This lane's rotation frequency, fetched once and here, beside the scalar loads of the slot head: read where a
+    // piece is opened, the load would sit behind the tile's K/V loads in the (in-order) queue, and the angles and
+    // the rotation of q -- some 400 instructions -- would start only after the tile has arrived instead of running
+    // while it travels.
+    float lane_freq = 0.f;
+    if (ROPE_Q) {
+        lane_freq = a.freqs.f[lane];
+        asm("" : "+v"(lane_freq)); // (kept in its register: not fetched again at the point of use)
+    }
     if (g_begin >= g_end) return;
     const int ahead = max(ahead_raw, 0);
 
@@ -233,25 +234,38 @@ __global__ __launch_bounds__(64, 2) void decode_mfma_kernel(MfmaDecodeArgs a, co
     // page ids it points at and the piece it belongs to, and leaves 10 ints in LDS:
     //   [pid0, pid1, t, seq | kvh, flags (1: first tile of its piece, 2: last), partial, tok_end | seq_len, kv head]
     struct Desc { int v[10]; };
-    auto fetch_info = [&](int base) -> Desc {
+    // (in three steps, so that the prologue can put other loads between them: the record, what the record points at,
+    // and the arithmetic on both)
+    struct InfoRaw { int4 m0, m1, m2; int pid0, pid1; };
+    // (lanes past the slot's last tile fetch that tile once more: loads under a lane mask would make the compiler
+    // wait for them on the spot, before it zeroes the other lanes' registers)
+    auto fetch_rec = [&](int base) -> MfmaTile { return tiles[min(base + (lane & (kInfoChunk - 1)), g_end - 1)]; };
+    auto fetch_dep = [&](const MfmaTile& rec) -> InfoRaw {
+        InfoRaw r;
+        r.m0 = *reinterpret_cast<const int4*>(&pieces[rec.piece]);
+        r.m1 = *(reinterpret_cast<const int4*>(&pieces[rec.piece]) + 1);
+        r.m2 = *(reinterpret_cast<const int4*>(&pieces[rec.piece]) + 2);
+        r.pid0 = indices[rec.idx0];
+        r.pid1 = indices[rec.idx1];
+        return r;
+    };
+    auto make_desc = [&](const MfmaTile& rec, const InfoRaw& r) -> Desc {
         Desc d;
-        const int g = base + (lane & (kInfoChunk - 1));
-        const bool live = g < g_end;
-        const MfmaTile rec = live ? tiles[g] : MfmaTile{0, 0, 0, 0};
-        const int4 m0 = live ? *reinterpret_cast<const int4*>(&pieces[rec.piece]) : make_int4(0, 0, 0, 0);
-        const int4 m1 = live ? *(reinterpret_cast<const int4*>(&pieces[rec.piece]) + 1) : make_int4(0, 0, 0, 0);
-        const int4 m2 = live ? *(reinterpret_cast<const int4*>(&pieces[rec.piece]) + 2) : make_int4(0, 0, 0, 0);
-        d.v[0] = live ? indices[rec.idx0] : 0;
-        d.v[1] = live ? indices[rec.idx1] : 0;
+        d.v[0] = r.pid0;
+        d.v[1] = r.pid1;
         d.v[2] = rec.t;
-        d.v[3] = m0.x;                                             // seq
-        d.v[4] = m0.y;                                             // kvh
-        d.v[5] = (rec.t == m0.z ? 1 : 0) | (rec.t + 1 == m0.w ? 2 : 0);
-        d.v[6] = a.step_mode ? rec.piece : m1.x;                   // partial slot or -1
-        d.v[8] = max(m2.z - ahead - a.step_mode, 0);               // tokens attended over at present
-        d.v[7] = min(m0.w * kTileTok, d.v[8]);                     // tok_end of the piece
-        d.v[9] = m2.w;                                             // kv head whose K/V are read (kvh is the scheduled unit)
+        d.v[3] = r.m0.x;                                           // seq
+        d.v[4] = r.m0.y;                                           // kvh
+        d.v[5] = (rec.t == r.m0.z ? 1 : 0) | (rec.t + 1 == r.m0.w ? 2 : 0);
+        d.v[6] = a.step_mode ? rec.piece : r.m1.x;                 // partial slot or -1
+        d.v[8] = max(r.m2.z - ahead - a.step_mode, 0);             // tokens attended over at present
+        d.v[7] = min(r.m0.w * kTileTok, d.v[8]);                   // tok_end of the piece
+        d.v[9] = r.m2.w;                                           // kv head whose K/V are read (kvh is the scheduled unit)
         return d;
+    };
+    auto fetch_info = [&](int base) -> Desc {
+        const MfmaTile rec = fetch_rec(base);
+        return make_desc(rec, fetch_dep(rec));
     };
     auto stash_info = [&](const Desc& d, int buf) {
         if (lane < kInfoChunk) {
@@ -326,35 +340,41 @@ __global__ __launch_bounds__(64, 2) void decode_mfma_kernel(MfmaDecodeArgs a, co
         }
     };
     // q rows of a piece as MFMA B operand: lane (head n, group j) holds q[head][32*ks + 8*j .. +7]
+    // (every lane loads: columns past the group fetch its last head again and are zeroed where the piece is opened --
+    // loads under a lane mask would make the compiler wait for them on the spot)
     auto issue_q = [&](const TileUni& u) {
+        const char* qrow = q_ptr + ((size_t)u.seq * a.num_qo_heads + (size_t)u.kvh * G + min(n, G - 1)) * 256;
 #pragma unroll
-        for (int ks = 0; ks < 4; ++ks) qnext[ks] = make_uint4(0, 0, 0, 0);
-        if (n < G) {
-            const char* qrow = q_ptr + ((size_t)u.seq * a.num_qo_heads + (size_t)u.kvh * G + n) * 256;
-#pragma unroll
-            for (int ks = 0; ks < 4; ++ks) qnext[ks] = *reinterpret_cast<const uint4*>(qrow + d_of(ks) * 2);
-        }
+        for (int ks = 0; ks < 4; ++ks) qnext[ks] = *reinterpret_cast<const uint4*>(qrow + d_of(ks) * 2);
     };
 
-    // The records of the first tiles are requested first and the first tile's q, K and V right behind
-    // them (its description came with the slot head), so parking the records in LDS waits for them only.
-    // (a slot with a single tile -- small batches -- needs no records at all, and fetching them would put two more
-    // dependent round trips in front of its K/V loads)
-    Desc d0 = {};
-    if (g_end - g_begin > 1) d0 = fetch_info(g_begin);
+    // The records of the first tiles are requested together with the two page ids of the first tile (whose
+    // description came with the slot head); what the records point at -- pieces, page ids -- goes out as soon as both
+    // are there, and the first tile's q, K and V right behind it, so that the records are turned into descriptions
+    // and parked in LDS while the first tile travels.  (With the whole fetch in front, its second round trip stood
+    // between the slot head and the first K/V loads.  A slot with a single tile -- small batches -- needs no records.)
+    const bool multi = g_end - g_begin > 1;
     TileUni un; // description of the tile whose loads are issued next
     un.pid0 = indices[first.idx0];
     un.pid1 = indices[first.idx1];
+    MfmaTile rec0 = {0, 0, 0, 0};
+    if (multi) rec0 = fetch_rec(g_begin);
+    asm("" : "+s"(un.pid0), "+s"(un.pid1)); // (asked for here, beside the records, not where the addresses are formed)
     un.t = first.t; un.seq = first.seq; un.kvh = first.kvh; un.flags = first.flags;
     un.partial = a.step_mode ? first.piece : first.partial;
     un.kvr = first.kv_head;
     un.seq_len = max(first.seq_len - ahead - a.step_mode, 0);
     un.tok_end = min(first.tile_end * kTileTok, un.seq_len);
+    __builtin_amdgcn_sched_barrier(0);
+    InfoRaw raw0 = {};
+    if (multi) raw0 = fetch_dep(rec0);
+    __builtin_amdgcn_sched_barrier(0);
     issue_q(un);
     if constexpr (KV8) issue_loads_kv8(tile_base(un), std::integral_constant<int, 0>{}, true);
     else issue_loads(tile_base(un));
-    if (g_end - g_begin > 1) {
-        stash_info(d0, 0);
+    __builtin_amdgcn_sched_barrier(0);
+    if (multi) {
+        stash_info(make_desc(rec0, raw0), 0);
         wave_lds_sync();
     }
     int chunk_base = g_begin, buf = 0;
@@ -377,7 +397,7 @@ __global__ __launch_bounds__(64, 2) void decode_mfma_kernel(MfmaDecodeArgs a, co
     // ================= first tile of a piece =================
     auto open_piece = [&](const TileUni& uc) __attribute__((always_inline)) {
 #pragma unroll
-        for (int ks = 0; ks < 4; ++ks) { qhi[ks] = qnext[ks]; qlo[ks] = make_uint4(0, 0, 0, 0); }
+        for (int ks = 0; ks < 4; ++ks) { qhi[ks] = n < G ? qnext[ks] : make_uint4(0, 0, 0, 0); qlo[ks] = make_uint4(0, 0, 0, 0); }
         if (ROPE_Q) {
             float sn1, cs1;
             sincosf((float)(uc.seq_len - 1 + a.step_mode) * lane_freq, &sn1, &cs1); // q sits at the last token
