@@ -227,7 +227,20 @@ __global__ __launch_bounds__(64, 2) void decode_mfma_kernel(MfmaDecodeArgs a, co
         lane_freq = a.freqs.f[lane];
         asm("" : "+v"(lane_freq)); // (kept in its register: not fetched again at the point of use)
     }
-    if (g_begin >= g_end) return;
+    // Left to the compiler, the slot head is fetched in two steps (its tile range, then, behind the test for an empty
+    // slot, the rest together with most of the kernel's arguments): one more scalar round trip in front of the first
+    // page ids.  The empty asm below needs a value made of all of them, so they are all asked for here, in one batch.
+    uint32_t early = (uint32_t)first.idx0 ^ (uint32_t)first.idx1 ^ (uint32_t)first.t ^ (uint32_t)first.seq ^ (uint32_t)first.kvh ^
+                     (uint32_t)first.flags ^ (uint32_t)first.partial ^ (uint32_t)first.tile_end ^ (uint32_t)first.seq_len ^
+                     (uint32_t)first.kv_head ^ (uint32_t)first.piece;
+    early ^= (uint32_t)(uintptr_t)tiles ^ (uint32_t)(uintptr_t)indices ^ (uint32_t)(uintptr_t)pieces ^ (uint32_t)(uintptr_t)k_data ^
+             (uint32_t)(uintptr_t)v_data ^ (uint32_t)(uintptr_t)q_ptr;
+    early ^= (uint32_t)a.stride_page ^ (uint32_t)a.stride_n ^ (uint32_t)a.stride_h ^ a.page_size ^ a.num_qo_heads ^ a.group ^
+             (uint32_t)a.step_mode;
+    asm("" : "+s"(early));
+    // (g_begin is never negative: the second term only keeps the value above in use)
+    if (g_begin >= g_end || (g_begin < 0 && early == 0x9e3779b9u)) return;
+    int first_pid0 = indices[first.idx0], first_pid1 = indices[first.idx1];
     const int ahead = max(ahead_raw, 0);
 
     // ---- descriptions of kInfoChunk tiles at a time: lane l < kInfoChunk fetches the record of tile base+l, the two
@@ -355,8 +368,8 @@ __global__ __launch_bounds__(64, 2) void decode_mfma_kernel(MfmaDecodeArgs a, co
     // between the slot head and the first K/V loads.  A slot with a single tile -- small batches -- needs no records.)
     const bool multi = g_end - g_begin > 1;
     TileUni un; // description of the tile whose loads are issued next
-    un.pid0 = indices[first.idx0];
-    un.pid1 = indices[first.idx1];
+    un.pid0 = first_pid0;
+    un.pid1 = first_pid1;
     MfmaTile rec0 = {0, 0, 0, 0};
     if (multi) rec0 = fetch_rec(g_begin);
     asm("" : "+s"(un.pid0), "+s"(un.pid1)); // (asked for here, beside the records, not where the addresses are formed)
