@@ -271,6 +271,28 @@ def test_e4m3_pool_with_several_tiles_per_wave_slot(case, rope_mode):
     assert (np.abs(got - ref) <= ulp_tol(ref, p.dtype, 3e-2)).all()
 
 
+@pytest.mark.parametrize("Hq,Hkv,kv_dtype", [(8, 8, None), (16, 8, None), (64, 4, None), (8, 8, BZ_E4M3)])
+def test_many_finished_pieces_per_wave_slot(Hq, Hkv, kv_dtype):
+    """Thousands of sequences of one or two tiles: a wave slot finishes ten and more (sequence, kv head)s, whose
+    normalised rows wait in LDS until the slot is done.  The space holds 8 pieces or 16 rows, so it is emptied in
+    the middle of a slot: by the piece count with one or two q heads per kv head, by the row count with sixteen.
+    Final rows (16-bit and fp32) and log-sum-exps are checked for every sequence."""
+    rng = np.random.default_rng(81)
+    B = 2600 if Hkv == 8 else 5200
+    ctx = rng.integers(1, 41, size=B).tolist()
+    p = DecodeProblem(700 + Hq, ctx, Hq, Hkv, 128, 16, BZ_BF16, kv_dtype=kv_dtype)
+    ref, ref_lse = oracle.batch_decode(p.q, p.dtype, p.oracle_kv(), p.Hq, k_scale=p.k_scale, v_scale=p.v_scale, want_lse=True,
+                                       parallel=True)
+    dev = DeviceDecode(p, float_ws_bytes=128 << 20)
+    info = dev.plan(0)
+    assert info["segments"] >= 9 * info["workgroups"]  # pieces per wave slot
+    got32, lse = dev.decode(BZ_F32, BZ_ROPE_NONE, 1e4, want_lse=True)
+    assert np.abs(got32 - ref).max() <= (3e-2 if kv_dtype == BZ_E4M3 else 2e-5)
+    assert np.abs(lse - ref_lse).max() < 1e-3
+    got = dev.decode(None, BZ_ROPE_NONE, 1e4)
+    assert (np.abs(got - ref) <= ulp_tol(ref, p.dtype, 3e-2 if kv_dtype == BZ_E4M3 else 2e-3)).all()
+
+
 @pytest.mark.parametrize("dtype,kv_dtype", [(BZ_F16, None), (BZ_BF16, None), (BZ_BF16, BZ_E4M3)])
 def test_logits_with_a_large_dynamic_range(dtype, kv_dtype):
     """q rows eight times the usual size: logits of +-40 base-2 units, rows that attend to one or two tokens, and

@@ -24,7 +24,7 @@ from _util import DecodeProblem, ulp_tol
 pytestmark = pytest.mark.gpu
 
 
-def run_step(p, split_tokens=0, rope=True, theta=5e5, expect_units=True, form="one_call"):
+def run_step(p, split_tokens=0, rope=True, theta=5e5, expect_units=True, form="one_call", float_ws_bytes=128 << 20):
     """form "one_call": the two-launch form wherever it applies, also on batches where the library would choose
     the two calls (BZ_DECODE_PATH=one_call at plan time); "library": the library's own choice.  Returns the form
     that ran beside the results."""
@@ -42,7 +42,7 @@ def run_step(p, split_tokens=0, rope=True, theta=5e5, expect_units=True, form="o
     pool_two = to_host_bits(two.pool)
 
     # ---- the one call
-    dev = DeviceDecode(p, float_ws_bytes=128 << 20)  # the reference's size (src/model/llama.h:111): one partial per piece fits
+    dev = DeviceDecode(p, float_ws_bytes=float_ws_bytes)  # default: the reference's size (src/model/llama.h:111), one partial per piece fits
     if form == "one_call":
         os.environ["BZ_DECODE_PATH"] = "one_call"
     try:
@@ -137,6 +137,15 @@ def test_step_takes_the_faster_form():
     ctx = np.random.default_rng(80).integers(1, 120, size=1100).tolist()
     dev, _, _ = run_step(DecodeProblem(309, ctx, 16, 4, 128, 16, BZ_BF16), form="library")
     assert dev.form == "two_calls"
+
+
+def test_step_with_many_finished_pieces_per_wave_slot():
+    """2 600 sequences of one or two tiles on 8 kv heads, one q head each: a wave slot finishes ten and more pieces,
+    more than the space for their parked rows holds, in the two-launch form (every piece a partial row)."""
+    ctx = np.random.default_rng(82).integers(1, 41, size=2600).tolist()
+    dev, _, _ = run_step(DecodeProblem(310, ctx, 8, 8, 128, 16, BZ_BF16), form="one_call", float_ws_bytes=256 << 20)  # 8 KB per piece
+    info = dev.handler.info()
+    assert info["segments"] >= 9 * info["workgroups"]
 
 
 def test_step_without_rope_and_with_many_partials():
