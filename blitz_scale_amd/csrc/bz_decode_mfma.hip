@@ -1142,8 +1142,12 @@ static int launch_step_finish(const DecodePlan* p, const StepFinishArgs& a, hipS
             hipLaunchKernelGGL((decode_step_finish_kernel<QT, PT, OT, 1, 1>), dim3(p->mfma_units, G), dim3(32, 1, 1), 0, s, a);
     } else if (p->mfma_unit_max_count > 32 && p->mfma_unit_max_count <= 64) {
         hipLaunchKernelGGL((decode_step_finish_kernel<QT, PT, OT, 4, 2>), dim3(p->mfma_units, (G + 1) / 2), dim3(32, 2, 4), 0, s, a);
-    } else { // 17..32 partials: one batch of four per slice, a single round of loads; more than 64: eight slices as well
-
+    } else if (p->mfma_unit_max_count <= 32) {
+        // 17..32 partials (batches of eight sequences or so): one batch of four per slice, a single round of loads, and
+        // one head per workgroup -- four waves; measured on 32 layers at batch 8 against two heads (eight waves) 497
+        // against 505 us per step, four heads (sixteen waves) 527, four slices of two heads 507
+        hipLaunchKernelGGL((decode_step_finish_kernel<QT, PT, OT, 8, 1>), dim3(p->mfma_units, G), dim3(32, 1, 8), 0, s, a);
+    } else { // more than 64 partials: eight slices as well
         hipLaunchKernelGGL((decode_step_finish_kernel<QT, PT, OT, 8, 2>), dim3(p->mfma_units, (G + 1) / 2), dim3(32, 2, 8), 0, s, a);
     }
     BZ_LAUNCH_CHECK();
