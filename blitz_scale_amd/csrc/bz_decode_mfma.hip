@@ -1142,13 +1142,13 @@ static int launch_step_finish(const DecodePlan* p, const StepFinishArgs& a, hipS
             hipLaunchKernelGGL((decode_step_finish_kernel<QT, PT, OT, 1, 1>), dim3(p->mfma_units, G), dim3(32, 1, 1), 0, s, a);
     } else if (p->mfma_unit_max_count > 32 && p->mfma_unit_max_count <= 64) {
         hipLaunchKernelGGL((decode_step_finish_kernel<QT, PT, OT, 4, 2>), dim3(p->mfma_units, (G + 1) / 2), dim3(32, 2, 4), 0, s, a);
-    } else if (p->mfma_unit_max_count <= 32) {
-        // 17..32 partials (batches of eight sequences or so): one batch of four per slice, a single round of loads, and
-        // one head per workgroup -- four waves; measured on 32 layers at batch 8 against two heads (eight waves) 497
-        // against 505 us per step, four heads (sixteen waves) 527, four slices of two heads 507
+    } else {
+        // 17..32 partials (batches of eight sequences or so): eight slices, so one batch of four per slice and a single
+        // round of loads, and one head per workgroup -- four waves.  Measured on 32 layers at batch 8: 497 us per step
+        // against 505 with two heads per workgroup (eight waves), 527 with four (sixteen), 507 with four slices of two
+        // heads.  More than 64 partials (a few very long sequences): the same shape (4 x 32 768 tokens: 90.8 against
+        // 91.8 us with two heads).
         hipLaunchKernelGGL((decode_step_finish_kernel<QT, PT, OT, 8, 1>), dim3(p->mfma_units, G), dim3(32, 1, 8), 0, s, a);
-    } else { // more than 64 partials: eight slices as well
-        hipLaunchKernelGGL((decode_step_finish_kernel<QT, PT, OT, 8, 2>), dim3(p->mfma_units, (G + 1) / 2), dim3(32, 2, 8), 0, s, a);
     }
     BZ_LAUNCH_CHECK();
     return 0;
