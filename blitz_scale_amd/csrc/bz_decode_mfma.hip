@@ -11,7 +11,8 @@
 //              (ds_read_b64_tr_b16) as MFMA B operands (contraction over tokens)
 //   softmax  : online, 8 scores per lane, row max / sum over the 4 lane groups with two shuffles
 // The loads of tile t+1 are issued before the arithmetic of tile t; with one-byte pools, whose tiles need half
-// the landing registers, two tiles are in flight per wave.
+// the landing registers, two tiles are in flight per wave.  The rows of a finished piece wait in LDS and are
+// stored when the wave slot is done: between its first load and its last tile a wave issues no store.
 #include <cmath>
 #include <type_traits>
 
@@ -828,8 +829,8 @@ __global__ __launch_bounds__(128 * S) void decode_mfma_combine_kernel(const Mfma
 // result per piece.  This kernel takes the newest token from the caller's rows instead of from the pool: it
 // rotates the new K row (and q, in registers) at position seq_len-1, writes K and V into their page slot -- the
 // append -- and folds the token's own term exp(q.k) v into the merge of the partials.  One workgroup per
-// (sequence, scheduled unit, q head): 128 lanes (one per output dimension) x S slices over the partials, as in
-// the combine kernel.  The appended rows carry the same bits the append kernel writes.
+// (sequence, scheduled unit, group of HB q heads): 32 lanes per head with four output dimensions each, x S slices
+// over the partials (thread layout below).  The appended rows carry the same bits the append kernel writes.
 template <typename T> __device__ __forceinline__ float pool_to_f32(T v) { return to_f32(v); }
 template <> __device__ __forceinline__ float pool_to_f32<e4m3_t>(e4m3_t v) {
     return __builtin_amdgcn_cvt_f32_fp8((int)v.bits, 0);
