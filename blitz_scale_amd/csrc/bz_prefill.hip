@@ -94,6 +94,16 @@ struct PrefillArgs {
     float sm_scale_log2;
 };
 
+// Keeps a value where it is computed: the compiler would otherwise sink the packs of the first half of an
+// iteration to their first use in the second and keep sixteen fp32 probabilities alive meanwhile.  (The pack
+// itself stays the compiler's: written as inline assembly, v_cvt_pk_bf16_f32 returned wrong values in the first
+// lanes of each half-wave -- the compiler adds wait states behind it that it cannot add behind an opaque
+// instruction.)
+__device__ __forceinline__ uint32_t pf_keep_here(uint32_t v) {
+    asm volatile("" : "+v"(v));
+    return v;
+}
+
 template <bool BF16> struct PfMma;
 template <> struct PfMma<false> {
     __device__ static __forceinline__ pf_f32x16 run(uint4 a, uint4 b, pf_f32x16 c) {
@@ -104,6 +114,7 @@ template <> struct PfMma<false> {
         const pf_f16x2 h = __builtin_convertvector(pf_f32x2{lo, hi}, pf_f16x2);
         return __builtin_bit_cast(uint32_t, h);
     }
+    __device__ static __forceinline__ uint32_t pack2_here(float lo, float hi) { return pf_keep_here(pack2(lo, hi)); }
     __device__ static __forceinline__ float lo(uint32_t w) { return (float)__builtin_bit_cast(pf_f16x2, w)[0]; }
     __device__ static __forceinline__ float hi(uint32_t w) { return (float)__builtin_bit_cast(pf_f16x2, w)[1]; }
 };
@@ -116,6 +127,7 @@ template <> struct PfMma<true> {
         const pf_bf16x2 b = __builtin_convertvector(pf_f32x2{lo, hi}, pf_bf16x2); // v_cvt_pk_bf16_f32, round to nearest even
         return __builtin_bit_cast(uint32_t, b);
     }
+    __device__ static __forceinline__ uint32_t pack2_here(float lo, float hi) { return pf_keep_here(pack2(lo, hi)); }
     __device__ static __forceinline__ float lo(uint32_t w) { return __uint_as_float(w << 16); }
     __device__ static __forceinline__ float hi(uint32_t w) { return __uint_as_float(w & 0xffff0000u); }
 };
@@ -445,6 +457,467 @@ __global__ __launch_bounds__(256, 2) void prefill_kernel(PrefillArgs a, const ch
     }
 }
 
+// ---------------------------------------------------------------------------------------------------------
+// The software-pipelined kernel.  One workgroup of 4 waves takes 128 consecutive q rows of one (request,
+// q head) as prefill_kernel does, two workgroups per CU; what differs is the loop.  K/V tiles are 32 tokens
+// and a wave's instruction stream for tile j is one interleaved sequence
+//     8 x { matrix: S(j+1) += K(j+1) Q^T step i | LDS: next operand | vector: exp, pack, row sum of S(j) }
+//     8 x { matrix: O += V(j)^T P(j)^T step i   | LDS: next operand }
+// so that a wave always has matrix instructions in flight while it does its vector work (a wave issues about one
+// instruction per five cycles whatever its kind, a matrix instruction keeps the pipe busy for 32, and the matrix
+// and vector instructions of the two waves of a SIMD share one issue port: the vector work has to sit in
+// the shadow of the matrix instructions of the same wave to be free).  Operands come from LDS through two rings
+// of four registers each, read four matrix instructions ahead of their use.  Tiles are copied global -> LDS
+// kSNK (K) and kSNV (V) tiles deep, which is about three tiles (two microseconds) ahead of their first read;
+// there is one workgroup barrier per tile, at the top of the iteration, where the tile that arrives next is
+// published and the buffers of the tiles just finished are handed back to the copies.  The steady state
+// (`full`) has no conditions in it; everything ragged or masked goes through `generic`.
+#ifndef BZ_PF_ABL
+#define BZ_PF_ABL 0 // timing experiments (results wrong): 1 no softmax arithmetic, 2 no LDS operand reads, 4 no tile copies, 8 no barriers in the steady state, 16 no matrix instructions
+#endif
+constexpr int kSN = 32;                      // kv tokens per tile
+constexpr int kSTile = kSN * 256;            // bytes of one K or V tile in LDS
+#ifndef BZ_PF_NK
+#define BZ_PF_NK 5
+#endif
+#ifndef BZ_PF_NV
+#define BZ_PF_NV 4
+#endif
+constexpr int kSNK = BZ_PF_NK, kSNV = BZ_PF_NV; // K and V tiles in flight per workgroup
+constexpr int kSLds = (kSNK + kSNV) * kSTile;   // 73 728 bytes per workgroup: K slots, then V slots
+
+__device__ __forceinline__ void lds_direct_load16x2(const char* uniform_base, uint32_t o0, uint32_t o1, uint32_t lds_addr) {
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\t"
+                 "global_load_lds_dwordx4 %1, %3\n\t"
+                 "global_load_lds_dwordx4 %2, %3 offset:1024"
+                 :
+                 : "s"(lds_addr), "v"(o0), "v"(o1), "s"(uniform_base)
+                 : "memory", "m0");
+}
+// workgroup barrier that the compiler moves no memory access across (it waits for nothing by itself)
+__device__ __forceinline__ void sp_barrier() {
+    __builtin_amdgcn_sched_barrier(0);
+    asm volatile("s_barrier" ::: "memory");
+    __builtin_amdgcn_sched_barrier(0);
+}
+// wait until at most `tiles` of this wave's tile copies (two instructions each) are still in flight
+__device__ __forceinline__ void sp_wait_copies(int tiles) {
+    __builtin_amdgcn_sched_barrier(0);
+    switch (tiles) {
+        case 0: __builtin_amdgcn_s_waitcnt(0x0F70); break;
+        case 1: __builtin_amdgcn_s_waitcnt(0x0F72); break;
+        case 2: __builtin_amdgcn_s_waitcnt(0x0F74); break;
+        case 3: __builtin_amdgcn_s_waitcnt(0x0F76); break;
+        case 4: __builtin_amdgcn_s_waitcnt(0x0F78); break;
+        case 5: __builtin_amdgcn_s_waitcnt(0x0F7A); break;
+        case 6: __builtin_amdgcn_s_waitcnt(0x0F7C); break;
+        default: __builtin_amdgcn_s_waitcnt(0x0F7E); break;
+    }
+    __builtin_amdgcn_sched_barrier(0);
+}
+// Copies are issued in pairs (K(i + kSNK), V(i + kSNV - 1)) at the top of iteration i, the first kSNK pairs
+// (i = -kSNK .. -1, tiles below 0 left out) in the prologue.  The tiles first read in iteration j are K(j+2) and
+// V(j): this counts the copies that exist (tile < n) behind the later of the two, up to those of iteration j-1.
+__device__ __forceinline__ int sp_copies_behind(int j, int n) {
+    const int pk = 2 * (j + 2 - kSNK), pv = 2 * (j + 1 - kSNV) + 1; // positions of K(j+2), V(j) in the issue order
+    int c = 0;
+    for (int pos = max(pk, pv) + 1; pos <= 2 * j - 1; ++pos) {
+        const int i = pos >> 1; // (arithmetic shift: positions may be negative in the first iterations)
+        const int tile = (pos & 1) ? i + kSNV - 1 : i + kSNK;
+        c += (tile >= 0 && tile < n) ? 1 : 0;
+    }
+    return c;
+}
+constexpr int sp_copies_behind_steady() { // the same when every tile exists
+    const int pk = 2 * (2 - kSNK), pv = 2 * (1 - kSNV) + 1;
+    return -1 - (pk > pv ? pk : pv);
+}
+__device__ __forceinline__ int sp_wrap(int x, int m) { return x >= m ? x - m : x; } // x < 2 m
+
+#ifdef BZ_PF_TIMING
+// Diagnostic build: every workgroup leaves the shader clock at a few points of its life in bz_pf_wg (read
+// through bz_pf_wg_table); the library proper compiles none of it.
+constexpr int kPftMaxWg = 32768;
+__device__ unsigned long long bz_pf_wg[kPftMaxWg * 8];
+#define BZ_PF_WG(k) do { __builtin_amdgcn_sched_barrier(0); pft[k] = __builtin_amdgcn_s_memtime(); __builtin_amdgcn_sched_barrier(0); } while (0)
+#else
+#define BZ_PF_WG(k) do { } while (0)
+#endif
+
+template <bool BF16, bool SPLIT_P, bool ROPE_Q>
+__global__ __launch_bounds__(256, 2) void prefill_sp_kernel(PrefillArgs a, const char* __restrict__ q_ptr,
+                                                            const char* __restrict__ k_ptr,
+                                                            const char* __restrict__ v_ptr) {
+    using M = PfMma<BF16>;
+    constexpr bool QSCALED = ROPE_Q; // q carries sm_scale * log2(e)
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+#ifdef BZ_PF_TIMING
+    unsigned long long pft[8];
+    pft[0] = __builtin_amdgcn_s_memtime();
+    pft[7] = __builtin_amdgcn_s_memrealtime();
+#endif
+
+    const PrefillItem it = a.items[blockIdx.x];
+    if (it.len <= 0) return;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wv = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int head = it.head;
+    const int Hq = (int)a.num_qo_heads, Hkv = (int)a.num_kv_heads;
+    const int kvh = head / (Hq / Hkv);
+    const int qn = lane & 31, h = lane >> 5;
+    const int L = it.len;
+    const int wave_q_lo = it.q0 + 32 * wv;
+    const int q_pos = wave_q_lo + qn;
+    const int kv_limit = a.causal ? min(L, it.q0 + kBM) : L; // tokens any row of this workgroup can see
+    const int n = (kv_limit + kSN - 1) / kSN;                // tiles of the job
+    // tiles this wave computes (causal: up to its diagonal tile; none for rows past the end of the request)
+    const int n_w = wave_q_lo >= L ? 0 : (a.causal ? min(n, wave_q_lo / kSN + 1) : n);
+    const int t_diag = a.causal ? wave_q_lo / kSN : 0x7fffffff;
+    const int kv_max = a.causal ? min(q_pos, L - 1) : L - 1; // last token this row may see
+
+    // ---- global -> LDS staging: wave wv moves rows 8wv .. 8wv+7 of a tile, two instructions of four 256-byte
+    // rows each for K and for V (chunk XOR patterns as in prefill_kernel)
+    const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) unsigned char*)smem;
+    const int r4 = lane >> 4, p16 = lane & 15;
+    const uint32_t row_stride = (uint32_t)Hkv * 256u;
+    uint32_t kcol[2], kfast[2], vfast[2];
+#pragma unroll
+    for (int i = 0; i < 2; ++i) kcol[i] = (uint32_t)((p16 ^ ((8 * wv + 4 * i + r4) & 15)) * 16);
+    const uint32_t vcol = (uint32_t)((p16 ^ BZ_VSWZ(r4)) * 16);
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+        kfast[i] = (uint32_t)(4 * i + r4) * row_stride + kcol[i] - (uint32_t)(i * 1024);
+        vfast[i] = (uint32_t)(4 * i + r4) * row_stride + vcol - (uint32_t)(i * 1024);
+    }
+    const size_t kv_row0 = ((size_t)it.tok0 * Hkv + kvh) * 256; // byte offset of the request's first K/V row
+    const char* const k_wave = k_ptr + kv_row0 + (size_t)(8 * wv) * row_stride;
+    const char* const v_wave = v_ptr + kv_row0 + (size_t)(8 * wv) * row_stride;
+    const uint32_t m0_wave = lds0 + (uint32_t)(8 * wv * 256);
+    const size_t tile_stride = (size_t)kSN * row_stride;
+    // a whole tile inside the request: one wave-uniform base, lane constants for the rest
+    auto issue_k_fast = [&](int t, int slot) __attribute__((always_inline)) {
+        if (BZ_PF_ABL & 4) return;
+        lds_direct_load16x2(k_wave + (size_t)t * tile_stride, kfast[0], kfast[1], m0_wave + (uint32_t)(slot * kSTile));
+    };
+    auto issue_v_fast = [&](int t, int slot) __attribute__((always_inline)) {
+        if (BZ_PF_ABL & 4) return;
+        lds_direct_load16x2(v_wave + (size_t)t * tile_stride, vfast[0], vfast[1], m0_wave + (uint32_t)((kSNK + slot) * kSTile));
+    };
+    auto issue_k = [&](int t, int slot) __attribute__((always_inline)) {
+        if ((t + 1) * kSN <= L) {
+            issue_k_fast(t, slot);
+        } else { // rows past the end of the request re-read its last row (masked later)
+            const char* base = k_ptr + kv_row0 + (size_t)t * tile_stride;
+            const uint32_t m0 = m0_wave + (uint32_t)(slot * kSTile);
+#pragma unroll
+            for (int i = 0; i < 2; ++i) {
+                const int row = min(t * kSN + 8 * wv + 4 * i + r4, L - 1) - t * kSN;
+                lds_direct_load16(base, (uint32_t)row * row_stride + kcol[i], m0 + i * 1024);
+            }
+        }
+    };
+    auto issue_v = [&](int t, int slot) __attribute__((always_inline)) {
+        if ((t + 1) * kSN <= L) {
+            issue_v_fast(t, slot);
+        } else {
+            const char* base = v_ptr + kv_row0 + (size_t)t * tile_stride;
+            const uint32_t m0 = m0_wave + (uint32_t)((kSNK + slot) * kSTile);
+#pragma unroll
+            for (int i = 0; i < 2; ++i) {
+                const int row = min(t * kSN + 8 * wv + 4 * i + r4, L - 1) - t * kSN;
+                lds_direct_load16(base, (uint32_t)row * row_stride + vcol, m0 + i * 1024);
+            }
+        }
+    };
+    // the copies of the prologue go first: the q rows, the angles and the job itself travel in their shadow
+#pragma unroll
+    for (int i = -kSNK; i < 0; ++i) {
+        if (i + kSNK < n) issue_k(i + kSNK, i + kSNK);
+        if (i + kSNV - 1 >= 0 && i + kSNV - 1 < n) issue_v(i + kSNV - 1, i + kSNV - 1);
+    }
+
+    // ---- Q rows as B operands: lane (q, h) holds q[q][16*ks + 8*h .. +7], ks = 0..7 (as in prefill_kernel)
+    uint4 qreg[8];
+    {
+        const size_t qtok = (size_t)it.tok0 + (size_t)min(q_pos, L - 1);
+        const char* qrow = q_ptr + (qtok * Hq + head) * 256;
+#pragma unroll
+        for (int ks = 0; ks < 8; ++ks) qreg[ks] = *reinterpret_cast<const uint4*>(qrow + ks * 32 + h * 16);
+        if constexpr (ROPE_Q) {
+            const float2* tab = a.rope_table + min(q_pos, L - 1);
+            float2 cs[32];
+#pragma unroll
+            for (int e = 0; e < 32; ++e) cs[e] = tab[(size_t)(16 * (e >> 3) + 8 * h + (e & 7)) * a.rope_pitch];
+#pragma unroll
+            for (int ks = 0; ks < 4; ++ks)
+#pragma unroll
+                for (int w = 0; w < 4; ++w) {
+                    const float2 c0 = cs[8 * ks + 2 * w], c1 = cs[8 * ks + 2 * w + 1];
+                    const uint32_t xw = pf_u4(qreg[ks], w), yw = pf_u4(qreg[ks + 4], w);
+                    float x0, y0, x1, y1;
+                    rope_pair(M::lo(xw), M::lo(yw), c0.x, c0.y, x0, y0);
+                    rope_pair(M::hi(xw), M::hi(yw), c1.x, c1.y, x1, y1);
+                    pf_u4(qreg[ks], w) = M::pack2(x0 * a.sm_scale_log2, x1 * a.sm_scale_log2);
+                    pf_u4(qreg[ks + 4], w) = M::pack2(y0 * a.sm_scale_log2, y1 * a.sm_scale_log2);
+                }
+        }
+    }
+
+    // Operand reads.  K: lane (row qn, half h) needs chunk 2 ks + h of its row for step ks, which sits at position
+    // (2 ks + h) ^ (qn % 16); V, through the transposing read: chunk 4 db + zl' of its row for d block db (see
+    // prefill_kernel).  Tiles are 256-byte aligned in LDS, so the step / block index is one XOR on a lane constant.
+    const uint32_t kbase = lds0 + (uint32_t)(qn * 256 + ((h ^ (qn & 15)) * 16));
+    uint32_t vbase;
+    {
+        const int srow = (lane & 15) >> 2;
+        const int zl = ((((lane >> 4) & 1) << 1) | ((lane & 3) >> 1)) ^ BZ_VSWZ(srow);
+        vbase = lds0 + (uint32_t)(kSNK * kSTile + (4 * h + srow) * 256 + zl * 16 + (lane & 1) * 8);
+    }
+    uint4 kring[4], vring[4]; // operands of the matrix instructions, read four instructions ahead of their use
+    if (BZ_PF_ABL & 2)
+        for (int i = 0; i < 4; ++i) kring[i] = vring[i] = make_uint4(lane, 2 * lane, 3, 4);
+    typedef uint32_t __attribute__((ext_vector_type(4))) pf_u32x4;
+    // (these issue the reads; the first use of a register waits for it)
+    auto read_k = [&](uint4& dst, uint32_t kb, int ks) __attribute__((always_inline)) { // kb: kbase + the tile's slot
+        if (BZ_PF_ABL & 2) { asm volatile("" : "+v"(dst.x)); return; }
+        const pf_u32x4 r = *reinterpret_cast<const pf_u32x4 __attribute__((address_space(3)))*>(
+            (const unsigned char __attribute__((address_space(3)))*)(uintptr_t)(kb ^ (uint32_t)(ks << 5)));
+        dst = make_uint4(r.x, r.y, r.z, r.w);
+    };
+    // operand i = 4 st + db of the second contraction (tokens 16 st .., d block db): two reads, rows +0 and +8
+    auto read_v = [&](uint4& dst, uint32_t vt, int i) __attribute__((always_inline)) { // vt: vbase + the tile's slot
+        if (BZ_PF_ABL & 2) { asm volatile("" : "+v"(dst.x)); return; }
+        const uint32_t vb = (vt ^ (uint32_t)((i & 3) << 6)) + (uint32_t)((i >> 2) * 16 * 256);
+        const pf_s16x4 t0 =
+            __builtin_amdgcn_ds_read_tr16_b64_v4i16((pf_s16x4 __attribute__((address_space(3)))*)(uintptr_t)(vb));
+        const pf_s16x4 t1 = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+            (pf_s16x4 __attribute__((address_space(3)))*)(uintptr_t)(vb + 8 * 256));
+        const uint2 w0 = __builtin_bit_cast(uint2, t0), w1 = __builtin_bit_cast(uint2, t1);
+        dst = make_uint4(w0.x, w0.y, w1.x, w1.y);
+    };
+    auto k_at = [&](int slot) __attribute__((always_inline)) { return kbase + (uint32_t)(slot * kSTile); };
+    auto v_at = [&](int slot) __attribute__((always_inline)) { return vbase + (uint32_t)(slot * kSTile); };
+
+    // ---- softmax state (see prefill_kernel: one reference maximum per row, moved only when it has to be)
+    float m_run = 0.f, l_run = 0.f; // l_run: this lane's half of the row sum
+    pf_f32x16 cinit;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) cinit[i] = 0.f;
+    pf_f32x16 acc[4]; // O^T: block db covers d = 32*db .. +31; element 4b+r is d = 32*db + 8b + 4h + r
+#pragma unroll
+    for (int db = 0; db < 4; ++db)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) acc[db][i] = 0.f;
+    pf_f32x16 s[2];     // scores of two tiles in flight: tile t lives in s[t % 2]
+    uint4 pa[2], pb[2]; // P^T operands of the two 16-token steps of a tile (head, and tail when SPLIT_P)
+    float psum = 0.f;
+
+    auto mask_tile = [&](int t, pf_f32x16& sc) __attribute__((always_inline)) {
+        // element 4b+r of a score block is token 32t + 8b + 4h + r
+        if (t == t_diag || (t + 1) * kSN > L) {
+#pragma unroll
+            for (int i = 0; i < 16; ++i) {
+                const int kv = t * kSN + 8 * (i >> 2) + 4 * h + (i & 3);
+                sc[i] = kv > kv_max ? -INFINITY : sc[i];
+            }
+        }
+    };
+    auto exp_of = [&](float x, float shift) __attribute__((always_inline)) {
+        return __builtin_amdgcn_exp2f(QSCALED ? x - shift : (x - shift) * a.sm_scale_log2);
+    };
+    auto take_pair = [&](float p0, float p1, int i) __attribute__((always_inline)) { // elements 2i, 2i+1 -> word i%4 of operand i/4
+        psum += p0 + p1;
+        const uint32_t hw = M::pack2_here(p0, p1);
+        pf_u4(pa[i >> 2], i & 3) = hw;
+        if (SPLIT_P) pf_u4(pb[i >> 2], i & 3) = M::pack2_here(p0 - M::lo(hw), p1 - M::hi(hw));
+    };
+    // The first half of an iteration: scores of the next tile into s[PAR ^ 1] (QK) from K at k1 (steps 0..3 are in
+    // the ring), probabilities of this tile from s[PAR] (EX), first V operands of this tile (at vj) into the ring.
+    // The exponentials of step i are consumed in step i + 1 (their latency is longer than one instruction).
+    auto first_half = [&](auto par_c, auto qk_c, auto ex_c, uint32_t k1, uint32_t vj) __attribute__((always_inline)) {
+        constexpr int PAR = decltype(par_c)::value;
+        constexpr bool QK = decltype(qk_c)::value, EX = decltype(ex_c)::value;
+        float e0 = 0.f, e1 = 0.f;
+        if (EX) psum = 0.f;
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            if (QK && !(BZ_PF_ABL & 16)) s[PAR ^ 1] = M::run(kring[i & 3], qreg[i], i == 0 ? cinit : s[PAR ^ 1]);
+            if (i < 4) read_k(kring[i], k1, i + 4);
+            else read_v(vring[i - 4], vj, i - 4);
+            if (EX && !(BZ_PF_ABL & 1)) {
+                const float n0 = exp_of(s[PAR][2 * i], 0.f), n1 = exp_of(s[PAR][2 * i + 1], 0.f);
+                if (i > 0) take_pair(e0, e1, i - 1);
+                e0 = n0;
+                e1 = n1;
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        if (EX && !(BZ_PF_ABL & 1)) take_pair(e0, e1, 7);
+        __builtin_amdgcn_sched_barrier(0);
+    };
+    // The second half: O += V^T P^T (PV), the rest of V (at vj) and the first K operands of the tile after the next
+    // (at k2) into the rings
+    auto second_half = [&](auto pv_c, uint32_t vj, uint32_t k2) __attribute__((always_inline)) {
+        constexpr bool PV = decltype(pv_c)::value;
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            if (PV && !(BZ_PF_ABL & 16)) {
+                acc[i & 3] = M::run(vring[i & 3], pa[i >> 2], acc[i & 3]);
+                if (SPLIT_P) acc[i & 3] = M::run(vring[i & 3], pb[i >> 2], acc[i & 3]);
+            }
+            if (i < 4) read_v(vring[i], vj, i + 4);
+            else read_k(kring[i - 4], k2, i - 4);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    };
+    // the reference maximum has to move (some score of tile j is 15 or more above it): rare, wave-uniform
+    auto move_maximum = [&](pf_f32x16& cur, pf_f32x16& next) __attribute__((always_inline)) {
+        float tmax = -INFINITY;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) tmax = fmaxf(tmax, cur[i]);
+        tmax = lane_max_xor32(tmax);
+        const float shift = fmaxf(tmax, 0.f);
+        const float alpha = __builtin_amdgcn_exp2f(QSCALED ? -shift : -shift * a.sm_scale_log2);
+        m_run += shift;
+        l_run *= alpha;
+#pragma unroll
+        for (int db = 0; db < 4; ++db)
+#pragma unroll
+            for (int i = 0; i < 16; ++i) acc[db][i] *= alpha;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+            cinit[i] = -m_run;
+            next[i] -= shift; // the next tile's scores were taken against the old reference
+        }
+        psum = 0.f;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) take_pair(exp_of(cur[2 * i], shift), exp_of(cur[2 * i + 1], shift), i);
+    };
+
+    // ---- prologue: scores of tile 0 set the reference maximum, the ring takes the first K operands of tile 1.
+    // The wait is for everything in flight (the copies were issued together, so they arrive together), which
+    // also tells the compiler, who counts only the loads it knows of, that the q registers are complete: it would
+    // otherwise wait for "its" loads, and with them for every copy in flight, inside the loop.
+    BZ_PF_WG(1);
+    sp_wait_copies(0);
+    sp_barrier();
+    BZ_PF_WG(2);
+    {
+        uint4 k0[8];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) read_k(k0[i], k_at(0), i);
+        if (n_w > 0) {
+#pragma unroll
+            for (int i = 0; i < 8; ++i) s[0] = M::run(k0[i], qreg[i], i == 0 ? cinit : s[0]);
+            mask_tile(0, s[0]);
+            float tmax = -INFINITY;
+#pragma unroll
+            for (int i = 0; i < 16; ++i) tmax = fmaxf(tmax, s[0][i]);
+            tmax = lane_max_xor32(tmax); // finite: token 0 is visible to every row
+            m_run = tmax;
+#pragma unroll
+            for (int i = 0; i < 16; ++i) {
+                s[0][i] -= tmax;
+                cinit[i] = -tmax;
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < 4; ++i) read_k(kring[i], k_at(1 % kSNK), i);
+    }
+    BZ_PF_WG(3);
+
+    // ---- the steady state: every tile touched exists, is whole and needs no mask
+    int kj = 0, vj = 0; // j % kSNK, j % kSNV
+    auto full = [&](int j, auto par_c) __attribute__((always_inline)) {
+        constexpr int PAR = decltype(par_c)::value;
+        sp_wait_copies(sp_copies_behind_steady()); // K(j+2) and V(j) have landed
+        if (!(BZ_PF_ABL & 8)) sp_barrier();
+        issue_k_fast(j + kSNK, kj);
+        issue_v_fast(j + kSNV - 1, sp_wrap(vj + kSNV - 1, kSNV));
+        first_half(par_c, std::true_type{}, std::true_type{}, k_at(sp_wrap(kj + 1, kSNK)), v_at(vj));
+        if (__any(!(psum < 32768.0f))) move_maximum(s[PAR], s[PAR ^ 1]);
+        l_run += psum;
+        second_half(std::true_type{}, v_at(vj), k_at(sp_wrap(kj + 2, kSNK)));
+        kj = sp_wrap(kj + 1, kSNK);
+        vj = sp_wrap(vj + 1, kSNV);
+    };
+    // ---- the same with every condition checked.  The operand reads are issued by every wave, also one that has
+    // nothing to compute, so that the registers have one definition per iteration.
+    auto generic = [&](int j, auto par_c) __attribute__((always_inline)) {
+        constexpr int PAR = decltype(par_c)::value;
+        const bool has_cur = j < n_w, has_next = j + 1 < n_w;
+        sp_wait_copies(sp_copies_behind(j, n));
+        sp_barrier();
+        if (j + kSNK < n) issue_k(j + kSNK, kj);
+        if (j + kSNV - 1 < n) issue_v(j + kSNV - 1, sp_wrap(vj + kSNV - 1, kSNV));
+        const uint32_t k1 = k_at(sp_wrap(kj + 1, kSNK)), k2 = k_at(sp_wrap(kj + 2, kSNK));
+        if (has_next) first_half(par_c, std::true_type{}, std::true_type{}, k1, v_at(vj));
+        else first_half(par_c, std::false_type{}, std::true_type{}, k1, v_at(vj)); // (harmless without a tile: p of stale scores, never used)
+        if (has_cur) {
+            if (__any(!(psum < 32768.0f))) move_maximum(s[PAR], s[PAR ^ 1]);
+            l_run += psum;
+            if (has_next) mask_tile(j + 1, s[PAR ^ 1]);
+            second_half(std::true_type{}, v_at(vj), k2);
+        } else {
+            second_half(std::false_type{}, v_at(vj), k2);
+        }
+        kj = sp_wrap(kj + 1, kSNK);
+        vj = sp_wrap(vj + 1, kSNV);
+    };
+    // full(j) needs: tiles j .. j+2 computed by this wave, tile j+1 unmasked, the tiles it copies whole and in range
+    const int j_full = min(min(n_w - 2, t_diag - 1), min(L / kSN, n) - kSNK);
+    int j = 0;
+    for (; j + 1 < j_full; j += 2) {
+        full(j, std::integral_constant<int, 0>{});
+        full(j + 1, std::integral_constant<int, 1>{});
+    }
+    BZ_PF_WG(4);
+    for (; j < n; j += 2) { // (j is even here)
+        generic(j, std::integral_constant<int, 0>{});
+        if (j + 1 < n) generic(j + 1, std::integral_constant<int, 1>{});
+    }
+    sp_barrier(); // nobody reads a tile any more: the epilogue takes their place
+    BZ_PF_WG(5);
+
+    // ---- epilogue: normalise, transpose the wave's 32 x 128 block through LDS (8 KiB per wave, 16-byte chunk c of
+    // row r at c ^ (r % 16)), store whole rows
+    const float l_row = lane_sum_xor32(l_run);
+    const float inv_l = l_row > 0.f ? 1.0f / l_row : 0.f;
+    unsigned char* o_lds = smem + wv * (32 * 256);
+#pragma unroll
+    for (int db = 0; db < 4; ++db)
+#pragma unroll
+        for (int b = 0; b < 4; ++b) {
+            const uint32_t w0 = M::pack2(acc[db][4 * b] * inv_l, acc[db][4 * b + 1] * inv_l);
+            const uint32_t w1 = M::pack2(acc[db][4 * b + 2] * inv_l, acc[db][4 * b + 3] * inv_l);
+            const int chunk = 4 * db + b; // d = 32 db + 8 b + 4 h .. +3: bytes 64 db + 16 b + 8 h
+            *reinterpret_cast<uint2*>(o_lds + qn * 256 + ((chunk ^ (qn & 15)) * 16) + 8 * h) = make_uint2(w0, w1);
+        }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+#pragma unroll
+    for (int ps = 0; ps < 8; ++ps) {
+        const int row = 4 * ps + (lane >> 4);
+        const int pos = wave_q_lo + row;
+        if (pos < L) {
+            const uint4 v = *reinterpret_cast<const uint4*>(o_lds + row * 256 + (((lane & 15) ^ (row & 15)) * 16));
+            char* orow = (char*)a.out + (((size_t)it.tok0 + pos) * Hq + head) * 256;
+            *reinterpret_cast<uint4*>(orow + (lane & 15) * 16) = v;
+        }
+    }
+#ifdef BZ_PF_TIMING
+    if (tid == 0 && blockIdx.x < kPftMaxWg) {
+        pft[6] = __builtin_amdgcn_s_memtime();
+        bz_pf_wg[blockIdx.x * 8 + 0] = ((unsigned long long)n << 32) | (unsigned)max(j_full, 0);
+        for (int i = 1; i < 7; ++i) bz_pf_wg[blockIdx.x * 8 + i] = pft[i] - pft[0];
+        bz_pf_wg[blockIdx.x * 8 + 7] = ((__builtin_amdgcn_s_memrealtime() - pft[7]) << 40) | (pft[7] & 0xffffffffffull);
+    }
+#endif
+}
+
 // ---- in-place RoPE of ragged q and k rows (used when the caller asks the attention call itself to rotate)
 struct RopeRaggedArgs {
     void* q;
@@ -678,6 +1151,38 @@ static int launch_prefill(const PrefillPlan* p, const PrefillArgs& a, const void
     return 0;
 }
 
+// Which attention kernel runs: the software-pipelined one unless BZ_PREFILL_KERNEL=single asks for prefill_kernel
+static bool prefill_use_sp() {
+    const char* e = getenv("BZ_PREFILL_KERNEL");
+    return !(e && strcmp(e, "single") == 0);
+}
+
+template <bool BF16, bool SPLIT_P, bool ROPE_Q>
+static int launch_prefill_sp(const PrefillPlan* p, const PrefillArgs& a, const void* q, const void* k, const void* v,
+                             hipStream_t s) {
+    auto kern = prefill_sp_kernel<BF16, SPLIT_P, ROPE_Q>;
+    static std::atomic<uint64_t> attr_done{0};
+    int dev = 0;
+    BZ_CHECK_HIP(hipGetDevice(&dev));
+    const uint64_t bit = 1ull << (dev & 63);
+    if (!(attr_done.load(std::memory_order_relaxed) & bit)) {
+        BZ_CHECK_HIP(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, kSLds));
+        attr_done.fetch_or(bit, std::memory_order_relaxed);
+    }
+    hipLaunchKernelGGL(kern, dim3(p->num_items), dim3(256), kSLds, s, a, (const char*)q, (const char*)k, (const char*)v);
+    BZ_LAUNCH_CHECK();
+    return 0;
+}
+
+#ifdef BZ_PF_TIMING
+// copies the table of the diagnostic build to the host: per workgroup 8 values (see prefill_sp_kernel)
+extern "C" int bz_pf_wg_table(unsigned long long* host, size_t count) {
+    if (count > sizeof(bz_pf_wg) / 8) count = sizeof(bz_pf_wg) / 8;
+    BZ_CHECK_HIP(hipMemcpyFromSymbol(host, HIP_SYMBOL(bz_pf_wg), count * 8, 0, hipMemcpyDeviceToHost));
+    return 0;
+}
+#endif
+
 extern "C" int bz_batch_prefill_ragged(bz_prefill_plan_t* plan_, void* q, const int32_t* qo_indptr, void* k, void* v,
                                        const int32_t* kv_indptr, void* out, int dtype, uint32_t batch_size,
                                        uint32_t num_qo_heads, uint32_t num_kv_heads, uint32_t head_dim, int causal,
@@ -728,6 +1233,14 @@ extern "C" int bz_batch_prefill_ragged(bz_prefill_plan_t* plan_, void* q, const 
     a.causal = causal ? 1 : 0;
     if (!(sm_scale > 0.f)) sm_scale = 1.0f / sqrtf((float)head_dim);
     a.sm_scale_log2 = sm_scale * 1.4426950408889634f;
+    if (prefill_use_sp()) {
+        if (rope_q) {
+            if (dtype == BZ_F16) return launch_prefill_sp<false, false, true>(p, a, q, k, v, s);
+            return launch_prefill_sp<true, true, true>(p, a, q, k, v, s);
+        }
+        if (dtype == BZ_F16) return launch_prefill_sp<false, false, false>(p, a, q, k, v, s);
+        return launch_prefill_sp<true, true, false>(p, a, q, k, v, s);
+    }
     if (rope_q) {
         if (dtype == BZ_F16) return launch_prefill<false, false, true>(p, a, q, k, v, s);
         return launch_prefill<true, true, true>(p, a, q, k, v, s);
