@@ -115,6 +115,10 @@ template <> struct PfMma<false> {
         return __builtin_bit_cast(uint32_t, h);
     }
     __device__ static __forceinline__ uint32_t pack2_here(float lo, float hi) { return pf_keep_here(pack2(lo, hi)); }
+    // acc + the two values of a packed word (v_dot2c_f32_f16 with ones: products and sum exact in fp32)
+    __device__ static __forceinline__ float add_pair(uint32_t w, float acc) {
+        return __builtin_amdgcn_fdot2(__builtin_bit_cast(pf_f16x2, w), pf_f16x2{(_Float16)1.0f, (_Float16)1.0f}, acc, false);
+    }
     __device__ static __forceinline__ float lo(uint32_t w) { return (float)__builtin_bit_cast(pf_f16x2, w)[0]; }
     __device__ static __forceinline__ float hi(uint32_t w) { return (float)__builtin_bit_cast(pf_f16x2, w)[1]; }
 };
@@ -128,6 +132,9 @@ template <> struct PfMma<true> {
         return __builtin_bit_cast(uint32_t, b);
     }
     __device__ static __forceinline__ uint32_t pack2_here(float lo, float hi) { return pf_keep_here(pack2(lo, hi)); }
+    __device__ static __forceinline__ float add_pair(uint32_t w, float acc) {
+        return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(pf_bf16x2, w), pf_bf16x2{(__bf16)1.0f, (__bf16)1.0f}, acc, false);
+    }
     __device__ static __forceinline__ float lo(uint32_t w) { return __uint_as_float(w << 16); }
     __device__ static __forceinline__ float hi(uint32_t w) { return __uint_as_float(w & 0xffff0000u); }
 };
@@ -478,13 +485,14 @@ __global__ __launch_bounds__(256, 2) void prefill_kernel(PrefillArgs a, const ch
 constexpr int kSN = 32;                      // kv tokens per tile
 constexpr int kSTile = kSN * 256;            // bytes of one K or V tile in LDS
 #ifndef BZ_PF_NK
-#define BZ_PF_NK 5
+#define BZ_PF_NK 4
 #endif
 #ifndef BZ_PF_NV
 #define BZ_PF_NV 4
 #endif
 constexpr int kSNK = BZ_PF_NK, kSNV = BZ_PF_NV; // K and V tiles in flight per workgroup
-constexpr int kSLds = (kSNK + kSNV) * kSTile;   // 73 728 bytes per workgroup: K slots, then V slots
+constexpr int kSLds = (kSNK + kSNV) * kSTile;   // 65 536 bytes per workgroup: K slots, then V slots
+static_assert(kSNK == 4 && kSNV == 4, "the steady state is unrolled over four slots");
 
 __device__ __forceinline__ void lds_direct_load16x2(const char* uniform_base, uint32_t o0, uint32_t o1, uint32_t lds_addr) {
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\t"
@@ -665,38 +673,48 @@ __global__ __launch_bounds__(256, 2) void prefill_sp_kernel(PrefillArgs a, const
 
     // Operand reads.  K: lane (row qn, half h) needs chunk 2 ks + h of its row for step ks, which sits at position
     // (2 ks + h) ^ (qn % 16); V, through the transposing read: chunk 4 db + zl' of its row for d block db (see
-    // prefill_kernel).  Tiles are 256-byte aligned in LDS, so the step / block index is one XOR on a lane constant.
-    const uint32_t kbase = lds0 + (uint32_t)(qn * 256 + ((h ^ (qn & 15)) * 16));
-    uint32_t vbase;
+    // prefill_kernel).  One address register per step / d block (complete LDS addresses inside slot 0); the slot and
+    // the token offsets of the V operands go into the instruction's offset field where they are compile-time constants.
+    uint32_t koff[8], voff[4];
     {
+        const int y = h ^ (qn & 15);
+#pragma unroll
+        for (int ks = 0; ks < 8; ++ks) {
+            koff[ks] = lds0 + (uint32_t)(qn * 256 + (((2 * ks) ^ y) * 16));
+            asm volatile("" : "+v"(koff[ks])); // keep the sum: the compiler would rebuild it at every use
+        }
         const int srow = (lane & 15) >> 2;
         const int zl = ((((lane >> 4) & 1) << 1) | ((lane & 3) >> 1)) ^ BZ_VSWZ(srow);
-        vbase = lds0 + (uint32_t)(kSNK * kSTile + (4 * h + srow) * 256 + zl * 16 + (lane & 1) * 8);
+#pragma unroll
+        for (int db = 0; db < 4; ++db) {
+            voff[db] = lds0 + (uint32_t)(kSNK * kSTile + (4 * h + srow) * 256 + ((((db << 2)) ^ zl) * 16) + (lane & 1) * 8);
+            asm volatile("" : "+v"(voff[db]));
+        }
     }
     uint4 kring[4], vring[4]; // operands of the matrix instructions, read four instructions ahead of their use
     if (BZ_PF_ABL & 2)
         for (int i = 0; i < 4; ++i) kring[i] = vring[i] = make_uint4(lane, 2 * lane, 3, 4);
     typedef uint32_t __attribute__((ext_vector_type(4))) pf_u32x4;
-    // (these issue the reads; the first use of a register waits for it)
-    auto read_k = [&](uint4& dst, uint32_t kb, int ks) __attribute__((always_inline)) { // kb: kbase + the tile's slot
+    // (these issue the reads; the first use of a register waits for it.  `soff`: byte offset of the tile's slot)
+    auto read_k = [&](uint4& dst, uint32_t soff, int ks) __attribute__((always_inline)) {
         if (BZ_PF_ABL & 2) { asm volatile("" : "+v"(dst.x)); return; }
         const pf_u32x4 r = *reinterpret_cast<const pf_u32x4 __attribute__((address_space(3)))*>(
-            (const unsigned char __attribute__((address_space(3)))*)(uintptr_t)(kb ^ (uint32_t)(ks << 5)));
+            (const unsigned char __attribute__((address_space(3)))*)(uintptr_t)(koff[ks]) + soff);
         dst = make_uint4(r.x, r.y, r.z, r.w);
     };
     // operand i = 4 st + db of the second contraction (tokens 16 st .., d block db): two reads, rows +0 and +8
-    auto read_v = [&](uint4& dst, uint32_t vt, int i) __attribute__((always_inline)) { // vt: vbase + the tile's slot
+    auto read_v = [&](uint4& dst, uint32_t soff, int i) __attribute__((always_inline)) {
         if (BZ_PF_ABL & 2) { asm volatile("" : "+v"(dst.x)); return; }
-        const uint32_t vb = (vt ^ (uint32_t)((i & 3) << 6)) + (uint32_t)((i >> 2) * 16 * 256);
-        const pf_s16x4 t0 =
-            __builtin_amdgcn_ds_read_tr16_b64_v4i16((pf_s16x4 __attribute__((address_space(3)))*)(uintptr_t)(vb));
-        const pf_s16x4 t1 = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-            (pf_s16x4 __attribute__((address_space(3)))*)(uintptr_t)(vb + 8 * 256));
+        typedef pf_s16x4 __attribute__((address_space(3)))* lds_s16x4_ptr;
+        const unsigned char __attribute__((address_space(3)))* vb =
+            (const unsigned char __attribute__((address_space(3)))*)(uintptr_t)(voff[i & 3]) + soff + (i >> 2) * 16 * 256;
+        const pf_s16x4 t0 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_ptr)(vb));
+        const pf_s16x4 t1 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_ptr)(vb + 8 * 256));
         const uint2 w0 = __builtin_bit_cast(uint2, t0), w1 = __builtin_bit_cast(uint2, t1);
         dst = make_uint4(w0.x, w0.y, w1.x, w1.y);
     };
-    auto k_at = [&](int slot) __attribute__((always_inline)) { return kbase + (uint32_t)(slot * kSTile); };
-    auto v_at = [&](int slot) __attribute__((always_inline)) { return vbase + (uint32_t)(slot * kSTile); };
+    auto k_at = [&](int slot) __attribute__((always_inline)) { return (uint32_t)(slot * kSTile); };
+    auto v_at = [&](int slot) __attribute__((always_inline)) { return (uint32_t)(slot * kSTile); };
 
     // ---- softmax state (see prefill_kernel: one reference maximum per row, moved only when it has to be)
     float m_run = 0.f, l_run = 0.f; // l_run: this lane's half of the row sum
@@ -725,11 +743,17 @@ __global__ __launch_bounds__(256, 2) void prefill_sp_kernel(PrefillArgs a, const
     auto exp_of = [&](float x, float shift) __attribute__((always_inline)) {
         return __builtin_amdgcn_exp2f(QSCALED ? x - shift : (x - shift) * a.sm_scale_log2);
     };
-    auto take_pair = [&](float p0, float p1, int i) __attribute__((always_inline)) { // elements 2i, 2i+1 -> word i%4 of operand i/4
-        psum += p0 + p1;
+    // elements 2i, 2i+1 -> word i%4 of operand i/4.  The row sum takes the probabilities as they enter the second
+    // contraction (rounded to the storage type; head + tail when SPLIT_P), one instruction per packed word.
+    auto take_pair = [&](float p0, float p1, int i) __attribute__((always_inline)) {
         const uint32_t hw = M::pack2_here(p0, p1);
         pf_u4(pa[i >> 2], i & 3) = hw;
-        if (SPLIT_P) pf_u4(pb[i >> 2], i & 3) = M::pack2_here(p0 - M::lo(hw), p1 - M::hi(hw));
+        psum = M::add_pair(hw, psum);
+        if (SPLIT_P) {
+            const uint32_t tw = M::pack2_here(p0 - M::lo(hw), p1 - M::hi(hw));
+            pf_u4(pb[i >> 2], i & 3) = tw;
+            psum = M::add_pair(tw, psum);
+        }
     };
     // The first half of an iteration: scores of the next tile into s[PAR ^ 1] (QK) from K at k1 (steps 0..3 are in
     // the ring), probabilities of this tile from s[PAR] (EX), first V operands of this tile (at vj) into the ring.
@@ -828,20 +852,37 @@ __global__ __launch_bounds__(256, 2) void prefill_sp_kernel(PrefillArgs a, const
     }
     BZ_PF_WG(3);
 
-    // ---- the steady state: every tile touched exists, is whole and needs no mask
-    int kj = 0, vj = 0; // j % kSNK, j % kSNV
-    auto full = [&](int j, auto par_c) __attribute__((always_inline)) {
-        constexpr int PAR = decltype(par_c)::value;
-        sp_wait_copies(sp_copies_behind_steady()); // K(j+2) and V(j) have landed
-        if (!(BZ_PF_ABL & 8)) sp_barrier();
-        issue_k_fast(j + kSNK, kj);
-        issue_v_fast(j + kSNV - 1, sp_wrap(vj + kSNV - 1, kSNV));
-        first_half(par_c, std::true_type{}, std::true_type{}, k_at(sp_wrap(kj + 1, kSNK)), v_at(vj));
+    // ---- the steady state: every tile touched exists, is whole and needs no mask.  SL = j % 4 is the slot of
+    // K(j) and of V(j), a compile-time constant (the loop is unrolled by four), so that LDS addresses are one
+    // register plus an immediate and the copies' LDS targets are constants as well.
+    int kj = 0, vj = 0; // j % kSNK, j % kSNV (used by `generic`)
+    const char* k_next = k_wave + (size_t)kSNK * tile_stride;       // K(j + kSNK)
+    const char* v_next = v_wave + (size_t)(kSNV - 1) * tile_stride; // V(j + kSNV - 1)
+    // COND: the copies and the count of copies in flight are looked at (the last few tiles of a job), otherwise
+    // the tiles copied are known to exist and to be whole.
+    auto full = [&](int j, auto par_c, auto sl_c, auto cond_c) __attribute__((always_inline)) {
+        constexpr int PAR = decltype(par_c)::value, SL = decltype(sl_c)::value;
+        constexpr bool COND = decltype(cond_c)::value;
+        if (!COND) {
+            sp_wait_copies(sp_copies_behind_steady()); // K(j+2) and V(j) have landed
+            if (!(BZ_PF_ABL & 8)) sp_barrier();
+            if (!(BZ_PF_ABL & 4)) {
+                lds_direct_load16x2(k_next, kfast[0], kfast[1], m0_wave + (uint32_t)(SL * kSTile));
+                lds_direct_load16x2(v_next, vfast[0], vfast[1], m0_wave + (uint32_t)((kSNK + (SL + kSNV - 1) % kSNV) * kSTile));
+            }
+            k_next += tile_stride;
+            v_next += tile_stride;
+        } else {
+            // behind K(j+2): V(j+1), K(j+3), V(j+2), of which only K(j+3) may be missing here
+            sp_wait_copies(2 + (j + 3 < n ? 1 : 0));
+            sp_barrier();
+            if (j + kSNK < n) issue_k(j + kSNK, SL);
+            if (j + kSNV - 1 < n) issue_v(j + kSNV - 1, (SL + kSNV - 1) % kSNV);
+        }
+        first_half(par_c, std::true_type{}, std::true_type{}, k_at((SL + 1) % kSNK), v_at(SL));
         if (__any(!(psum < 32768.0f))) move_maximum(s[PAR], s[PAR ^ 1]);
         l_run += psum;
-        second_half(std::true_type{}, v_at(vj), k_at(sp_wrap(kj + 2, kSNK)));
-        kj = sp_wrap(kj + 1, kSNK);
-        vj = sp_wrap(vj + 1, kSNV);
+        second_half(std::true_type{}, v_at(SL), k_at((SL + 2) % kSNK));
     };
     // ---- the same with every condition checked.  The operand reads are issued by every wave, also one that has
     // nothing to compute, so that the registers have one definition per iteration.
@@ -866,14 +907,43 @@ __global__ __launch_bounds__(256, 2) void prefill_sp_kernel(PrefillArgs a, const
         kj = sp_wrap(kj + 1, kSNK);
         vj = sp_wrap(vj + 1, kSNV);
     };
-    // full(j) needs: tiles j .. j+2 computed by this wave, tile j+1 unmasked, the tiles it copies whole and in range
-    const int j_full = min(min(n_w - 2, t_diag - 1), min(L / kSN, n) - kSNK);
+    // full needs: tiles j .. j+2 computed by this wave and tile j+1 unmasked; without COND also the tiles it copies
+    // whole and in range
+    const int j_cond = min(n_w - 2, t_diag - 1);
+    const int j_full = min(j_cond, min(L / kSN, n) - kSNK);
+    const std::integral_constant<int, 0> c0{};
+    const std::integral_constant<int, 1> c1{};
+    const std::integral_constant<int, 2> c2{};
+    const std::integral_constant<int, 3> c3{};
     int j = 0;
-    for (; j + 1 < j_full; j += 2) {
-        full(j, std::integral_constant<int, 0>{});
-        full(j + 1, std::integral_constant<int, 1>{});
+    for (; j + 3 < j_full; j += 4) {
+        full(j, c0, c0, std::false_type{});
+        full(j + 1, c1, c1, std::false_type{});
+        full(j + 2, c0, c2, std::false_type{});
+        full(j + 3, c1, c3, std::false_type{});
     }
+    for (; j + 3 < j_cond; j += 4) {
+        full(j, c0, c0, std::true_type{});
+        full(j + 1, c1, c1, std::true_type{});
+        full(j + 2, c0, c2, std::true_type{});
+        full(j + 3, c1, c3, std::true_type{});
+    }
+    if (j < j_cond) { // (j is a multiple of four here: up to three more, slots known)
+        full(j, c0, c0, std::true_type{});
+        if (++j < j_cond) {
+            full(j, c1, c1, std::true_type{});
+            if (++j < j_cond) {
+                full(j, c0, c2, std::true_type{});
+                ++j;
+            }
+        }
+    }
+    kj = vj = j & 3;
     BZ_PF_WG(4);
+    if ((j & 1) && j < n) {
+        generic(j, c1);
+        ++j;
+    }
     for (; j < n; j += 2) { // (j is even here)
         generic(j, std::integral_constant<int, 0>{});
         if (j + 1 < n) generic(j + 1, std::integral_constant<int, 1>{});
@@ -911,8 +981,13 @@ __global__ __launch_bounds__(256, 2) void prefill_sp_kernel(PrefillArgs a, const
 #ifdef BZ_PF_TIMING
     if (tid == 0 && blockIdx.x < kPftMaxWg) {
         pft[6] = __builtin_amdgcn_s_memtime();
-        bz_pf_wg[blockIdx.x * 8 + 0] = ((unsigned long long)n << 32) | (unsigned)max(j_full, 0);
-        for (int i = 1; i < 7; ++i) bz_pf_wg[blockIdx.x * 8 + i] = pft[i] - pft[0];
+        // HW_ID: wave 3:0, simd 5:4, pipe 7:6, cu 11:8, sh 12, se 15:13 (...); XCC_ID: 3:0
+        unsigned hw = 0, xcc = 0;
+        asm volatile("s_getreg_b32 %0, hwreg(HW_REG_HW_ID)" : "=s"(hw));
+        asm volatile("s_getreg_b32 %0, hwreg(HW_REG_XCC_ID)" : "=s"(xcc));
+        bz_pf_wg[blockIdx.x * 8 + 0] = ((unsigned long long)n << 32) | (unsigned)max(j_cond, 0);
+        bz_pf_wg[blockIdx.x * 8 + 2] = ((unsigned long long)(xcc & 15) << 32) | hw; // (replaces the K0-landed stamp)
+        for (int i = 1; i < 7; ++i) if (i != 2) bz_pf_wg[blockIdx.x * 8 + i] = pft[i] - pft[0];
         bz_pf_wg[blockIdx.x * 8 + 7] = ((__builtin_amdgcn_s_memrealtime() - pft[7]) << 40) | (pft[7] & 0xffffffffffull);
     }
 #endif
