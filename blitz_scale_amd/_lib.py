@@ -14,6 +14,7 @@ BZ_F16, BZ_BF16, BZ_E4M3, BZ_F32 = 0, 1, 2, 3
 BZ_ROPE_NONE, BZ_ROPE_Q_ONLY, BZ_ROPE_FULL = 0, 1, 2
 BZ_LAYOUT_NHD, BZ_LAYOUT_HND = 0, 1
 BZ_NUM_TOKENS_FROM_INDPTR = 0xFFFFFFFF
+BZ_PREFILL_BF16_WIDEN_V, BZ_PREFILL_BF16_HEAD_TAIL = 0, 1
 BZ_ERR_BAD_ARG, BZ_ERR_UNSUPPORTED, BZ_ERR_WORKSPACE, BZ_ERR_NOT_PLANNED, BZ_ERR_NO_PAGES = 10001, 10002, 10003, 10004, 10005
 
 
@@ -66,6 +67,7 @@ SIGNATURES = {
     "bz_prefill_plan": (_i32, [_vp, _vp, _sz, _vp, _sz, _vp, _vp, _u32, _u32, _u32, _u32, _u32, _vp]),
     "bz_prefill_plan_workspace": (_i32, [_vp, _vp, _vp, _u32, _u32, _u32, _u32, C.POINTER(_sz), C.POINTER(_sz)]),
     "bz_prefill_plan_host_schedule": (_i32, [_vp, C.POINTER(_vp), C.POINTER(_sz), C.POINTER(_u32)]),
+    "bz_prefill_plan_set_bf16_mode": (_i32, [_vp, _i32]),
     "bz_batch_prefill_ragged": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i32, _u32, _u32, _u32, _u32, _i32, _i32,
                                        _f32, _f32, _vp]),
     "bz_store_prefill_kv": (_i32, [_kvp, _vp, _vp, _i32, _vp, _u32, _vp, _u32, _i32, _f32, _vp, _vp, _vp]),

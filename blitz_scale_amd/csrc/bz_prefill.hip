@@ -3,13 +3,13 @@
 // worker.  head_dim 128, f16 or bf16, any number of q heads per kv head.
 //
 // One workgroup of 4 waves takes 128 consecutive q rows of one (request, q head); wave w owns rows
-// 32w..32w+31.  K/V tiles of 64 tokens are staged through double-buffered LDS and shared by the four
+// 32w..32w+31.  K/V tiles of 32 tokens travel global -> LDS four tiles deep and are shared by the four
 // waves.  Both contractions are issued "transposed" on v_mfma_f32_32x32x16:
 //     S^T[kv][q] = K[kv][:] . Q[q][:]      (A = K tile from LDS,      B = Q rows from registers)
 //     O^T[d][q]  = V^T[d][kv] . P^T[kv][q] (A = V tile, transposed LDS read, B = P from registers)
 // so that in both results a lane's column index is its own q row: the softmax statistics, the
-// rescaling of O and the P operand of the second contraction are all lane-local (one shuffle per
-// tile joins the two half-waves).
+// rescaling of O and the P operand of the second contraction are all lane-local (the two half-waves of a
+// row are joined once, at the end).
 #include <algorithm>
 #include <atomic>
 #include <cmath>
@@ -32,10 +32,7 @@ typedef __attribute__((ext_vector_type(2))) float pf_f32x2;
 typedef __attribute__((ext_vector_type(16))) float pf_f32x16;
 typedef __attribute__((ext_vector_type(4))) short pf_s16x4;
 
-constexpr int kBM = 128;       // q rows per workgroup
-constexpr int kBN = 64;        // kv tokens per tile
-constexpr int kTile = kBN * 256; // bytes of one K or V tile in LDS (rows unpadded); LDS holds K0 K1 V0 V1
-constexpr int kORow = 272;       // LDS row stride of the output transpose in the epilogue (256 B + 16)
+constexpr int kBM = 128; // q rows per workgroup
 
 // 16 bytes per lane from global memory straight into LDS: lane l's data lands at lds_addr + 16*l.
 // The compiler does not know that this is a load (it would otherwise wait for every such load before
@@ -44,20 +41,6 @@ __device__ __forceinline__ void lds_direct_load16(const char* uniform_base, uint
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
                  :
                  : "s"(lds_addr), "v"(lane_offset), "s"(uniform_base)
-                 : "memory", "m0");
-}
-
-// Four such loads into four consecutive KiB of LDS with one M0 value: the instruction offset moves the
-// LDS address and the global address alike, so lane offset i is passed less i KiB.
-__device__ __forceinline__ void lds_direct_load16x4(const char* uniform_base, uint32_t o0, uint32_t o1, uint32_t o2,
-                                                    uint32_t o3, uint32_t lds_addr) {
-    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\t"
-                 "global_load_lds_dwordx4 %1, %5\n\t"
-                 "global_load_lds_dwordx4 %2, %5 offset:1024\n\t"
-                 "global_load_lds_dwordx4 %3, %5 offset:2048\n\t"
-                 "global_load_lds_dwordx4 %4, %5 offset:3072"
-                 :
-                 : "s"(lds_addr), "v"(o0), "v"(o1), "v"(o2), "v"(o3), "s"(uniform_base)
                  : "memory", "m0");
 }
 
@@ -70,6 +53,7 @@ struct PrefillItem { // one workgroup's job, in launch order
 
 struct PrefillPlan {
     bool planned = false;
+    bool bf16_head_tail = false; // bf16: probabilities as head + tail of bf16 instead of V widened to f16 (bz_prefill_plan_set_bf16_mode)
     uint32_t batch_size = 0, num_qo_heads = 0, num_kv_heads = 0, head_dim = 0, num_items = 0;
     uint32_t total_tokens = 0, max_len = 0;
     const PrefillItem* items_d = nullptr;
@@ -141,347 +125,41 @@ template <> struct PfMma<true> {
 
 __device__ __forceinline__ uint32_t& pf_u4(uint4& v, int i) { return reinterpret_cast<uint32_t*>(&v)[i]; }
 
-// SPLIT_P: the probabilities enter the second contraction as head + tail of the storage type (two
-// MFMAs), used for bf16 whose 8-bit significand alone would eat the error budget.
 // XOR applied to the 16-byte chunk index of V rows in LDS, by row % 4: 0, 4, 10, 14 (see the staging comment)
 #define BZ_VSWZ(r) (((r) << 2) ^ (((r) >> 1) << 1))
-// ROPE_Q: the q rows are rotated in registers on their way in (position = offset inside the request, angles
-// from a table), so q is read once and never written; k is expected rotated.
-template <bool BF16, bool SPLIT_P, bool ROPE_Q>
-__global__ __launch_bounds__(256, 2) void prefill_kernel(PrefillArgs a, const char* __restrict__ q_ptr,
-                                                         const char* __restrict__ k_ptr,
-                                                         const char* __restrict__ v_ptr) {
-    using M = PfMma<BF16>;
-    constexpr bool QSCALED = ROPE_Q; // q carries sm_scale * log2(e) (see the prologue)
-    extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
-
-    const PrefillItem it = a.items[blockIdx.x];
-    if (it.len <= 0) return;
-    const int head = it.head;
-    const int Hq = (int)a.num_qo_heads, Hkv = (int)a.num_kv_heads;
-    const int kvh = head / (Hq / Hkv);
-    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
-    const int qn = lane & 31; // q row of this lane inside the wave's 32 rows
-    const int h = lane >> 5;  // half-wave: which 8 of the 16 contraction indices of an MFMA step
-    const int L = it.len;
-    const int q_pos = it.q0 + 32 * wave + qn; // position inside the request (may be >= L: masked at the end)
-    const int wave_q_lo = it.q0 + 32 * wave, wave_q_hi = wave_q_lo + 31;
-
-    // ---- Q rows as B operands: lane (q, h) holds q[q][16*ks + 8*h .. +7], ks = 0..7
-    uint4 qreg[8];
-    {
-        const size_t qtok = (size_t)it.tok0 + (size_t)min(q_pos, L - 1);
-        const char* qrow = q_ptr + (qtok * Hq + head) * 256;
-#pragma unroll
-        for (int ks = 0; ks < 8; ++ks) qreg[ks] = *reinterpret_cast<const uint4*>(qrow + ks * 32 + h * 16);
-        if constexpr (ROPE_Q) {
-            // d = 16 ks + 8 h + e (ks < 4) pairs with d + 64, which this lane holds at step ks + 4.  The table is
-            // laid out pair by pair, so the 32 rows of a half-wave read 256 consecutive bytes per pair.
-            const float2* tab = a.rope_table + min(q_pos, L - 1);
-            float2 cs[32];
-#pragma unroll
-            for (int e = 0; e < 32; ++e) cs[e] = tab[(size_t)(16 * (e >> 3) + 8 * h + (e & 7)) * a.rope_pitch];
-#pragma unroll
-            for (int ks = 0; ks < 4; ++ks)
-#pragma unroll
-                for (int w = 0; w < 4; ++w) {
-                    const float2 c0 = cs[8 * ks + 2 * w], c1 = cs[8 * ks + 2 * w + 1]; // pairs i = 16 ks + 8 h + 2 w, i + 1
-                    const uint32_t xw = pf_u4(qreg[ks], w), yw = pf_u4(qreg[ks + 4], w);
-                    float x0, y0, x1, y1;
-                    rope_pair(M::lo(xw), M::lo(yw), c0.x, c0.y, x0, y0);
-                    rope_pair(M::hi(xw), M::hi(yw), c1.x, c1.y, x1, y1);
-                    // (the softmax scale rides on the one rounding of the rotated row, see below)
-                    pf_u4(qreg[ks], w) = M::pack2(x0 * a.sm_scale_log2, x1 * a.sm_scale_log2);
-                    pf_u4(qreg[ks + 4], w) = M::pack2(y0 * a.sm_scale_log2, y1 * a.sm_scale_log2);
-                }
-        }
-        // Rows rotated here carry the softmax scale (times log2 e) in their one rounding: the scores then come
-        // out of the matrix pipe as base-2 logits and go into exp2 as they are, one vector instruction less per
-        // score.  Rows that arrive as they are keep their bits -- a second rounding would move a logit of
-        // magnitude 30 by 30 * 2^-12 (f16) or 30 * 2^-9 (bf16), visibly more than the stated tolerance -- and the
-        // scale is applied to the score instead.
-    }
-
-    const int kv_limit = a.causal ? min(L, it.q0 + kBM) : L; // tokens any row of this workgroup can see
-    const int n_tiles = (kv_limit + kBN - 1) / kBN;
-    // tiles this wave computes: under the causal mask its rows see nothing past token wave_q_hi; a wave whose
-    // rows all lie past the end of the request (last q tile of a request) computes nothing at all, it only
-    // takes part in the copies and barriers
-    const int n_w = wave_q_lo >= L ? 0 : (a.causal ? min(n_tiles, wave_q_hi / kBN + 1) : n_tiles);
-    // the last tile of a wave whose rows start on a tile boundary (causal): its second 32 tokens lie past
-    // every row of the wave, so only the first block is computed
-    const int t_half = (a.causal && (wave_q_lo % kBN) == 0) ? wave_q_lo / kBN : -1;
-
-    // ---- global -> LDS staging of a K/V tile with LDS-direct loads (no registers, no LDS stores): a
-    // wave instruction moves 64 x 16 B to 1 KiB of consecutive LDS, i.e. 4 unpadded 256-byte rows; wave w
-    // moves rows 16w .. 16w+15 of the tile with four instructions each for K and V.  What keeps the
-    // operand reads free of bank conflicts is an XOR on the 16-byte column chunk instead of padding:
-    //   K: chunk c of row r sits at position c ^ (r % 16)      (8 lanes read 8 rows, one chunk each)
-    //   V: chunk c of row r sits at position c ^ g(r % 4), g = 0, 4, 10, 14.  The transposing read takes 8 B
-    //      per lane; a 16-lane group reads 4 rows x 32 B and two groups (32 lanes, 4 rows x 64 B) go through
-    //      the 64 banks together, so the 8 (row, group) pieces must land in 8 different 32-byte bank groups
-    //      (with c ^ 2*(r % 4), enough for 32 banks, the hardware counted a conflict on a third of the LDS
-    //      cycles; with g, 3.5 %)
-    // and a lane of the copy simply fetches the chunk that belongs at its position.  Rows past the end
-    // of the request re-read its last row (valid memory; masked later).
-    const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) unsigned char*)smem;
-    const int wv = __builtin_amdgcn_readfirstlane(wave);
-    const int r4 = lane >> 4, p16 = lane & 15;
-    const uint32_t row_stride = (uint32_t)Hkv * 256u;
-    uint32_t kcol[4], kfast[4], vfast[4];
-#pragma unroll
-    for (int i = 0; i < 4; ++i) kcol[i] = (uint32_t)((p16 ^ ((4 * i + r4) & 15)) * 16);
-    const uint32_t vcol = (uint32_t)((p16 ^ BZ_VSWZ(r4)) * 16);
-#pragma unroll
-    for (int i = 0; i < 4; ++i) { // lane offsets of copy i inside the wave's 16 rows when no row needs clamping,
-                                  // less the i KiB that the instruction offset of the grouped copy adds back
-        kfast[i] = (uint32_t)(4 * i + r4) * row_stride + kcol[i] - (uint32_t)(i * 1024);
-        vfast[i] = (uint32_t)(4 * i + r4) * row_stride + vcol - (uint32_t)(i * 1024);
-    }
-    auto issue_tile = [&](int t, int buf) __attribute__((always_inline)) {
-        const uint32_t m0k = lds0 + (uint32_t)(buf * kTile + 16 * wv * 256);
-        if ((t + 1) * kBN <= L) { // the whole tile lies inside the request: one wave-uniform base for K, one for V
-            const size_t base = (((size_t)it.tok0 + (size_t)(t * kBN + 16 * wv)) * Hkv + kvh) * 256;
-            lds_direct_load16x4(k_ptr + base, kfast[0], kfast[1], kfast[2], kfast[3], m0k);
-            lds_direct_load16x4(v_ptr + base, vfast[0], vfast[1], vfast[2], vfast[3], m0k + 2 * kTile);
-        } else {
-            const size_t base = (((size_t)it.tok0 + (size_t)t * kBN) * Hkv + kvh) * 256;
-#pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                const int row = min(t * kBN + 16 * wv + 4 * i + r4, L - 1) - t * kBN;
-                lds_direct_load16(k_ptr + base, (uint32_t)row * row_stride + kcol[i], m0k + i * 1024);
-                lds_direct_load16(v_ptr + base, (uint32_t)row * row_stride + vcol, m0k + 2 * kTile + i * 1024);
-            }
-        }
-    };
-    // the copies of this wave have landed; after the barrier so have everyone's
-    auto publish = [&]() __attribute__((always_inline)) {
-        __builtin_amdgcn_s_waitcnt(0x0F70); // vmcnt(0)
-        __syncthreads();
-    };
-
-    // Online softmax without a maximum per tile.  The scores leave the matrix pipe already shifted by the
-    // reference maximum m_run of their row: the first score step of a block accumulates onto `cinit`, a block
-    // of registers that holds -m_run, so p = exp2(score) needs no further arithmetic.  m_run is set from the
-    // first tile (in the units of the scores: base-2 logits when q carries the scale) and moved only when it has to be: a tile's probabilities are computed on the assumption that
-    // no score exceeds m_run by 15 or more (p < 2^15 fits the 16-bit operand of the second contraction, and
-    // fp32 sums hold it easily); the row sums, which are needed anyway, tell whether the assumption held
-    // (every p < 2^15 if their sum is), and a wave for which it did not takes the tile's maximum, moves m_run,
-    // rescales its accumulators and computes the tile's probabilities again.  m_run never exceeds the true
-    // running maximum, so the largest probability of a row so far is always at least 1.
-    float m_run = 0.f, l_run = 0.f;
-    pf_f32x16 cinit;
-#pragma unroll
-    for (int i = 0; i < 16; ++i) cinit[i] = 0.f;
-    pf_f32x16 acc[4]; // O^T: block db covers d = 32*db .. +31; element 4b+r is d = 32*db + 8b + 4h + r
-#pragma unroll
-    for (int db = 0; db < 4; ++db)
-#pragma unroll
-        for (int i = 0; i < 16; ++i) acc[db][i] = 0.f;
-
-    issue_tile(0, 0);
-    publish();
-
-    // operand read offsets inside a tile (lane constants).  K: row qn (+32 for the second block), chunk
-    // 2*ks + h.  V, through the transposing LDS read: a 16-lane group fetches 4 token rows x 16 d columns
-    // and every lane ends up with the 4 tokens of its own d column; the lane's row is 4h + srow (+16 per
-    // step, +8 for the second half) and its chunk 4*db + 2*(lane/16 % 2) + (lane % 4)/2.
-    uint32_t koff[8], voff[4];
-    {
-        const int y = h ^ (qn & 15);
-#pragma unroll
-        for (int ks = 0; ks < 8; ++ks) {
-            koff[ks] = lds0 + (uint32_t)(qn * 256 + (((2 * ks) ^ y) * 16));
-            asm volatile("" : "+v"(koff[ks])); // keep the sum: the compiler would re-add the base on every tile
-        }
-        const int srow = (lane & 15) >> 2;
-        const int zl = ((((lane >> 4) & 1) << 1) | ((lane & 3) >> 1)) ^ BZ_VSWZ(srow);
-#pragma unroll
-        for (int db = 0; db < 4; ++db) {
-            voff[db] = lds0 + (uint32_t)((4 * h + srow) * 256 + ((((db << 2)) ^ zl) * 16) + (lane & 1) * 8);
-            asm volatile("" : "+v"(voff[db]));
-        }
-    }
-
-    // the arithmetic of tile t (K/V in LDS buffer BUF = t % 2, a compile-time constant so that the buffer
-    // and step offsets fold into the immediate field of the LDS reads)
-    auto compute_tile = [&](int t, auto which, auto half_c) __attribute__((always_inline)) {
-        constexpr int BUF = decltype(which)::value;
-        constexpr bool HALF = decltype(half_c)::value; // only the first 32 tokens of the tile (see t_half)
-        constexpr int NS = HALF ? 8 : 16;              // score steps, and steps of the second contraction
-        constexpr int NKB = HALF ? 1 : 2;              // 32-token blocks
-        const int kv0 = t * kBN;
-        {
-            // Both contractions are scheduled by hand.  An LDS read takes several times as long as a
-            // matrix instruction, so the operand reads run kDK / kDV matrix instructions ahead of their
-            // use (rings ka / va); scheduling barriers keep the steps in this order.
-            constexpr int kDK = 4, kDV = 4;
-            uint4 ka[kDK], va[kDV];
-            auto k_read = [&](int i) __attribute__((always_inline)) { // operand of score step i: block i/8, d step i%8
-                // (koff / voff hold complete LDS addresses, so the rest is the instruction's immediate offset)
-                const unsigned char __attribute__((address_space(3)))* kb =
-                    (const unsigned char __attribute__((address_space(3)))*)(uintptr_t)koff[i & 7];
-                typedef uint32_t __attribute__((ext_vector_type(4))) pf_u32x4;
-                const pf_u32x4 r = *reinterpret_cast<const pf_u32x4 __attribute__((address_space(3)))*>(
-                    kb + (BUF * kTile + (i >> 3) * 32 * 256));
-                return make_uint4(r.x, r.y, r.z, r.w);
-            };
-            auto v_read = [&](int i) __attribute__((always_inline)) { // operand of step i: tokens 16*(i/4).., d block i%4
-                const uint32_t vb = voff[i & 3] + (uint32_t)((2 + BUF) * kTile + (i >> 2) * 16 * 256);
-                const pf_s16x4 t0 =
-                    __builtin_amdgcn_ds_read_tr16_b64_v4i16((pf_s16x4 __attribute__((address_space(3)))*)(uintptr_t)(vb));
-                const pf_s16x4 t1 = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-                    (pf_s16x4 __attribute__((address_space(3)))*)(uintptr_t)(vb + 8 * 256));
-                const uint2 w0 = __builtin_bit_cast(uint2, t0), w1 = __builtin_bit_cast(uint2, t1);
-                return make_uint4(w0.x, w0.y, w1.x, w1.y);
-            };
-            // ---- S^T = K Q^T: two 32-token blocks, eight 16-wide steps over d
-            pf_f32x16 s[2];
-#pragma unroll
-            for (int i = 0; i < kDK; ++i) ka[i] = k_read(i);
-            __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-            for (int i = 0; i < NS; ++i) {
-                if ((i & 7) == 0) {
-                    s[i >> 3] = M::run(ka[i % kDK], qreg[i & 7], cinit);
-                } else {
-                    s[i >> 3] = M::run(ka[i % kDK], qreg[i & 7], s[i >> 3]);
-                }
-                if (i + kDK < NS) ka[i % kDK] = k_read(i + kDK);
-                else va[i + kDK - NS] = v_read(i + kDK - NS); // the first V operands arrive during the softmax
-                __builtin_amdgcn_sched_barrier(0);
-            }
-            static_assert(kDV == kDK, "the tail of the score steps fills the whole V ring");
-            // ---- mask.  Element 4b+r of block kb is token kv0 + 32kb + 8b + 4h + r.
-            const bool need_mask = HALF || (a.causal && kv0 + kBN - 1 > wave_q_lo) || (kv0 + kBN > L);
-            if (need_mask) { // wave-uniform; selects, not branches, per element
-                const int kv_max = a.causal ? min(q_pos, L - 1) : L - 1; // last token this row may see
-#pragma unroll
-                for (int kb = 0; kb < NKB; ++kb)
-#pragma unroll
-                    for (int i = 0; i < 16; ++i) {
-                        const int kv = kv0 + 32 * kb + 8 * (i >> 2) + 4 * h + (i & 3);
-                        s[kb][i] = kv > kv_max ? -INFINITY : s[kb][i];
-                    }
-            }
-            float psum;
-            uint4 pa[4], pb[4]; // P^T operands of the four 16-token steps (head, and tail when SPLIT_P)
-            auto probabilities = [&](float shift) __attribute__((always_inline)) { // p = exp2(score - shift)
-                psum = 0.f;
-#pragma unroll
-                for (int st = 0; st < 2 * NKB; ++st) {
-                    const int kb = st >> 1, b0 = 2 * (st & 1);
-#pragma unroll
-                    for (int w = 0; w < 4; ++w) { // elements e = 2w, 2w+1 of the operand: block b0 + e/4, r = e%4
-                        const int i0 = 4 * (b0 + (w >> 1)) + 2 * (w & 1);
-                        const float p0 = __builtin_amdgcn_exp2f(QSCALED ? s[kb][i0] - shift : (s[kb][i0] - shift) * a.sm_scale_log2);
-                        const float p1 = __builtin_amdgcn_exp2f(QSCALED ? s[kb][i0 + 1] - shift : (s[kb][i0 + 1] - shift) * a.sm_scale_log2);
-                        psum += p0 + p1;
-                        const uint32_t hw = M::pack2(p0, p1);
-                        pf_u4(pa[st], w) = hw;
-                        if (SPLIT_P) pf_u4(pb[st], w) = M::pack2(p0 - M::lo(hw), p1 - M::hi(hw));
-                    }
-                }
-            };
-            bool moved = t == 0; // the first tile sets the reference maximum (token 0 is visible to every row)
-            if (!moved) {
-                probabilities(0.f);
-                moved = __any(!(psum < 32768.0f)); // some score is 15 or more above m_run (or the sum is not finite)
-            }
-            if (moved) { // wave-uniform, rare after the first tile
-                float tmax = -INFINITY;
-#pragma unroll
-                for (int kb = 0; kb < NKB; ++kb)
-#pragma unroll
-                    for (int i = 0; i < 16; ++i) tmax = fmaxf(tmax, s[kb][i]);
-                tmax = lane_max_xor32(tmax); // relative to the present m_run; -inf for a row that sees nothing here
-                const float shift = t == 0 ? tmax : fmaxf(tmax, 0.f);
-                const float alpha = __builtin_amdgcn_exp2f(QSCALED ? -shift : -shift * a.sm_scale_log2);
-                m_run += shift;
-                if (t != 0) { // (nothing has been accumulated before the first tile)
-                    l_run *= alpha;
-#pragma unroll
-                    for (int db = 0; db < 4; ++db)
-#pragma unroll
-                        for (int i = 0; i < 16; ++i) acc[db][i] *= alpha;
-                }
-#pragma unroll
-                for (int i = 0; i < 16; ++i) cinit[i] = -m_run;
-                probabilities(shift);
-            }
-            psum = lane_sum_xor32(psum);
-            l_run += psum;
-            __builtin_amdgcn_sched_barrier(0);
-            // ---- O^T += V^T P^T: step i takes tokens 16*(i/4) .. +15 and d block i%4
-#pragma unroll
-            for (int i = 0; i < NS; ++i) {
-                acc[i & 3] = M::run(va[i % kDV], pa[i >> 2], acc[i & 3]);
-                if (SPLIT_P) acc[i & 3] = M::run(va[i % kDV], pb[i >> 2], acc[i & 3]);
-                if (i + kDV < NS) va[i % kDV] = v_read(i + kDV);
-                __builtin_amdgcn_sched_barrier(0);
-            }
-        }
-    };
-    auto tile = [&](int t, auto which) __attribute__((always_inline)) {
-        if (t >= n_w) return;
-        if (t == t_half) compute_tile(t, which, std::true_type{});
-        else compute_tile(t, which, std::false_type{});
-    };
-    for (int t = 0; t < n_tiles; t += 2) {
-        if (t + 1 < n_tiles) issue_tile(t + 1, 1); // buffer 1 was last read before the previous barrier
-        tile(t, std::integral_constant<int, 0>{});
-        publish();
-        if (t + 1 < n_tiles) {
-            if (t + 2 < n_tiles) issue_tile(t + 2, 0);
-            tile(t + 1, std::integral_constant<int, 1>{});
-            publish();
-        }
-    }
-
-    // ---- epilogue: normalise, transpose the wave's 32 x 128 block through LDS, store whole rows
-    const float inv_l = l_run > 0.f ? 1.0f / l_run : 0.f;
-    unsigned char* o_lds = smem + wave * (32 * kORow); // the tiles are free now (barrier above)
-#pragma unroll
-    for (int db = 0; db < 4; ++db)
-#pragma unroll
-        for (int b = 0; b < 4; ++b) {
-            const uint32_t w0 = M::pack2(acc[db][4 * b] * inv_l, acc[db][4 * b + 1] * inv_l);
-            const uint32_t w1 = M::pack2(acc[db][4 * b + 2] * inv_l, acc[db][4 * b + 3] * inv_l);
-            *reinterpret_cast<uint2*>(o_lds + qn * kORow + (32 * db + 8 * b + 4 * h) * 2) = make_uint2(w0, w1);
-        }
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-    __builtin_amdgcn_wave_barrier();
-    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-#pragma unroll
-    for (int ps = 0; ps < 8; ++ps) {
-        const int row = 4 * ps + (lane >> 4);
-        const int pos = wave_q_lo + row;
-        if (pos < L) {
-            const uint4 v = *reinterpret_cast<const uint4*>(o_lds + row * kORow + (lane & 15) * 16);
-            char* orow = (char*)a.out + (((size_t)it.tok0 + pos) * Hq + head) * 256;
-            *reinterpret_cast<uint4*>(orow + (lane & 15) * 16) = v;
-        }
-    }
-}
 
 // ---------------------------------------------------------------------------------------------------------
-// The software-pipelined kernel.  One workgroup of 4 waves takes 128 consecutive q rows of one (request,
-// q head) as prefill_kernel does, two workgroups per CU; what differs is the loop.  K/V tiles are 32 tokens
-// and a wave's instruction stream for tile j is one interleaved sequence
+// The attention kernel.  A wave's instruction stream for tile j is one interleaved, software-pipelined sequence
 //     8 x { matrix: S(j+1) += K(j+1) Q^T step i | LDS: next operand | vector: exp, pack, row sum of S(j) }
 //     8 x { matrix: O += V(j)^T P(j)^T step i   | LDS: next operand }
-// so that a wave always has matrix instructions in flight while it does its vector work (a wave issues about one
+// so that a wave always has matrix instructions in flight while it does its vector work: a wave issues about one
 // instruction per five cycles whatever its kind, a matrix instruction keeps the pipe busy for 32, and the matrix
-// and vector instructions of the two waves of a SIMD share one issue port: the vector work has to sit in
-// the shadow of the matrix instructions of the same wave to be free).  Operands come from LDS through two rings
-// of four registers each, read four matrix instructions ahead of their use.  Tiles are copied global -> LDS
-// kSNK (K) and kSNV (V) tiles deep, which is about three tiles (two microseconds) ahead of their first read;
-// there is one workgroup barrier per tile, at the top of the iteration, where the tile that arrives next is
-// published and the buffers of the tiles just finished are handed back to the copies.  The steady state
-// (`full`) has no conditions in it; everything ragged or masked goes through `generic`.
-#ifndef BZ_PF_ABL
-#define BZ_PF_ABL 0 // timing experiments (results wrong): 1 no softmax arithmetic, 2 no LDS operand reads, 4 no tile copies, 8 no barriers in the steady state, 16 no matrix instructions
-#endif
+// and vector instructions of the two waves of a SIMD (two workgroups per CU) share one issue port, so the vector
+// work has to sit in the shadow of the matrix instructions of the same wave to be free.  Operands come from LDS
+// through two rings of four registers each, read four matrix instructions ahead of their use.  Tiles are copied
+// global -> LDS with LDS-direct loads, kSNK (K) and kSNV (V) tiles deep, two to three tiles (about two
+// microseconds) ahead of their first read; there is one workgroup barrier per tile, at the top of the iteration,
+// where the tiles read next are published and the buffers of the tiles just finished are handed back to the
+// copies.  The steady state (`full`) has no conditions in it; everything ragged or masked goes through `generic`.
+//
+// Softmax without a maximum per tile: q rows that are rotated here carry sm_scale * log2(e) in the one rounding of
+// the rotated row (rows that arrive as they are keep their bits and the scale stays on the score), and the first
+// score instruction of a tile accumulates onto `cinit`, a block of registers that holds -m_run, so the scores leave
+// the matrix pipe as base-2 logits relative to the reference maximum m_run of their row and go into v_exp_f32 as
+// they are.  m_run is set from the first tile and moved only when it has to be: a tile's probabilities are computed
+// on the assumption that no score exceeds m_run by 15 or more (p < 2^15 fits the 16-bit operand of the second
+// contraction and fp32 sums); the row sums, which are needed anyway, tell whether it held, and a wave for which it
+// did not takes the tile's maximum, moves m_run, rescales its accumulators and computes the tile's probabilities
+// again (move_maximum: rare, wave-uniform).  m_run never exceeds the true running maximum, so the largest
+// probability of a row so far is always at least 1.
+//
+// LDS layout of a tile: 32 rows of 256 bytes, unpadded (an LDS-direct load writes 64 x 16 B to consecutive LDS);
+// what keeps the operand reads free of bank conflicts is an XOR on the 16-byte column chunk:
+//   K: chunk c of row r sits at position c ^ (r % 16)      (16 lanes read 16 rows, one chunk each)
+//   V: chunk c of row r sits at position c ^ g(r % 4), g = 0, 4, 10, 14 (BZ_VSWZ).  The transposing read
+//      ds_read_b64_tr_b16 takes 8 B per lane; a 16-lane group reads 4 rows x 32 B and two groups (4 rows x 64 B) go
+//      through the 64 banks together, so the 8 (row, group) pieces must land in 8 different 32-byte bank groups
+// and a lane of the copy simply fetches the chunk that belongs at its position.
 constexpr int kSN = 32;                      // kv tokens per tile
 constexpr int kSTile = kSN * 256;            // bytes of one K or V tile in LDS
 #ifndef BZ_PF_NK
@@ -502,6 +180,24 @@ __device__ __forceinline__ void lds_direct_load16x2(const char* uniform_base, ui
                  : "s"(lds_addr), "v"(o0), "v"(o1), "s"(uniform_base)
                  : "memory", "m0");
 }
+// Loads the compiler keeps no count of: the kernel waits for them itself (sp_wait_copies counts them like copies),
+// so that a wait for the q rows does not become a wait for every tile copy in flight.  The registers must not be
+// read before sp_loads_arrived() has been passed over them.
+__device__ __forceinline__ uint4 sp_load16(const void* p) {
+    typedef uint32_t __attribute__((ext_vector_type(4))) u32x4;
+    u32x4 r;
+    asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(r) : "v"(p) : "memory");
+    return make_uint4(r.x, r.y, r.z, r.w);
+}
+__device__ __forceinline__ float2 sp_load8(const void* p) {
+    typedef float __attribute__((ext_vector_type(2))) f32x2;
+    f32x2 r;
+    asm volatile("global_load_dwordx2 %0, %1, off" : "=v"(r) : "v"(p) : "memory");
+    return make_float2(r.x, r.y);
+}
+__device__ __forceinline__ void sp_loads_arrived(uint4& r) { asm volatile("" : "+v"(r.x), "+v"(r.y), "+v"(r.z), "+v"(r.w)); }
+__device__ __forceinline__ void sp_loads_arrived(float2& r) { asm volatile("" : "+v"(r.x), "+v"(r.y)); }
+
 // workgroup barrier that the compiler moves no memory access across (it waits for nothing by itself)
 __device__ __forceinline__ void sp_barrier() {
     __builtin_amdgcn_sched_barrier(0);
@@ -525,20 +221,25 @@ __device__ __forceinline__ void sp_wait_copies(int tiles) {
 }
 // Copies are issued in pairs (K(i + kSNK), V(i + kSNV - 1)) at the top of iteration i, the first kSNK pairs
 // (i = -kSNK .. -1, tiles below 0 left out) in the prologue.  The tiles first read in iteration j are K(j+2) and
-// V(j): this counts the copies that exist (tile < n) behind the later of the two, up to those of iteration j-1.
-__device__ __forceinline__ int sp_copies_behind(int j, int n) {
+// V(j); with V_NEXT also V(j+1), which is then converted in place during iteration j.  This counts the copies that
+// exist (tile < n) behind the last of them, up to those of iteration j-1.
+__device__ __forceinline__ int sp_copies_behind(int j, int n, bool v_next) {
     const int pk = 2 * (j + 2 - kSNK), pv = 2 * (j + 1 - kSNV) + 1; // positions of K(j+2), V(j) in the issue order
+    int p = max(pk, pv);
+    if (v_next && j + 1 < n) p = max(p, pv + 2);
     int c = 0;
-    for (int pos = max(pk, pv) + 1; pos <= 2 * j - 1; ++pos) {
+    for (int pos = p + 1; pos <= 2 * j - 1; ++pos) {
         const int i = pos >> 1; // (arithmetic shift: positions may be negative in the first iterations)
         const int tile = (pos & 1) ? i + kSNV - 1 : i + kSNK;
         c += (tile >= 0 && tile < n) ? 1 : 0;
     }
     return c;
 }
-constexpr int sp_copies_behind_steady() { // the same when every tile exists
+constexpr int sp_copies_behind_steady(bool v_next) { // the same when every tile exists
     const int pk = 2 * (2 - kSNK), pv = 2 * (1 - kSNV) + 1;
-    return -1 - (pk > pv ? pk : pv);
+    int p = pk > pv ? pk : pv;
+    if (v_next && pv + 2 > p) p = pv + 2;
+    return -1 - p;
 }
 __device__ __forceinline__ int sp_wrap(int x, int m) { return x >= m ? x - m : x; } // x < 2 m
 
@@ -552,11 +253,19 @@ __device__ unsigned long long bz_pf_wg[kPftMaxWg * 8];
 #define BZ_PF_WG(k) do { } while (0)
 #endif
 
+// bf16 has two ways through the second contraction (the 8-bit significand of a bf16 probability alone would eat
+// the error budget).  SPLIT_P: the probabilities enter it as head + tail of bf16, two matrix instructions per step.
+// Otherwise (V_F16): the V tiles are widened to f16 in LDS, in place, one tile ahead of their use (each wave its
+// quarter of the tile), the probabilities are packed as f16 and the second contraction runs on the f16
+// instruction, one per step.  The widening is exact for |v| in f16's range (2^-24 .. 65504; smaller values round
+// to f16 subnormals or zero, larger ones become infinite), which is why SPLIT_P stays selectable.
 template <bool BF16, bool SPLIT_P, bool ROPE_Q>
-__global__ __launch_bounds__(256, 2) void prefill_sp_kernel(PrefillArgs a, const char* __restrict__ q_ptr,
+__global__ __launch_bounds__(256, 2) void prefill_kernel(PrefillArgs a, const char* __restrict__ q_ptr,
                                                             const char* __restrict__ k_ptr,
                                                             const char* __restrict__ v_ptr) {
-    using M = PfMma<BF16>;
+    constexpr bool V_F16 = BF16 && !SPLIT_P;
+    using M = PfMma<BF16>;            // q, k, the first contraction and the output
+    using MP = PfMma<BF16 && !V_F16>; // the probabilities and the second contraction
     constexpr bool QSCALED = ROPE_Q; // q carries sm_scale * log2(e)
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
 #ifdef BZ_PF_TIMING
@@ -584,7 +293,7 @@ __global__ __launch_bounds__(256, 2) void prefill_sp_kernel(PrefillArgs a, const
     const int kv_max = a.causal ? min(q_pos, L - 1) : L - 1; // last token this row may see
 
     // ---- global -> LDS staging: wave wv moves rows 8wv .. 8wv+7 of a tile, two instructions of four 256-byte
-    // rows each for K and for V (chunk XOR patterns as in prefill_kernel)
+    // rows each for K and for V (chunk XOR patterns: see the kernel's header)
     const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) unsigned char*)smem;
     const int r4 = lane >> 4, p16 = lane & 15;
     const uint32_t row_stride = (uint32_t)Hkv * 256u;
@@ -604,11 +313,9 @@ __global__ __launch_bounds__(256, 2) void prefill_sp_kernel(PrefillArgs a, const
     const size_t tile_stride = (size_t)kSN * row_stride;
     // a whole tile inside the request: one wave-uniform base, lane constants for the rest
     auto issue_k_fast = [&](int t, int slot) __attribute__((always_inline)) {
-        if (BZ_PF_ABL & 4) return;
         lds_direct_load16x2(k_wave + (size_t)t * tile_stride, kfast[0], kfast[1], m0_wave + (uint32_t)(slot * kSTile));
     };
     auto issue_v_fast = [&](int t, int slot) __attribute__((always_inline)) {
-        if (BZ_PF_ABL & 4) return;
         lds_direct_load16x2(v_wave + (size_t)t * tile_stride, vfast[0], vfast[1], m0_wave + (uint32_t)((kSNK + slot) * kSTile));
     };
     auto issue_k = [&](int t, int slot) __attribute__((always_inline)) {
@@ -637,43 +344,54 @@ __global__ __launch_bounds__(256, 2) void prefill_sp_kernel(PrefillArgs a, const
             }
         }
     };
-    // the copies of the prologue go first: the q rows, the angles and the job itself travel in their shadow
-#pragma unroll
-    for (int i = -kSNK; i < 0; ++i) {
-        if (i + kSNK < n) issue_k(i + kSNK, i + kSNK);
-        if (i + kSNV - 1 >= 0 && i + kSNV - 1 < n) issue_v(i + kSNV - 1, i + kSNV - 1);
-    }
-
-    // ---- Q rows as B operands: lane (q, h) holds q[q][16*ks + 8*h .. +7], ks = 0..7 (as in prefill_kernel)
+    // ---- Q rows as B operands: lane (q, h) holds q[q][16*ks + 8*h .. +7], ks = 0..7.  The
+    // loads of the q rows and of the angles go first, the tile copies of the prologue behind them; the rotation
+    // is done while the copies travel.
     uint4 qreg[8];
+    float2 cs[ROPE_Q ? 32 : 1];
     {
         const size_t qtok = (size_t)it.tok0 + (size_t)min(q_pos, L - 1);
         const char* qrow = q_ptr + (qtok * Hq + head) * 256;
 #pragma unroll
-        for (int ks = 0; ks < 8; ++ks) qreg[ks] = *reinterpret_cast<const uint4*>(qrow + ks * 32 + h * 16);
+        for (int ks = 0; ks < 8; ++ks) qreg[ks] = sp_load16(qrow + ks * 32 + h * 16);
         if constexpr (ROPE_Q) {
+            // d = 16 ks + 8 h + e (ks < 4) pairs with d + 64, which this lane holds at step ks + 4.  The table is
+            // laid out pair by pair, so the 32 rows of a half-wave read 256 consecutive bytes per pair.
             const float2* tab = a.rope_table + min(q_pos, L - 1);
-            float2 cs[32];
 #pragma unroll
-            for (int e = 0; e < 32; ++e) cs[e] = tab[(size_t)(16 * (e >> 3) + 8 * h + (e & 7)) * a.rope_pitch];
-#pragma unroll
-            for (int ks = 0; ks < 4; ++ks)
-#pragma unroll
-                for (int w = 0; w < 4; ++w) {
-                    const float2 c0 = cs[8 * ks + 2 * w], c1 = cs[8 * ks + 2 * w + 1];
-                    const uint32_t xw = pf_u4(qreg[ks], w), yw = pf_u4(qreg[ks + 4], w);
-                    float x0, y0, x1, y1;
-                    rope_pair(M::lo(xw), M::lo(yw), c0.x, c0.y, x0, y0);
-                    rope_pair(M::hi(xw), M::hi(yw), c1.x, c1.y, x1, y1);
-                    pf_u4(qreg[ks], w) = M::pack2(x0 * a.sm_scale_log2, x1 * a.sm_scale_log2);
-                    pf_u4(qreg[ks + 4], w) = M::pack2(y0 * a.sm_scale_log2, y1 * a.sm_scale_log2);
-                }
+            for (int e = 0; e < 32; ++e) cs[e] = sp_load8(tab + (size_t)(16 * (e >> 3) + 8 * h + (e & 7)) * a.rope_pitch);
         }
+    }
+    int copies = 0; // tile copies issued so far
+#pragma unroll
+    for (int i = -kSNK; i < 0; ++i) {
+        if (i + kSNK < n) { issue_k(i + kSNK, i + kSNK); ++copies; }
+        if (i + kSNV - 1 >= 0 && i + kSNV - 1 < n) { issue_v(i + kSNV - 1, i + kSNV - 1); ++copies; }
+    }
+    sp_wait_copies(copies); // the q rows (and the angles) are here
+#pragma unroll
+    for (int ks = 0; ks < 8; ++ks) sp_loads_arrived(qreg[ks]);
+    if constexpr (ROPE_Q) {
+#pragma unroll
+        for (int e = 0; e < 32; ++e) sp_loads_arrived(cs[e]);
+#pragma unroll
+        for (int ks = 0; ks < 4; ++ks)
+#pragma unroll
+            for (int w = 0; w < 4; ++w) {
+                const float2 c0 = cs[8 * ks + 2 * w], c1 = cs[8 * ks + 2 * w + 1]; // pairs i = 16 ks + 8 h + 2 w, i + 1
+                const uint32_t xw = pf_u4(qreg[ks], w), yw = pf_u4(qreg[ks + 4], w);
+                float x0, y0, x1, y1;
+                rope_pair(M::lo(xw), M::lo(yw), c0.x, c0.y, x0, y0);
+                rope_pair(M::hi(xw), M::hi(yw), c1.x, c1.y, x1, y1);
+                // (the softmax scale rides on the one rounding of the rotated row, see the kernel's header)
+                pf_u4(qreg[ks], w) = M::pack2(x0 * a.sm_scale_log2, x1 * a.sm_scale_log2);
+                pf_u4(qreg[ks + 4], w) = M::pack2(y0 * a.sm_scale_log2, y1 * a.sm_scale_log2);
+            }
     }
 
     // Operand reads.  K: lane (row qn, half h) needs chunk 2 ks + h of its row for step ks, which sits at position
     // (2 ks + h) ^ (qn % 16); V, through the transposing read: chunk 4 db + zl' of its row for d block db (see
-    // prefill_kernel).  One address register per step / d block (complete LDS addresses inside slot 0); the slot and
+    // the kernel's header).  One address register per step / d block (complete LDS addresses inside slot 0); the slot and
     // the token offsets of the V operands go into the instruction's offset field where they are compile-time constants.
     uint32_t koff[8], voff[4];
     {
@@ -692,19 +410,15 @@ __global__ __launch_bounds__(256, 2) void prefill_sp_kernel(PrefillArgs a, const
         }
     }
     uint4 kring[4], vring[4]; // operands of the matrix instructions, read four instructions ahead of their use
-    if (BZ_PF_ABL & 2)
-        for (int i = 0; i < 4; ++i) kring[i] = vring[i] = make_uint4(lane, 2 * lane, 3, 4);
     typedef uint32_t __attribute__((ext_vector_type(4))) pf_u32x4;
     // (these issue the reads; the first use of a register waits for it.  `soff`: byte offset of the tile's slot)
     auto read_k = [&](uint4& dst, uint32_t soff, int ks) __attribute__((always_inline)) {
-        if (BZ_PF_ABL & 2) { asm volatile("" : "+v"(dst.x)); return; }
         const pf_u32x4 r = *reinterpret_cast<const pf_u32x4 __attribute__((address_space(3)))*>(
             (const unsigned char __attribute__((address_space(3)))*)(uintptr_t)(koff[ks]) + soff);
         dst = make_uint4(r.x, r.y, r.z, r.w);
     };
     // operand i = 4 st + db of the second contraction (tokens 16 st .., d block db): two reads, rows +0 and +8
     auto read_v = [&](uint4& dst, uint32_t soff, int i) __attribute__((always_inline)) {
-        if (BZ_PF_ABL & 2) { asm volatile("" : "+v"(dst.x)); return; }
         typedef pf_s16x4 __attribute__((address_space(3)))* lds_s16x4_ptr;
         const unsigned char __attribute__((address_space(3)))* vb =
             (const unsigned char __attribute__((address_space(3)))*)(uintptr_t)(voff[i & 3]) + soff + (i >> 2) * 16 * 256;
@@ -713,10 +427,24 @@ __global__ __launch_bounds__(256, 2) void prefill_sp_kernel(PrefillArgs a, const
         const uint2 w0 = __builtin_bit_cast(uint2, t0), w1 = __builtin_bit_cast(uint2, t1);
         dst = make_uint4(w0.x, w0.y, w1.x, w1.y);
     };
+    // V_F16: this wave's quarter of the V tile in `slot` (the rows it copied), bf16 -> f16 in place
+    auto widen_v = [&](int slot) __attribute__((always_inline)) {
+        typedef pf_u32x4 __attribute__((address_space(3)))* lds_u32x4_ptr;
+        unsigned char __attribute__((address_space(3)))* base =
+            (unsigned char __attribute__((address_space(3)))*)(uintptr_t)(m0_wave + (uint32_t)((kSNK + slot) * kSTile)) + lane * 16;
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+            pf_u32x4 r = *(lds_u32x4_ptr)(base + i * 1024);
+#pragma unroll
+            for (int w = 0; w < 4; ++w)
+                r[w] = PfMma<false>::pack2(__uint_as_float(r[w] << 16), __uint_as_float(r[w] & 0xffff0000u));
+            *(lds_u32x4_ptr)(base + i * 1024) = r;
+        }
+    };
     auto k_at = [&](int slot) __attribute__((always_inline)) { return (uint32_t)(slot * kSTile); };
     auto v_at = [&](int slot) __attribute__((always_inline)) { return (uint32_t)(slot * kSTile); };
 
-    // ---- softmax state (see prefill_kernel: one reference maximum per row, moved only when it has to be)
+    // ---- softmax state (one reference maximum per row, moved only when it has to be: see the kernel's header)
     float m_run = 0.f, l_run = 0.f; // l_run: this lane's half of the row sum
     pf_f32x16 cinit;
 #pragma unroll
@@ -746,13 +474,13 @@ __global__ __launch_bounds__(256, 2) void prefill_sp_kernel(PrefillArgs a, const
     // elements 2i, 2i+1 -> word i%4 of operand i/4.  The row sum takes the probabilities as they enter the second
     // contraction (rounded to the storage type; head + tail when SPLIT_P), one instruction per packed word.
     auto take_pair = [&](float p0, float p1, int i) __attribute__((always_inline)) {
-        const uint32_t hw = M::pack2_here(p0, p1);
+        const uint32_t hw = MP::pack2_here(p0, p1);
         pf_u4(pa[i >> 2], i & 3) = hw;
-        psum = M::add_pair(hw, psum);
+        psum = MP::add_pair(hw, psum);
         if (SPLIT_P) {
-            const uint32_t tw = M::pack2_here(p0 - M::lo(hw), p1 - M::hi(hw));
+            const uint32_t tw = MP::pack2_here(p0 - MP::lo(hw), p1 - MP::hi(hw));
             pf_u4(pb[i >> 2], i & 3) = tw;
-            psum = M::add_pair(tw, psum);
+            psum = MP::add_pair(tw, psum);
         }
     };
     // The first half of an iteration: scores of the next tile into s[PAR ^ 1] (QK) from K at k1 (steps 0..3 are in
@@ -766,10 +494,10 @@ __global__ __launch_bounds__(256, 2) void prefill_sp_kernel(PrefillArgs a, const
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
-            if (QK && !(BZ_PF_ABL & 16)) s[PAR ^ 1] = M::run(kring[i & 3], qreg[i], i == 0 ? cinit : s[PAR ^ 1]);
+            if (QK) s[PAR ^ 1] = M::run(kring[i & 3], qreg[i], i == 0 ? cinit : s[PAR ^ 1]);
             if (i < 4) read_k(kring[i], k1, i + 4);
             else read_v(vring[i - 4], vj, i - 4);
-            if (EX && !(BZ_PF_ABL & 1)) {
+            if (EX) {
                 const float n0 = exp_of(s[PAR][2 * i], 0.f), n1 = exp_of(s[PAR][2 * i + 1], 0.f);
                 if (i > 0) take_pair(e0, e1, i - 1);
                 e0 = n0;
@@ -777,7 +505,7 @@ __global__ __launch_bounds__(256, 2) void prefill_sp_kernel(PrefillArgs a, const
             }
             __builtin_amdgcn_sched_barrier(0);
         }
-        if (EX && !(BZ_PF_ABL & 1)) take_pair(e0, e1, 7);
+        if (EX) take_pair(e0, e1, 7);
         __builtin_amdgcn_sched_barrier(0);
     };
     // The second half: O += V^T P^T (PV), the rest of V (at vj) and the first K operands of the tile after the next
@@ -787,9 +515,9 @@ __global__ __launch_bounds__(256, 2) void prefill_sp_kernel(PrefillArgs a, const
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
-            if (PV && !(BZ_PF_ABL & 16)) {
-                acc[i & 3] = M::run(vring[i & 3], pa[i >> 2], acc[i & 3]);
-                if (SPLIT_P) acc[i & 3] = M::run(vring[i & 3], pb[i >> 2], acc[i & 3]);
+            if (PV) {
+                acc[i & 3] = MP::run(vring[i & 3], pa[i >> 2], acc[i & 3]);
+                if (SPLIT_P) acc[i & 3] = MP::run(vring[i & 3], pb[i >> 2], acc[i & 3]);
             }
             if (i < 4) read_v(vring[i], vj, i + 4);
             else read_k(kring[i - 4], k2, i - 4);
@@ -821,11 +549,9 @@ __global__ __launch_bounds__(256, 2) void prefill_sp_kernel(PrefillArgs a, const
     };
 
     // ---- prologue: scores of tile 0 set the reference maximum, the ring takes the first K operands of tile 1.
-    // The wait is for everything in flight (the copies were issued together, so they arrive together), which
-    // also tells the compiler, who counts only the loads it knows of, that the q registers are complete: it would
-    // otherwise wait for "its" loads, and with them for every copy in flight, inside the loop.
+    // The copies were issued in the order K0 | K1 V0 | K2 V1 | K3 V2 (those that exist).
     BZ_PF_WG(1);
-    sp_wait_copies(0);
+    sp_wait_copies(copies - 1); // K0 has landed
     sp_barrier();
     BZ_PF_WG(2);
     {
@@ -847,8 +573,11 @@ __global__ __launch_bounds__(256, 2) void prefill_sp_kernel(PrefillArgs a, const
                 cinit[i] = -tmax;
             }
         }
+        sp_wait_copies(max(copies - (V_F16 ? 3 : 2), 0)); // K1 has landed (if there is one); V_F16: V0 as well
+        sp_barrier();
 #pragma unroll
         for (int i = 0; i < 4; ++i) read_k(kring[i], k_at(1 % kSNK), i);
+        if (V_F16) widen_v(0);
     }
     BZ_PF_WG(3);
 
@@ -864,21 +593,20 @@ __global__ __launch_bounds__(256, 2) void prefill_sp_kernel(PrefillArgs a, const
         constexpr int PAR = decltype(par_c)::value, SL = decltype(sl_c)::value;
         constexpr bool COND = decltype(cond_c)::value;
         if (!COND) {
-            sp_wait_copies(sp_copies_behind_steady()); // K(j+2) and V(j) have landed
-            if (!(BZ_PF_ABL & 8)) sp_barrier();
-            if (!(BZ_PF_ABL & 4)) {
-                lds_direct_load16x2(k_next, kfast[0], kfast[1], m0_wave + (uint32_t)(SL * kSTile));
-                lds_direct_load16x2(v_next, vfast[0], vfast[1], m0_wave + (uint32_t)((kSNK + (SL + kSNV - 1) % kSNV) * kSTile));
-            }
+            sp_wait_copies(sp_copies_behind_steady(V_F16)); // K(j+2) and V(j) have landed (V_F16: V(j+1) too)
+            sp_barrier();
+            lds_direct_load16x2(k_next, kfast[0], kfast[1], m0_wave + (uint32_t)(SL * kSTile));
+            lds_direct_load16x2(v_next, vfast[0], vfast[1], m0_wave + (uint32_t)((kSNK + (SL + kSNV - 1) % kSNV) * kSTile));
             k_next += tile_stride;
             v_next += tile_stride;
         } else {
             // behind K(j+2): V(j+1), K(j+3), V(j+2), of which only K(j+3) may be missing here
-            sp_wait_copies(2 + (j + 3 < n ? 1 : 0));
+            sp_wait_copies((V_F16 ? 1 : 2) + (j + 3 < n ? 1 : 0));
             sp_barrier();
             if (j + kSNK < n) issue_k(j + kSNK, SL);
             if (j + kSNV - 1 < n) issue_v(j + kSNV - 1, (SL + kSNV - 1) % kSNV);
         }
+        if (V_F16) widen_v((SL + 1) % kSNV); // V(j+1), first read after the next barrier
         first_half(par_c, std::true_type{}, std::true_type{}, k_at((SL + 1) % kSNK), v_at(SL));
         if (__any(!(psum < 32768.0f))) move_maximum(s[PAR], s[PAR ^ 1]);
         l_run += psum;
@@ -889,10 +617,11 @@ __global__ __launch_bounds__(256, 2) void prefill_sp_kernel(PrefillArgs a, const
     auto generic = [&](int j, auto par_c) __attribute__((always_inline)) {
         constexpr int PAR = decltype(par_c)::value;
         const bool has_cur = j < n_w, has_next = j + 1 < n_w;
-        sp_wait_copies(sp_copies_behind(j, n));
+        sp_wait_copies(sp_copies_behind(j, n, V_F16));
         sp_barrier();
         if (j + kSNK < n) issue_k(j + kSNK, kj);
         if (j + kSNV - 1 < n) issue_v(j + kSNV - 1, sp_wrap(vj + kSNV - 1, kSNV));
+        if (V_F16 && j + 1 < n) widen_v(sp_wrap(vj + 1, kSNV));
         const uint32_t k1 = k_at(sp_wrap(kj + 1, kSNK)), k2 = k_at(sp_wrap(kj + 2, kSNK));
         if (has_next) first_half(par_c, std::true_type{}, std::true_type{}, k1, v_at(vj));
         else first_half(par_c, std::false_type{}, std::true_type{}, k1, v_at(vj)); // (harmless without a tile: p of stale scores, never used)
@@ -1072,6 +801,13 @@ extern "C" bz_prefill_plan_t* bz_prefill_plan_create(void) {
     return reinterpret_cast<bz_prefill_plan_t*>(new (std::nothrow) PrefillPlan());
 }
 
+extern "C" int bz_prefill_plan_set_bf16_mode(bz_prefill_plan_t* plan_, int mode) {
+    PrefillPlan* p = reinterpret_cast<PrefillPlan*>(plan_);
+    if (!p || (mode != BZ_PREFILL_BF16_WIDEN_V && mode != BZ_PREFILL_BF16_HEAD_TAIL)) return BZ_ERR_BAD_ARG;
+    p->bf16_head_tail = mode == BZ_PREFILL_BF16_HEAD_TAIL;
+    return 0;
+}
+
 extern "C" void bz_prefill_plan_destroy(bz_prefill_plan_t* plan_) {
     PrefillPlan* p = reinterpret_cast<PrefillPlan*>(plan_);
     if (!p) return;
@@ -1208,34 +944,8 @@ extern "C" int bz_prefill_plan(bz_prefill_plan_t* plan_, void* float_buffer, siz
 
 template <bool BF16, bool SPLIT_P, bool ROPE_Q>
 static int launch_prefill(const PrefillPlan* p, const PrefillArgs& a, const void* q, const void* k, const void* v,
-                          hipStream_t s) {
-    const size_t smem = 4 * (size_t)kTile;
-    auto kern = prefill_kernel<BF16, SPLIT_P, ROPE_Q>;
-    // raising the dynamic LDS limit: once per device (idempotent, so a race between two host threads is harmless)
-    static std::atomic<uint64_t> attr_done{0};
-    int dev = 0;
-    BZ_CHECK_HIP(hipGetDevice(&dev));
-    const uint64_t bit = 1ull << (dev & 63);
-    if (!(attr_done.load(std::memory_order_relaxed) & bit)) {
-        BZ_CHECK_HIP(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
-        attr_done.fetch_or(bit, std::memory_order_relaxed);
-    }
-    hipLaunchKernelGGL(kern, dim3(p->num_items), dim3(256), smem, s, a, (const char*)q, (const char*)k,
-                       (const char*)v);
-    BZ_LAUNCH_CHECK();
-    return 0;
-}
-
-// Which attention kernel runs: the software-pipelined one unless BZ_PREFILL_KERNEL=single asks for prefill_kernel
-static bool prefill_use_sp() {
-    const char* e = getenv("BZ_PREFILL_KERNEL");
-    return !(e && strcmp(e, "single") == 0);
-}
-
-template <bool BF16, bool SPLIT_P, bool ROPE_Q>
-static int launch_prefill_sp(const PrefillPlan* p, const PrefillArgs& a, const void* q, const void* k, const void* v,
                              hipStream_t s) {
-    auto kern = prefill_sp_kernel<BF16, SPLIT_P, ROPE_Q>;
+    auto kern = prefill_kernel<BF16, SPLIT_P, ROPE_Q>;
     static std::atomic<uint64_t> attr_done{0};
     int dev = 0;
     BZ_CHECK_HIP(hipGetDevice(&dev));
@@ -1250,7 +960,7 @@ static int launch_prefill_sp(const PrefillPlan* p, const PrefillArgs& a, const v
 }
 
 #ifdef BZ_PF_TIMING
-// copies the table of the diagnostic build to the host: per workgroup 8 values (see prefill_sp_kernel)
+// copies the table of the diagnostic build to the host: per workgroup 8 values (see prefill_kernel)
 extern "C" int bz_pf_wg_table(unsigned long long* host, size_t count) {
     if (count > sizeof(bz_pf_wg) / 8) count = sizeof(bz_pf_wg) / 8;
     BZ_CHECK_HIP(hipMemcpyFromSymbol(host, HIP_SYMBOL(bz_pf_wg), count * 8, 0, hipMemcpyDeviceToHost));
@@ -1308,18 +1018,12 @@ extern "C" int bz_batch_prefill_ragged(bz_prefill_plan_t* plan_, void* q, const 
     a.causal = causal ? 1 : 0;
     if (!(sm_scale > 0.f)) sm_scale = 1.0f / sqrtf((float)head_dim);
     a.sm_scale_log2 = sm_scale * 1.4426950408889634f;
-    if (prefill_use_sp()) {
-        if (rope_q) {
-            if (dtype == BZ_F16) return launch_prefill_sp<false, false, true>(p, a, q, k, v, s);
-            return launch_prefill_sp<true, true, true>(p, a, q, k, v, s);
-        }
-        if (dtype == BZ_F16) return launch_prefill_sp<false, false, false>(p, a, q, k, v, s);
-        return launch_prefill_sp<true, true, false>(p, a, q, k, v, s);
-    }
     if (rope_q) {
         if (dtype == BZ_F16) return launch_prefill<false, false, true>(p, a, q, k, v, s);
-        return launch_prefill<true, true, true>(p, a, q, k, v, s);
+        if (p->bf16_head_tail) return launch_prefill<true, true, true>(p, a, q, k, v, s);
+        return launch_prefill<true, false, true>(p, a, q, k, v, s);
     }
     if (dtype == BZ_F16) return launch_prefill<false, false, false>(p, a, q, k, v, s);
-    return launch_prefill<true, true, false>(p, a, q, k, v, s);
+    if (p->bf16_head_tail) return launch_prefill<true, true, false>(p, a, q, k, v, s);
+    return launch_prefill<true, false, false>(p, a, q, k, v, s);
 }

@@ -208,6 +208,10 @@ class BatchPrefillRaggedHandler:
               "Handler workspace")
         return fb.value, ib.value
 
+    def set_bf16_mode(self, mode):
+        """BZ_PREFILL_BF16_WIDEN_V (default) or BZ_PREFILL_BF16_HEAD_TAIL: see include/bz_hip.h."""
+        check(_lib.load().bz_prefill_plan_set_bf16_mode(self._h, mode), "Handler bf16 mode")
+
     def host_schedule(self):
         """numpy copy [workgroups, 4] of the last job list: tok0, len (0 = padding), q0, head."""
         data, n, k = C.c_void_p(), C.c_size_t(), C.c_uint32()

@@ -224,6 +224,16 @@ int bz_prefill_plan_workspace(bz_prefill_plan_t* plan, const int32_t* qo_indptr_
 int bz_prefill_plan_host_schedule(const bz_prefill_plan_t* plan, const int32_t** data, size_t* num_records,
                                   uint32_t* ints_per_record);
 
+/* How bz_batch_prefill_ragged takes bf16 through its second contraction (no counterpart in the reference, whose
+ * FlashInfer call rounds the probabilities to bf16's 8-bit significand; the stated tolerance does not allow that).
+ * BZ_PREFILL_BF16_WIDEN_V (default): V tiles are widened to f16 on chip and the probabilities are f16 -- exact for
+ * |v| in f16's range (2^-24 .. 65504; smaller values round to f16 subnormals or zero, larger ones become infinite).
+ * BZ_PREFILL_BF16_HEAD_TAIL: V stays bf16 and the probabilities enter as head + tail of bf16 -- any range, two
+ * matrix instructions per step.  A setting of the plan: it holds for every later call with it. */
+#define BZ_PREFILL_BF16_WIDEN_V 0
+#define BZ_PREFILL_BF16_HEAD_TAIL 1
+int bz_prefill_plan_set_bf16_mode(bz_prefill_plan_t* plan, int mode);
+
 /*
  * batch_prefill_attention (src/kernel/attention.h:9-22, attention_prefill.cu:11-46): ragged
  * self-attention, q [N,Hq,D], k,v [N,Hkv,D], out [N,Hq,D], qo_indptr == kv_indptr (the only

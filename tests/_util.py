@@ -82,10 +82,56 @@ def dense_attention_f64(q, K, V, scale):
     return out
 
 
-def ulp_tol(ref, dtype, base=2e-3):
+def ulp_tol(ref, dtype, base=2e-3, before_rounding=0.0):
     """Per-element tolerance for a result stored in `dtype`: `base`, widened to just over half a
-    unit in the last place where the storage grid itself is coarser than that."""
+    unit in the last place where the storage grid itself is coarser than that.  `before_rounding`: the error
+    allowed for the value before it is rounded to the storage grid (a value that close to the middle between two
+    grid points may round either way, which puts the stored result half a unit plus that much from the reference)."""
     mant = 10 if dtype == BZ_F16 else 7
     a = np.maximum(np.abs(ref), 1e-30)
     half_ulp = 2.0 ** (np.floor(np.log2(a)) - mant - 1)
-    return np.maximum(base, 1.02 * half_ulp + 1e-6)
+    return np.maximum(base, 1.02 * half_ulp + 1e-6 + before_rounding)
+
+
+# bf16 prefill with V widened to f16 on chip (the default, BZ_PREFILL_BF16_WIDEN_V): the probabilities enter the
+# second contraction as f16 (relative 2^-12), which leaves the result within this of the reference before it is
+# rounded to bf16 (measured 1.5e-4 .. 3e-4); the head + tail mode keeps ~1e-6 and is held to the plain bar
+PREFILL_BF16_WIDEN_V_ERR = 5e-4
+
+
+def prefill_angle_table(float_ws, max_len, D=128):
+    """The (cos, sin) table the prefill call keeps in its float workspace for the q rotation: fp32 [D/2 pairs][max_len
+    positions][2], as the device computed it (sincosf(pos * f_i)); max_len is the longest request of the plan."""
+    raw = float_ws[: (D // 2) * max_len * 8].cpu().numpy().view(np.float32)
+    return raw.reshape(D // 2, max_len, 2)
+
+
+def prefill_q_as_fed(q_bits, dtype, indptr, Hq, D, theta, table, sm_scale=None):
+    """The q rows as the prefill kernel feeds them to the matrix cores when it rotates them itself
+    (BZ_ROPE_Q_ONLY / BZ_ROPE_FULL): rotated at their offset inside the request with the angles of the device's own
+    table (`table`, from prefill_angle_table: the device's sincosf may differ from the host's in the last place, and
+    one such difference, rounded the other way and multiplied by logits of +-40, is visible in the output),
+    multiplied by sm_scale * log2(e) and rounded ONCE to the storage type -- every step an IEEE fp32 operation in
+    the kernel's order, so the bits are the kernel's.  Attention over these rows with sm_scale = ln 2
+    (exp(s ln 2) = 2^s) and no further rotation of q is what the kernel computes, so the comparison needs no
+    allowance for that rounding.  The table itself is held against the host's sincos (two units in the last place)."""
+    q = wl.to_f32(q_bits, dtype)
+    N = q.shape[0]
+    indptr = np.asarray(indptr)
+    pos = np.arange(N) - np.repeat(indptr[:-1], np.diff(indptr))
+    f = oracle.rope_freqs(D, theta)
+    ang = pos[None, :].astype(np.float32) * f[:, None]  # [pairs][tokens], one fp32 multiply as on the device
+    c, s_ = table[:, pos, 0], table[:, pos, 1]
+    assert np.abs(c - np.cos(ang.astype(np.float64))).max() <= 2.0 ** -22 and np.abs(s_ - np.sin(ang.astype(np.float64))).max() <= 2.0 ** -22
+    c, s_ = c.T[:, None, :], s_.T[:, None, :]            # [tokens][1][pairs]
+    x, y = q[:, :, : D // 2], q[:, :, D // 2:]
+    xr = (x * c).astype(np.float32) - (y * s_).astype(np.float32)
+    yr = (y * c).astype(np.float32) + (x * s_).astype(np.float32)
+    if sm_scale is None:
+        sm_scale = np.float32(1.0) / np.sqrt(np.float32(D))
+    scale = np.float32(np.float32(sm_scale) * np.float32(1.4426950408889634))
+    out = np.concatenate([xr, yr], axis=2).astype(np.float32) * scale
+    return wl.to_bits(out.astype(np.float32), dtype)
+
+
+LN2 = float(np.float32(0.6931471805599453))
