@@ -51,6 +51,9 @@ def parse():
                     help="C4: where q is rotated. attention: in registers inside the attention kernel (q read once, "
                          "never written; the page store rotates k only); store: in place by the page-store kernel "
                          "(the attention kernel then takes q and k as they are)")
+    ap.add_argument("--prefill-dtype", default="f16", choices=["f16", "bf16", "bf16-head-tail"],
+                    help="C4: storage type of q, k, v and the output; bf16 runs the second product in f16 with V widened in "
+                         "LDS, bf16-head-tail with the probabilities as two bf16 operands (any range of V)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also launch a few plain device copies of 1 GiB (reference point for rocprofv3 --pmc byte counters)")
     args = ap.parse_args()
@@ -242,7 +245,7 @@ def bench_decode(args, name):
 
     # ---- the same steps as a layer loop would issue them in production: L consecutive layers' steps recorded
     # into one HIP graph and replayed (no host work between the launches); outputs compared with the eager step
-    ms_per_step, graph_note = eager_ms, "eager launches (no graph pass)"
+    ms_per_step, graph_note, region_us, device_us = eager_ms, "eager launches (no graph pass)", None, None
     if not args.no_graph:
         step(L - 1, None)
         torch.cuda.synchronize()
@@ -251,22 +254,64 @@ def bench_decode(args, name):
         with torch.cuda.stream(side):
             step(0, None, side.cuda_stream)  # warm-up on the capture stream, outside the capture
         torch.cuda.synchronize()
-        graph = torch.cuda.CUDAGraph()
-        with torch.cuda.graph(graph, stream=side):
-            for l in range(L):
-                step(l, None, torch.cuda.current_stream().cuda_stream)
-        torch.cuda.synchronize()
+        graphs = {}
+
+        def graph_of(n):
+            """n consecutive steps (layer planes 0 .. L-1, cyclically) as one HIP graph"""
+            if n not in graphs:
+                gr = torch.cuda.CUDAGraph()
+                with torch.cuda.graph(gr, stream=side):
+                    for l in range(n):
+                        step(l % L, None, torch.cuda.current_stream().cuda_stream)
+                torch.cuda.synchronize()
+                graphs[n] = gr
+            return graphs[n]
+
+        # A timed region of exactly `steps` steps: one graph of that many steps while that is a graph of modest
+        # size (every graph launch at the start of a region is host time inside the bracket), else whole replays
+        # of a 64-step graph and one shorter graph for the rest.
+        GN = 64
+
+        def run_steps(n):
+            for _ in range(n // GN):
+                graph_of(GN).replay()
+            if n % GN:
+                graph_of(n % GN).replay()
+
         out.zero_()
-        graph.replay()
+        graph_of(L).replay()
         torch.cuda.synchronize()
         same = bool(torch.equal(out.view(torch.int16), want.view(torch.int16)))
-        reps = max(1, steps // L)
-        wreps = max(1, warmup // L)
-        g_ms, _ = timed(lambda i, e: graph.replay(), reps, wreps, torch_events=False)
-        ms_per_step = g_ms / L
-        steps, warmup = reps * L, wreps * L
-        graph_note = (f"one HIP graph of {L} consecutive layers' steps, replayed {reps} times; last layer's output "
-                      f"bit-identical to the eager step: {same}")
+        for n in {GN if max(steps, warmup) >= GN else 0, steps % GN, warmup % GN} - {0}:
+            graph_of(n)
+        replays = steps // GN + (1 if steps % GN else 0)
+        regions = max(5, -(-25 // replays))  # >= 25 graph replays in all, >= 5 timed regions
+        done = torch.cuda.Event()
+        dev_ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(regions)]
+        run_steps(warmup)
+        torch.cuda.synchronize()
+        region_ms = []
+        for r in range(regions):
+            # one timed region: exactly `steps` steps between two device synchronisations.  The host polls an
+            # event for the end of the last step before it synchronises, so that the wake-up of a blocked
+            # host thread (tens of microseconds) is not counted into a region of a few milliseconds.
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            dev_ev[r][0].record()
+            run_steps(steps)
+            dev_ev[r][1].record()
+            done.record()
+            while not done.query():
+                pass
+            torch.cuda.synchronize()
+            region_ms.append((time.perf_counter() - t0) * 1e3)
+        region_us = np.array(region_ms) / steps  # ms per step of each region; pct() scales to us
+        device_us = np.array([a.elapsed_time(b) for a, b in dev_ev]) / steps
+        ms_per_step = float(region_us.mean())
+        graph_note = (f"HIP graphs of up to {GN} consecutive layers' steps (layer planes cycled); a timed region is exactly "
+                      f"{steps} steps ({replays} graph launches) between two device synchronisations by the host's "
+                      f"clock (graph launch latency included), value = mean of {regions} regions "
+                      f"after {warmup} warm-up steps; last layer's output bit-identical to the eager step: {same}")
     alg_bytes = wl.decode_algorithmic_bytes(ctx, Hq, Hkv, D, kv_bytes, 2, P)
     achieved = alg_bytes / (float(kern_ms.mean()) * 1e-3) / 1e9
     traffic = measured_traffic(name, args)
@@ -294,12 +339,18 @@ def bench_decode(args, name):
                       else "bz_decode_step (2 launches: decode kernel, then append + new-token term + split-K fold)"
                       if handler.step_form() == "one_call"
                       else "bz_decode_step (its choice for this plan: append, decode kernel, split-K combine)",
+        "value_method": "graph replay (a layer loop without host work between the launches); the same steps launched "
+                        "one by one from Python are eager_us_per_step" if not args.no_graph else "eager launches",
+        "step_us_per_region": pct(region_us) if region_us is not None else None,
+        "step_us_per_region_on_device": pct(device_us) if device_us is not None else None,
         "eager_us_per_step": round(eager_ms * 1e3, 3),
         "decode_call_us": pct(dec_ms),
         "decode_kernel_us": pct(kern_ms),
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBPS, 4),
                      "frac_call": round(frac_call, 4), "frac_step": round(frac_step, 4),
+                     "frac_step_device": round(alg_bytes / (float(device_us.mean()) * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4)
+                     if device_us is not None else None,
                      "traffic": traffic,
                      "traffic_source": "offline: rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this workload "
                                        "(profiles/), not measured in this run",
@@ -308,36 +359,51 @@ def bench_decode(args, name):
                                "of the step over that kernel's own duration (HIP events recorded by the library on the "
                                "launch stream right around its launch); frac_call is the same bytes over the whole "
                                "attention call(s) of the step (decode_call_us: every launch needed for the result), "
-                               "frac_step over ms_per_step"},
+                               "frac_step over ms_per_step (the host's clock around the timed regions), frac_step_device "
+                               "over the same regions between two events on the stream (first kernel's start to last "
+                               "kernel's end: without the host's launch latency at the head of a region)"},
     }
     if not args.no_cpu_baseline:
         import oracle  # the checker, used here only as the timed CPU baseline
         sb = B if name != "C5" else 16  # bounded sample: C5 in full would be minutes of CPU time
         odt = oracle.E4M3 if fp8 else (oracle.F16 if tdt == torch.float16 else oracle.BF16)
-        plane0 = pool[:plane]
-        plane0 = plane0.cpu().numpy() if fp8 else plane0.view(torch.int16).cpu().numpy().view(np.uint16)
         qh = q.view(torch.int16).cpu().numpy().view(np.uint16)
         sp, sn, sh = wl.strides(BZ_LAYOUT_HND, Hkv, P, D)
-        kv = oracle.PagedKV(plane0, plane0[sp // 2:], indices[:int(indptr[sb])], indptr[:sb + 1], lpl[:sb], P, Hkv, D, sp,
-                            sn, sh, odt)
         ks = k_scale.cpu().numpy() if fp8 else None
         vs = v_scale.cpu().numpy() if fp8 else None
         qdt = oracle.F16 if tdt == torch.float16 else oracle.BF16
+        # the timed call once more on layer plane 0, then the checker over the very bits the device cached
+        pt.set_layer(0, pool_pages)
+        attention()
+        out32 = torch.empty((B, Hq, D), dtype=torch.float32, device=dev)
+        if not args.two_call:
+            K.decode_step(handler, q, k_new, v_new, pt, out32, Hq, rope=rope, rope_theta=theta or 1e4, k_scale=k_scale,
+                          v_scale=v_scale)
+        else:
+            K.batch_decode_attention(handler, q, pt, out32, Hq, rope_mode=BZ_ROPE_Q_ONLY if rope else BZ_ROPE_NONE,
+                                     rope_theta=theta or 1e4, k_scale=k_scale, v_scale=v_scale)
+        torch.cuda.synchronize()
+        plane0 = pool[:plane]
+        plane0 = plane0.cpu().numpy() if fp8 else plane0.view(torch.int16).cpu().numpy().view(np.uint16)
+        kv = oracle.PagedKV(plane0, plane0[sp // 2:], indices[:int(indptr[sb])], indptr[:sb + 1], lpl[:sb], P, Hkv, D, sp,
+                            sn, sh, odt)
         reps, t0 = 0, time.perf_counter()
         while reps == 0 or (time.perf_counter() - t0 < 10.0 and reps < 200):  # about 10 s of CPU work
-            ref = oracle.batch_decode(qh[:sb], qdt, kv, Hq, k_scale=ks, v_scale=vs, parallel=True)
+            ref = oracle.batch_decode(qh[:sb], qdt, kv, Hq, rope_mode=oracle.ROPE_Q_ONLY if rope else oracle.ROPE_NONE,
+                                      rope_theta=theta or 1e4, k_scale=ks, v_scale=vs, parallel=True)
             reps += 1
         cpu_s = (time.perf_counter() - t0) / reps
-        pt.set_layer(0, pool_pages)
-        out32 = torch.empty((B, Hq, D), dtype=torch.float32, device=dev)
-        K.batch_decode_attention(handler, q, pt, out32, Hq, rope_mode=BZ_ROPE_NONE, k_scale=k_scale, v_scale=v_scale)
-        torch.cuda.synchronize()
-        res_json["max_abs_err_vs_cpu"] = float(np.abs(out32[:sb].cpu().numpy() - ref).max())
+        res_json["max_abs_err_vs_cpu"] = float(np.abs(out[:sb].float().cpu().numpy() - ref).max())
+        res_json["max_abs_err_vs_cpu_f32_out"] = float(np.abs(out32[:sb].cpu().numpy() - ref).max())
+        res_json["checked"] = ("the output of the timed call (append with RoPE, then attention with q rotated inside), "
+                               f"first {sb} sequences, against the CPU checker run on the pool as the call left it: "
+                               "max_abs_err_vs_cpu for the 16-bit output the timed steps write, ..._f32_out for the same "
+                               "call with an fp32 output")
         scale_up = float(ctx.sum()) / float(ctx[:sb].sum())
         res_json["cpu_baseline"] = {
             "value": round(cpu_s * scale_up * 1e6, 1), "unit": "us/step", "cores": oracle.num_threads(True),
             "kind": "port",
-            "sample": f"batch decode only (no append) of the first {sb} of {B} sequences, mean of {reps} repetitions "
+            "sample": f"batch decode (q rotated, no append) of the first {sb} of {B} sequences, mean of {reps} repetitions "
                       f"({cpu_s:.2f} s each), OpenMP over sequences, scaled by total/sample context tokens ({scale_up:.2f}x)",
             "host_cpus": os.cpu_count()}
     return res_json
@@ -348,9 +414,10 @@ def bench_prefill(args):
     import torch
 
     from blitz_scale_amd import kernel as K, workloads as wl
-    from blitz_scale_amd._lib import BZ_LAYOUT_HND, BZ_ROPE_NONE, BZ_ROPE_Q_ONLY
+    from blitz_scale_amd._lib import BZ_LAYOUT_HND, BZ_PREFILL_BF16_HEAD_TAIL, BZ_ROPE_NONE, BZ_ROPE_Q_ONLY
 
     dev = "cuda"
+    tdt = torch.float16 if args.prefill_dtype == "f16" else torch.bfloat16
     cfg = wl.CONFIGS["C4"]
     B, Hq, Hkv, D, P, theta = cfg["batch"], cfg["Hq"], cfg["Hkv"], cfg["D"], cfg["P"], cfg["rope_theta"]
     rng = np.random.default_rng(args.seed)
@@ -368,12 +435,11 @@ def bench_prefill(args):
     warmup = args.warmup if args.warmup is not None else 60
     g = torch.Generator(device=dev)
     g.manual_seed(args.seed)
-    q0 = torch.randn((N, Hq, D), dtype=torch.float16, device=dev, generator=g)
-    k0 = torch.randn((N, Hkv, D), dtype=torch.float16, device=dev, generator=g)
-    v = torch.randn((N, Hkv, D), dtype=torch.float16, device=dev, generator=g)
-    q, k = q0.clone(), k0.clone()
+    q = torch.randn((N, Hq, D), dtype=tdt, device=dev, generator=g)
+    k = torch.randn((N, Hkv, D), dtype=tdt, device=dev, generator=g)
+    v = torch.randn((N, Hkv, D), dtype=tdt, device=dev, generator=g)
     out = torch.empty_like(q)
-    pool = torch.zeros(pool_pages * stride_page, dtype=torch.float16, device=dev)
+    pool = torch.zeros(pool_pages * stride_page, dtype=tdt, device=dev)
     pt = K.PageTable(B, P, Hkv, D, pool, layout=BZ_LAYOUT_HND)
     pt.indices, pt.indptr, pt.last_page_len = indices, pindptr, lpl
     pt.upload()
@@ -381,6 +447,8 @@ def bench_prefill(args):
     float_ws = torch.empty(128 << 20, dtype=torch.uint8, device=dev)
     int_ws = torch.empty(8 << 20, dtype=torch.uint8, device=dev)
     handler = K.BatchPrefillRaggedHandler()
+    if args.prefill_dtype == "bf16-head-tail":
+        handler.set_bf16_mode(BZ_PREFILL_BF16_HEAD_TAIL)
     t0 = time.perf_counter()
     for _ in range(10):
         handler.plan(float_ws, float_ws.numel(), int_ws, int_ws.numel(), indptr, indptr, B, Hq, Hkv, D, P)
@@ -408,7 +476,7 @@ def bench_prefill(args):
     res_json = {
         "metric": "ragged_causal_prefill_ms_per_step", "value": round(ms_per_step, 4), "unit": "ms/step",
         "n_gpus": 1, "steps": steps, "warmup": warmup, "ms_per_step": round(ms_per_step, 6),
-        "higher_is_better": False, "scaling": "weak", "vs_baseline": None, "dtype": "f16", "data": "synthetic",
+        "higher_is_better": False, "scaling": "weak", "vs_baseline": None, "dtype": args.prefill_dtype, "data": "synthetic",
         "config": {"workload": "C4: Llama-2-13B-shaped ragged causal prefill with RoPE + KV page store, one layer per step",
                    "batch": B, "num_qo_heads": Hq, "num_kv_heads": Hkv, "head_dim": D, "page_size": P,
                    "lens": "uniform[128,4096]", "tokens": N, "pool_pages": pool_pages, "rope_theta": theta,
@@ -431,7 +499,8 @@ def bench_prefill(args):
         K.batch_prefill_attention(handler, q, ip, k, v, ip, out, B, Hq, Hkv, D, causal=True, rope_mode=BZ_ROPE_NONE)
         torch.cuda.synchronize()
         t0 = time.perf_counter()  # (checked without RoPE on either side: the same q and k bits, used as they are)
-        ref = oracle.batch_prefill_ragged(qh, kh, vh, oracle.F16, indptr, Hq, Hkv, D, causal=True, rows=rows, parallel=True)
+        ref = oracle.batch_prefill_ragged(qh, kh, vh, oracle.F16 if tdt == torch.float16 else oracle.BF16, indptr, Hq, Hkv, D,
+                                          causal=True, rows=rows, parallel=True)
         cpu_s = time.perf_counter() - t0
         res_json["max_abs_err_vs_cpu"] = float(np.abs(out[torch.from_numpy(rows.astype(np.int64)).to(dev)].float().cpu().numpy() - ref).max())
         seen = sum(int(r - indptr[np.searchsorted(indptr, r, side="right") - 1]) + 1 for r in rows)

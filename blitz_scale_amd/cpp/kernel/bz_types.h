@@ -48,11 +48,31 @@ struct AttentionOptions {
     bool append_rotates_k = true;           // append_decode_kv_cache rotates the new K row
     int decode_rope_mode = BZ_ROPE_Q_ONLY;  // batch_decode_attention: rotate q only, cached K is rotated
     uint32_t split_tokens = 0;              // 0: library default (2048)
+    int prefill_bf16_mode = BZ_PREFILL_BF16_WIDEN_V; // bf16 prefill: second product in f16 with V widened (exact for
+                                            // |v| in f16's range), or BZ_PREFILL_BF16_HEAD_TAIL for any range of V
     void* stream = nullptr;                 // hipStream_t; nullptr = the legacy default stream the reference uses
 };
 inline AttentionOptions& attention_options() {
     static AttentionOptions opts;
     return opts;
+}
+
+/// The options of the handler that planned last on this host thread (a copy, taken by plan()).  The page
+/// writes of the reference's calls take a PageTable and no handler; a table that points at no options of its own
+/// falls back to these, so that an engine which sets the RoPE base on its handlers only -- and builds a new
+/// PageTable per batch -- still gets the pages written with the base its attention calls use.  (Per thread: two
+/// models on two threads do not see each other; two models on one thread each plan before their layers run.)
+struct PlannedOptions {
+    AttentionOptions value;
+    bool valid = false;
+};
+inline PlannedOptions& planned_options() {
+    thread_local PlannedOptions p;
+    return p;
+}
+inline void note_planned_options(const AttentionOptions& o) {
+    planned_options().value = o;
+    planned_options().valid = true;
 }
 
 /// "no stream argument given": the element-wise wrappers then launch on attention_options().stream

@@ -21,6 +21,9 @@ class BatchPrefillRaggedHandler {
                                  reinterpret_cast<const int32_t*>(kv_indptr_h), batch_size, num_qo_heads, num_kv_heads,
                                  head_dim, page_size, options.stream),
                  "Handler plan:");
+        bz_throw(bz_prefill_plan_set_bf16_mode(static_cast<bz_prefill_plan_t*>(handler_), options.prefill_bf16_mode),
+                 "Handler plan:");
+        note_planned_options(options);
     }
     BatchPrefillRaggedHandler(void* handler_ptr = nullptr) : handler_(handler_ptr) {}
     void* get() noexcept { return handler_; }
@@ -47,6 +50,7 @@ class BlitzBatchDecodeHandler {
                                 reinterpret_cast<const int32_t*>(last_page_len_h), batch_size, num_qo_heads,
                                 num_kv_heads, head_dim, page_size, o.split_tokens, o.stream),
                  "Handler plan:");
+        note_planned_options(options);
     }
     BlitzBatchDecodeHandler(void* handler_ptr = nullptr) : handler_(handler_ptr) {}
     void* get() noexcept { return handler_; }

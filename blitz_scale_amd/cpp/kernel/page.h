@@ -46,9 +46,13 @@ struct PageTable {
     // (pages of the tokens to come already listed); nullptr = the table is the present
     IdType* steps_ahead_d = nullptr;
     // RoPE base / placement and stream of the page writes made through this table: the model's own
-    // (e.g. &decode_handler.options), or nullptr = the process-wide default
+    // (e.g. &decode_handler.options); nullptr = those of the handler that planned last on this thread, and
+    // the process-wide default before any plan
     const AttentionOptions* options = nullptr;
-    const AttentionOptions& opts() const { return options ? *options : attention_options(); }
+    const AttentionOptions& opts() const {
+        if (options) return *options;
+        return planned_options().valid ? planned_options().value : attention_options();
+    }
 
     PageTable(uint32_t batch_size_, uint32_t page_size_, uint32_t num_heads_, uint32_t head_size_, DType* base_ptr,
               int layout_ = BZ_LAYOUT_HND) :
@@ -84,14 +88,15 @@ struct PageTable {
 /// place by the same angles, so that batch_prefill_attention runs with BZ_ROPE_NONE afterwards.
 /// rotate: 1 / 0 force K rotation on / off, 2 = rotate K into the pages AND in place in the caller's rows
 /// (q is then left to batch_prefill_attention with BZ_ROPE_Q_ONLY), < 0 = on when q_inout is given, else
-/// opts().store_rotates_k.
+/// opts().store_rotates_k.  options: whose RoPE base and stream to use (a layer passes its handler's, so that
+/// the pages and the attention call cannot disagree); nullptr = page_table.opts().
 template<typename DType, typename IdType, typename SrcType = DType>
 void store_prefill_kv_cache(PageTable<DType, IdType>& page_table, SrcType* k_data, SrcType* v_data,
                             IdType* ragged_indptr, uint32_t num_tokens, SrcType* q_inout = nullptr,
                             uint32_t num_qo_heads = 0, const float* k_scale = nullptr,
-                            const float* v_scale = nullptr, int rotate = -1) {
+                            const float* v_scale = nullptr, int rotate = -1, const AttentionOptions* options = nullptr) {
     static_assert(sizeof(IdType) == 4, "page tables are int32");
-    const AttentionOptions& o = page_table.opts();
+    const AttentionOptions& o = options ? *options : page_table.opts();
     const bz_paged_kv_t kv = page_table.c_view();
     const int rot = rotate < 0 ? ((q_inout != nullptr || o.store_rotates_k) ? 1 : 0) : rotate;
     bz_throw(bz_store_prefill_kv(&kv, k_data, v_data, bz_dtype<SrcType>::value,
@@ -116,12 +121,13 @@ void store_prefill_kv_cache(PageTable<DType, IdType>& page_table, SrcType* k_dat
 /// q_inout (optional, [B, num_qo_heads, D]) is the fused form: q is rotated in place as well, and
 /// batch_decode_attention runs with BZ_ROPE_NONE afterwards.
 /// rotate: 1 / 0 force K rotation on / off, < 0 = on when q_inout is given, else opts().append_rotates_k.
+/// options: as for store_prefill_kv_cache.
 template<typename DType, typename IdType, typename SrcType = DType>
 void append_decode_kv_cache(PageTable<DType, IdType>& page_table, SrcType* k_data, SrcType* v_data,
                             SrcType* q_inout = nullptr, uint32_t num_qo_heads = 0, const float* k_scale = nullptr,
-                            const float* v_scale = nullptr, int rotate = -1) {
+                            const float* v_scale = nullptr, int rotate = -1, const AttentionOptions* options = nullptr) {
     static_assert(sizeof(IdType) == 4, "page tables are int32");
-    const AttentionOptions& o = page_table.opts();
+    const AttentionOptions& o = options ? *options : page_table.opts();
     const bz_paged_kv_t kv = page_table.c_view();
     const bool rot = rotate < 0 ? (q_inout != nullptr || o.append_rotates_k) : rotate != 0;
     bz_throw(bz_append_decode_kv(&kv, k_data, v_data, bz_dtype<SrcType>::value, q_inout, num_qo_heads, rot ? 1 : 0,

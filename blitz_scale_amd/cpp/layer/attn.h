@@ -59,8 +59,8 @@ class Attention {
         DType* attn_state = v + N * Hkv_ * D_;
         DType* o_proj = input;
 
-        // stream and RoPE base travel with the handlers (one set per model); the page writes take theirs
-        // from the table (page_table.options, which an engine points at the same handler's options)
+        // stream and RoPE base travel with the handlers (one set per model); the page writes are handed the same
+        // handler's options, whatever the table points at, so pages and attention cannot disagree
         void* stream = (qo_indptr_d ? prefill_->options : decode_->options).stream;
         kernel::rms_norm(residual, norm_w_, input, num_tokens, hidden_, 1e-5f, stream);
         // Three projections into three planes.  (The reference batches them into one or two row-major
@@ -74,7 +74,7 @@ class Attention {
             // K rotated once, into the pages and in place, while the pages are written; q is rotated in registers
             // inside the attention kernel (read once, never written)
             kernel::store_prefill_kv_cache(page_table, k, v, qo_indptr_d, num_tokens, static_cast<DType*>(nullptr), 0,
-                                           nullptr, nullptr, /*rotate=*/2);
+                                           nullptr, nullptr, /*rotate=*/2, &prefill_->options);
             kernel::batch_prefill_attention(*prefill_, q, qo_indptr_d, k, v, qo_indptr_d, attn_state,
                                             page_table.batch_size, Hq_, Hkv_, D_, BZ_ROPE_Q_ONLY);
         } else {

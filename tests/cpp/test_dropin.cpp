@@ -118,8 +118,10 @@ static double max_abs_diff(const uint16_t* a, const uint16_t* b, size_t n) {
 
 int main() {
     const uint32_t hidden = 256, Hq = 4, Hkv = 2, D = 128, inter = 512, P = 16, max_pages = 64, layers = 2;
-    const float theta = 1e4f;
-    blitz::kernel::attention_options().rope_theta = theta;
+    // The model's RoPE base is set on its two handlers and nowhere else: the process-wide default stays 1e4 and
+    // the page tables point at no options, so a page write that took its base from anywhere but the layer's
+    // handlers would fail the comparison below.
+    const float theta = 5e5f;
 
     // ---- weights: attention segment then GLU segment, as one device buffer walked by seg_iter
     const size_t attn_w = hidden + 2 * (size_t)Hq * D * hidden + 2 * (size_t)Hkv * D * hidden;
@@ -139,6 +141,7 @@ int main() {
     blitz::kernel::BatchPrefillRaggedHandler<half_t, int32_t> prefill_h(blitz::kernel::create_flashinfer_prefill_handler());
     blitz::kernel::BlitzBatchDecodeHandler<half_t, int32_t> decode_h(blitz::kernel::create_flashinfer_decode_handler());
     if (prefill_h.empty() || decode_h.empty()) return 3;
+    prefill_h.options.rope_theta = decode_h.options.rope_theta = theta;
     const uint32_t maxN = 64;
     const size_t ws_elems = maxN * (hidden + 3 * (size_t)std::max<uint32_t>(hidden, inter) + (size_t)(2 * Hq + 2 * Hkv) * D);
     half_t* ws_d;

@@ -87,7 +87,9 @@ struct Result {
 };
 
 // One model: its own handlers (and with them its own RoPE base and stream), pool and page table.
-static void run_model(float theta, uint64_t seed, Result* res) {
+// link_table: the page table points at the handler's options; without it the table has none of its own and the
+// page writes must find the base of the handler that planned last on this thread.
+static void run_model(float theta, uint64_t seed, bool link_table, Result* res) {
     const uint32_t num_qo_head = 8, num_kv_head = 2, head_size = 128, tp_size = 1, P = 16, max_pages = 96;
     Rng rng{seed};
     hipStream_t stream;
@@ -109,7 +111,7 @@ static void run_model(float theta, uint64_t seed, Result* res) {
     std::vector<int32_t> lens = {20, 37, 130};
     blitz::HostBatch<half_t, int32_t> batch(&cm, lens);
     auto& page_table = batch.page_table;
-    page_table.options = &decode_handle.options;
+    if (link_table) page_table.options = &decode_handle.options;
     cm.set_layer(page_table, 0);
     const uint32_t B = (uint32_t)lens.size(), N = (uint32_t)batch.ragged_indptr[B];
     int32_t* table_d;
@@ -219,14 +221,18 @@ int main() {
     HIP_OK(hipSetDevice(0));
     // the process-wide default stays what it is (theta 1e4, null stream): the two models below differ from it
     // and from each other only through their handlers
-    Result a, b;
-    std::thread ta([&] { HIP_OK(hipSetDevice(0)); run_model(1e4f, 0x5EED, &a); });
-    std::thread tb([&] { HIP_OK(hipSetDevice(0)); run_model(5e5f, 0xBEEF, &b); });
-    ta.join();
-    tb.join();
-    printf("%s%s", a.log.c_str(), b.log.c_str());
-    // a wrong base would not go unnoticed: the same inputs under the other model's base differ by far more than the bar
-    const bool ok = a.ok && b.ok;
+    bool ok = true;
+    for (int link = 1; link >= 0; --link) {
+        Result a, b;
+        std::thread ta([&] { HIP_OK(hipSetDevice(0)); run_model(1e4f, 0x5EED, link != 0, &a); });
+        std::thread tb([&] { HIP_OK(hipSetDevice(0)); run_model(5e5f, 0xBEEF, link != 0, &b); });
+        ta.join();
+        tb.join();
+        printf("%s:\n%s%s", link ? "table points at the handler's options" : "base set on the handlers only", a.log.c_str(),
+               b.log.c_str());
+        // a wrong base would not go unnoticed: the same inputs under the other model's base differ by far more than the bar
+        ok = ok && a.ok && b.ok;
+    }
     printf(ok ? "PASS\n" : "FAIL\n");
     return ok ? 0 : 1;
 }
