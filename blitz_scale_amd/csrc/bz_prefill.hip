@@ -59,7 +59,7 @@ struct PrefillPlan {
     const PrefillItem* items_d = nullptr;
     // cos / sin of position * frequency for every position a request of this batch has (float workspace),
     // filled by the first attention call that rotates q after a plan(), for the RoPE base of that call
-    float* rope_table = nullptr; // [max_len][64] pairs (cos, sin); nullptr: the float workspace has no room
+    float* rope_table = nullptr; // [32 couples of pairs][max_len] x (cos, sin, cos, sin); nullptr: the float workspace has no room
     float rope_table_theta = 0.f;
     bool rope_table_valid = false;
     std::vector<PrefillItem> h_items; // host copy of the last job list (kept between calls)
@@ -71,7 +71,7 @@ struct PrefillPlan {
 struct PrefillArgs {
     void* out;
     const PrefillItem* items;
-    const float2* rope_table; // ROPE_Q: [64 pairs][rope_pitch positions] x (cos, sin)
+    const float4* rope_table; // ROPE_Q: [32 couples of pairs][rope_pitch positions] x (cos i, sin i, cos i+1, sin i+1), i even
     uint32_t rope_pitch;
     uint32_t num_qo_heads, num_kv_heads;
     int causal;
@@ -348,7 +348,7 @@ __global__ __launch_bounds__(256, 2) void prefill_kernel(PrefillArgs a, const ch
     // loads of the q rows and of the angles go first, the tile copies of the prologue behind them; the rotation
     // is done while the copies travel.
     uint4 qreg[8];
-    float2 cs[ROPE_Q ? 32 : 1];
+    uint4 cs[ROPE_Q ? 16 : 1];
     {
         const size_t qtok = (size_t)it.tok0 + (size_t)min(q_pos, L - 1);
         const char* qrow = q_ptr + (qtok * Hq + head) * 256;
@@ -356,10 +356,11 @@ __global__ __launch_bounds__(256, 2) void prefill_kernel(PrefillArgs a, const ch
         for (int ks = 0; ks < 8; ++ks) qreg[ks] = sp_load16(qrow + ks * 32 + h * 16);
         if constexpr (ROPE_Q) {
             // d = 16 ks + 8 h + e (ks < 4) pairs with d + 64, which this lane holds at step ks + 4.  The table is
-            // laid out pair by pair, so the 32 rows of a half-wave read 256 consecutive bytes per pair.
-            const float2* tab = a.rope_table + min(q_pos, L - 1);
+            // laid out couple of pairs by couple of pairs, so the 32 rows of a half-wave read 512 consecutive bytes
+            // per load.
+            const float4* tab = a.rope_table + min(q_pos, L - 1);
 #pragma unroll
-            for (int e = 0; e < 32; ++e) cs[e] = sp_load8(tab + (size_t)(16 * (e >> 3) + 8 * h + (e & 7)) * a.rope_pitch);
+            for (int e = 0; e < 16; ++e) cs[e] = sp_load16(tab + (size_t)(8 * (e >> 2) + 4 * h + (e & 3)) * a.rope_pitch);
         }
     }
     int copies = 0; // tile copies issued so far
@@ -373,12 +374,14 @@ __global__ __launch_bounds__(256, 2) void prefill_kernel(PrefillArgs a, const ch
     for (int ks = 0; ks < 8; ++ks) sp_loads_arrived(qreg[ks]);
     if constexpr (ROPE_Q) {
 #pragma unroll
-        for (int e = 0; e < 32; ++e) sp_loads_arrived(cs[e]);
+        for (int e = 0; e < 16; ++e) sp_loads_arrived(cs[e]);
 #pragma unroll
         for (int ks = 0; ks < 4; ++ks)
 #pragma unroll
             for (int w = 0; w < 4; ++w) {
-                const float2 c0 = cs[8 * ks + 2 * w], c1 = cs[8 * ks + 2 * w + 1]; // pairs i = 16 ks + 8 h + 2 w, i + 1
+                const uint4 cw = cs[4 * ks + w]; // pairs i = 16 ks + 8 h + 2 w, i + 1
+                const float2 c0 = make_float2(__uint_as_float(cw.x), __uint_as_float(cw.y));
+                const float2 c1 = make_float2(__uint_as_float(cw.z), __uint_as_float(cw.w));
                 const uint32_t xw = pf_u4(qreg[ks], w), yw = pf_u4(qreg[ks + 4], w);
                 float x0, y0, x1, y1;
                 rope_pair(M::lo(xw), M::lo(yw), c0.x, c0.y, x0, y0);
@@ -782,13 +785,15 @@ __global__ __launch_bounds__(256) void rope_ragged_kernel(RopeRaggedArgs a) {
     }
 }
 
-// cos / sin table for the q rotation inside the attention kernel, pair by pair: table[i][pos]
-__global__ __launch_bounds__(256) void rope_table_kernel(float2* table, uint32_t positions, uint32_t pitch, RopeFreqs freqs) {
-    const uint32_t pos = blockIdx.x * 256 + threadIdx.x, i = blockIdx.y;
+// cos / sin table for the q rotation inside the attention kernel: table[i / 2][pos] = (cos, sin) of pair i (even)
+// and of pair i + 1 at that position
+__global__ __launch_bounds__(256) void rope_table_kernel(float4* table, uint32_t positions, uint32_t pitch, RopeFreqs freqs) {
+    const uint32_t pos = blockIdx.x * 256 + threadIdx.x, i = 2 * blockIdx.y;
     if (pos >= positions) return;
-    float s, c;
-    sincosf((float)pos * freqs.f[i], &s, &c);
-    table[(size_t)i * pitch + pos] = make_float2(c, s);
+    float s0, c0, s1, c1;
+    sincosf((float)pos * freqs.f[i], &s0, &c0);
+    sincosf((float)pos * freqs.f[i + 1], &s1, &c1);
+    table[(size_t)blockIdx.y * pitch + pos] = make_float4(c0, s0, c1, s1);
 }
 
 static inline size_t pf_align_up(size_t x, size_t a) { return (x + a - 1) / a * a; }
@@ -990,7 +995,7 @@ extern "C" int bz_batch_prefill_ragged(bz_prefill_plan_t* plan_, void* q, const 
         const float theta = rope_theta > 0.f ? rope_theta : 1e4f;
         const RopeFreqs freqs = make_rope_freqs(128, theta);
         if (p->rope_table && (!p->rope_table_valid || p->rope_table_theta != theta)) {
-            hipLaunchKernelGGL(rope_table_kernel, dim3((p->max_len + 255) / 256, 64), dim3(256), 0, s, (float2*)p->rope_table,
+            hipLaunchKernelGGL(rope_table_kernel, dim3((p->max_len + 255) / 256, 32), dim3(256), 0, s, (float4*)p->rope_table,
                                p->max_len, p->max_len, freqs);
             BZ_LAUNCH_CHECK();
             p->rope_table_theta = theta;
@@ -1012,7 +1017,7 @@ extern "C" int bz_batch_prefill_ragged(bz_prefill_plan_t* plan_, void* q, const 
     PrefillArgs a;
     a.out = out;
     a.items = p->items_d;
-    a.rope_table = (const float2*)p->rope_table;
+    a.rope_table = (const float4*)p->rope_table;
     a.rope_pitch = p->max_len;
     a.num_qo_heads = num_qo_heads; a.num_kv_heads = num_kv_heads;
     a.causal = causal ? 1 : 0;

@@ -100,10 +100,11 @@ PREFILL_BF16_WIDEN_V_ERR = 5e-4
 
 
 def prefill_angle_table(float_ws, max_len, D=128):
-    """The (cos, sin) table the prefill call keeps in its float workspace for the q rotation: fp32 [D/2 pairs][max_len
-    positions][2], as the device computed it (sincosf(pos * f_i)); max_len is the longest request of the plan."""
+    """The (cos, sin) table the prefill call keeps in its float workspace for the q rotation, as the device computed
+    it (sincosf(pos * f_i)), returned as fp32 [D/2 pairs][max_len positions][2]; max_len is the longest request of the
+    plan.  (The device keeps it as [pairs / 2][max_len][cos i, sin i, cos i+1, sin i+1].)"""
     raw = float_ws[: (D // 2) * max_len * 8].cpu().numpy().view(np.float32)
-    return raw.reshape(D // 2, max_len, 2)
+    return raw.reshape(D // 4, max_len, 2, 2).transpose(0, 2, 1, 3).reshape(D // 2, max_len, 2)
 
 
 def prefill_q_as_fed(q_bits, dtype, indptr, Hq, D, theta, table, sm_scale=None):
