@@ -48,6 +48,7 @@ struct DecodeArgs {
     int rope_mode;
     float sm_scale_log2; // sm_scale * log2(e)
     const float2* rope_table; // BZ_ROPE_FULL: (cos, sin) per [position][pair] or nullptr (angles computed on the fly)
+    int rope_positions;       // positions the table holds: every slot of every page the plan lists
     RopeFreqs freqs;
 };
 
@@ -187,7 +188,9 @@ __global__ __launch_bounds__(256) void decode_general_kernel(DecodeArgs a) {
         int(&jj)[UNROLL] = S.jj;
         float4 cs[TABLE ? TU : 1][4]; // (cos, sin) of this lane's eight pairs at the positions of TU tokens
         auto fetch_cs = [&](int u) {
-            const int jc = valid[u] ? jj[u] : tok_begin;
+            // (a sequence cannot be longer than its planned pages hold, which the table covers; the bound keeps the
+            // read inside the table whatever the device-side lengths say)
+            const int jc = min(valid[u] ? jj[u] : tok_begin, a.rope_positions - 1);
             const float4* row = cs_lane + (size_t)jc * (D / 4); // D/2 pairs of 8 bytes = D/4 float4 per position
 #pragma unroll
             for (int i = 0; i < 4; ++i) cs[u % TU][i] = row[i];
@@ -478,6 +481,7 @@ static int batch_decode_impl(DecodePlan* p, const void* q, int q_dtype, const bz
     a.group_div = 1;
     a.rope_mode = rope_mode;
     a.rope_table = nullptr;
+    a.rope_positions = 0;
     if (!(sm_scale > 0.f)) sm_scale = 1.0f / sqrtf((float)D);
     a.sm_scale_log2 = sm_scale * 1.4426950408889634f;
     a.freqs = make_rope_freqs(D, rope_theta > 0.f ? rope_theta : 1e4f);
@@ -488,7 +492,6 @@ static int batch_decode_impl(DecodePlan* p, const void* q, int q_dtype, const bz
             rc = decode_fast_path(p, q, out, lse, q_dtype, out_dtype, rope_mode, a.sm_scale_log2, a.freqs, kv,
                                   num_qo_heads, k_scale, v_scale, bufs.mfma_part_o, bufs.mfma_part_lse, false, s);
         if (rc == 0) {
-            if (!bufs_or_null) p->rope_table_valid = false; // its partials share the workspace with the angle table
             // the MFMA path brings its own combine; only empty sequences are left to do
             if (p->num_empty > 0) {
                 const uint32_t row = num_qo_heads * D;
@@ -506,22 +509,22 @@ static int batch_decode_impl(DecodePlan* p, const void* q, int q_dtype, const bz
             while (G % Gk) Gk >>= 1;
             a.group_div = (uint32_t)(G / Gk);
             // kRoPELlama on a raw-K cache: the angle table behind the general partials of the plan's own float
-            // workspace, when it fits (512 bytes per position at head_dim 128)
+            // workspace, when it fits (512 bytes per position at head_dim 128).  It is written by every call, on the
+            // call's stream, in front of the kernel that reads it (a few microseconds): the workspace may be shared
+            // with other handlers between calls, calls may change streams, and a captured call must replay its own
+            // fill -- a table kept from an earlier call could be stale in each of these cases without any sign of it.
             if (rope_mode == BZ_ROPE_FULL && !bufs_or_null && p->max_seq_len > 0) {
                 const size_t off = (p->general_part_bytes + 255) / 256 * 256;
-                const size_t tbytes = (size_t)p->max_seq_len * (size_t)(D / 2) * sizeof(float2);
+                const uint32_t positions = (p->max_seq_len + p->page_size - 1) / p->page_size * p->page_size;
+                const size_t tbytes = (size_t)positions * (size_t)(D / 2) * sizeof(float2);
                 if (off + tbytes <= p->float_buffer_bytes) {
                     float2* table = reinterpret_cast<float2*>(reinterpret_cast<char*>(p->part_o) + off);
-                    const float theta = rope_theta > 0.f ? rope_theta : 1e4f;
-                    if (!p->rope_table_valid || p->rope_table_theta != theta) {
-                        const uint32_t n = p->max_seq_len * (uint32_t)(D / 2);
-                        hipLaunchKernelGGL(decode_rope_table_kernel, dim3((n + 255) / 256), dim3(256), 0, s, table,
-                                           p->max_seq_len, (uint32_t)(D / 2), a.freqs);
-                        BZ_LAUNCH_CHECK();
-                        p->rope_table_valid = true;
-                        p->rope_table_theta = theta;
-                    }
+                    const uint32_t n = positions * (uint32_t)(D / 2);
+                    hipLaunchKernelGGL(decode_rope_table_kernel, dim3((n + 255) / 256), dim3(256), 0, s, table, positions,
+                                       (uint32_t)(D / 2), a.freqs);
+                    BZ_LAUNCH_CHECK();
                     a.rope_table = table;
+                    a.rope_positions = (int)positions;
                 }
             }
             dim3 grid(p->num_segments, kv->num_kv_heads * a.group_div);
@@ -569,8 +572,9 @@ constexpr int kMaxDevices = 64;
 static std::mutex g_scratch_mutex;
 static void* g_scratch_ptr[kMaxDevices] = {nullptr};
 
-// Device address of this GPU's copy of the scratch array (looked up on the first call per device,
-// with that device current).
+// Device address of this GPU's copy of the scratch array (looked up once per device, with that device
+// current: by bz_decode_plan through decode_noalloc_prepare, so that bz_batch_decode_noalloc itself finds it
+// there and does nothing but launch).
 static int decode_scratch_for_current_device(unsigned char** ptr) {
     int dev = 0;
     BZ_CHECK_HIP(hipGetDevice(&dev));
@@ -584,6 +588,11 @@ static int decode_scratch_for_current_device(unsigned char** ptr) {
     }
     *ptr = static_cast<unsigned char*>(g_scratch_ptr[dev]);
     return 0;
+}
+
+int decode_noalloc_prepare() {
+    unsigned char* ptr = nullptr;
+    return decode_scratch_for_current_device(&ptr);
 }
 
 static inline size_t scratch_align(size_t x) { return (x + 255) / 256 * 256; }
@@ -621,7 +630,6 @@ extern "C" int bz_decode_step(bz_decode_plan_t* plan_, const void* q, int q_dtyp
         const RopeFreqs freqs = make_rope_freqs(D, rope_theta > 0.f ? rope_theta : 1e4f);
         rc = decode_step_fast_path(p, q, k_new, v_new, out, lse, q_dtype, out_dtype, rope, scale * 1.4426950408889634f,
                                    freqs, kv, num_qo_heads, k_scale, v_scale, s);
-        if (rc == 0) p->rope_table_valid = false; // the step's partials share the workspace with the angle table
         if (rc == 0 && p->num_empty > 0) { // sequences without pages: nothing to append, zero rows
             const uint32_t row = num_qo_heads * D;
             if (out_dtype == BZ_F32) launch_zero<float>(p, out, row, s);
@@ -648,11 +656,13 @@ extern "C" int bz_batch_decode_noalloc(bz_decode_plan_t* plan_, const void* q, i
     DecodePlan* p = reinterpret_cast<DecodePlan*>(plan_);
     if (!p) return BZ_ERR_BAD_ARG;
     if (!p->planned) return BZ_ERR_NOT_PLANNED;
-    // partial results of whichever kernel the call ends up running must fit the fixed array
+    // The partial results must fit the fixed array.  Which of the two kernels a call runs depends on its arguments
+    // as well as on the plan, so the rule is the conservative one: what either kernel would need, unless the plan
+    // is pinned to the general kernel.
     const size_t gen_o = scratch_align((size_t)p->num_partials * p->num_qo_heads * p->head_dim * sizeof(float));
     const size_t gen_l = scratch_align((size_t)p->num_partials * p->num_qo_heads * sizeof(float));
-    const size_t mf_o = p->mfma_ok ? scratch_align((size_t)p->mfma_partials * 16 * 128 * sizeof(float)) : 0;
-    const size_t mf_l = p->mfma_ok ? scratch_align((size_t)p->mfma_partials * 16 * sizeof(float)) : 0;
+    const size_t mf_o = (p->mfma_ok && !p->force_general) ? scratch_align((size_t)p->mfma_partials * 16 * 128 * sizeof(float)) : 0;
+    const size_t mf_l = (p->mfma_ok && !p->force_general) ? scratch_align((size_t)p->mfma_partials * 16 * sizeof(float)) : 0;
     if (gen_o + gen_l > (size_t)BZ_DECODE_NOALLOC_SCRATCH_BYTES || mf_o + mf_l > (size_t)BZ_DECODE_NOALLOC_SCRATCH_BYTES)
         return BZ_ERR_WORKSPACE;
     unsigned char* base = nullptr;

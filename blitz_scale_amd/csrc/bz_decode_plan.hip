@@ -352,7 +352,6 @@ extern "C" int bz_decode_plan(bz_decode_plan_t* plan_, void* float_buffer, size_
     p->empty_d = (const int32_t*)((char*)int_buffer + seg_bytes + combo_bytes);
     p->float_buffer_bytes = float_buffer_bytes;
     p->general_part_bytes = part_o_bytes + part_lse_bytes;
-    p->rope_table_valid = false;
     p->max_seq_len = 0;
     for (uint32_t b = 0; b < batch_size; ++b) {
         const int32_t np = indptr_h[b + 1] - indptr_h[b];
@@ -411,6 +410,7 @@ extern "C" int bz_decode_plan(bz_decode_plan_t* plan_, void* float_buffer, size_
         p->step_one_call = applies && (force_one_call || mostly_split);
     }
 
+    (void)decode_noalloc_prepare(); // (a failure is reported by bz_batch_decode_noalloc itself, should it be called)
     p->planned = true;
     return 0;
 }

@@ -129,8 +129,6 @@ struct DecodePlan {
     // a plan() (any call that puts matrix-core partials into the workspace invalidates it)
     uint32_t max_seq_len = 0;       // longest sequence of the planned table
     size_t general_part_bytes = 0;  // bytes of the general kernel's partials at the start of the float workspace
-    bool rope_table_valid = false;
-    float rope_table_theta = 0.f;
     // host scratch of plan(), kept between calls so that a step's plan neither allocates nor faults in
     // fresh pages (the schedule of a large batch is around a megabyte)
     std::vector<DecodeSegment> h_segs;
@@ -147,5 +145,9 @@ struct DecodePlan {
     hipEvent_t time_start = nullptr, time_stop = nullptr; // optional: bracket the decode kernel launch
     int device = -1;
 };
+
+// Looks up, for the current device, the address of the fixed array that bz_batch_decode_noalloc keeps its
+// partial results in (bz_decode.hip); called by bz_decode_plan so that the call itself only launches kernels.
+int decode_noalloc_prepare();
 
 } // namespace bz

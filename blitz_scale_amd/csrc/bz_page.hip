@@ -29,8 +29,9 @@ struct PageWriteArgs {
 };
 
 // The rows of one token (q heads to rotate in place, then the k heads, then the v heads) on their way into
-// page `page`, slot `slot`.  A row of D elements is handled by D/16 lanes; each lane owns 8 elements of the
-// lower half and the 8 elements of the upper half that form rotate-half pairs with them.
+// page `page`, slot `slot` (page < 0: the token has no page; its rows are still rotated in place where the call
+// rotates in place, and nothing goes to the pool).  A row of D elements is handled by D/16 lanes; each lane owns
+// 8 elements of the lower half and the 8 elements of the upper half that form rotate-half pairs with them.
 template <typename ST, typename PT, int D, bool PREFILL>
 __device__ __forceinline__ void page_write_rows(const PageWriteArgs& a, int64_t page, int slot, size_t src_tok,
                                                 const float* s_cos, const float* s_sin) {
@@ -71,6 +72,9 @@ __device__ __forceinline__ void page_write_rows(const PageWriteArgs& a, int64_t 
         }
         const bool is_k = r < Hq + Hkv;
         const int h = is_k ? r - Hq : r - Hq - Hkv;
+        const bool to_pool = page >= 0;
+        const bool in_place = PREFILL && is_k && a.rope && (Hq > 0 || a.rope == 2);
+        if (!to_pool && !in_place) continue;
         const ST* src = reinterpret_cast<const ST*>(is_k ? a.k_src : a.v_src) + (src_tok * Hkv + h) * D;
         char* pool = is_k ? a.k_data : a.v_data;
         const size_t off = ((size_t)page * a.stride_page + (size_t)slot * a.stride_n + (size_t)h * a.stride_h);
@@ -113,6 +117,7 @@ __device__ __forceinline__ void page_write_rows(const PageWriteArgs& a, int64_t 
             lr.store(srcw + lane * 8);
             hr.store(srcw + D / 2 + lane * 8);
         }
+        if (!to_pool) continue;
         if (scale) {
             const float sc = scale[h];
 #pragma unroll
@@ -137,6 +142,7 @@ __global__ __launch_bounds__(256) void page_write_kernel(PageWriteArgs a) {
     for (int unit = blockIdx.x; unit < total; unit += gridDim.x) {
         int b, pos;
         size_t src_tok;
+        bool no_page = false;
         if (PREFILL) {
             const int n = unit; // global token index; largest b with ragged_indptr[b] <= n (wave-uniform search)
             int lo = 0, hi = (int)a.batch_size;
@@ -148,9 +154,11 @@ __global__ __launch_bounds__(256) void page_write_kernel(PageWriteArgs a) {
             pos = n - a.ragged_indptr[b];
             src_tok = (size_t)n;
             // a request longer than the pages its table row lists (the reference asserts seq_len >= append
-            // length, src/kernel/page.cu:43): the tokens without a page are dropped, nothing is written
-            // outside the listed pages
-            if (pos / (int)a.page_size >= a.indptr[b + 1] - a.indptr[b]) continue;
+            // length, src/kernel/page.cu:43): the tokens without a page are not cached -- nothing is written
+            // outside the listed pages -- but a call that rotates q / k in place still rotates their rows, so
+            // that the attention call which follows sees every row of the request rotated alike
+            no_page = pos / (int)a.page_size >= a.indptr[b + 1] - a.indptr[b];
+            if (no_page && !(a.rope && (a.q_inout || a.rope == 2))) continue;
         } else {
             b = unit;
             const int ahead = a.steps_ahead ? *a.steps_ahead : 0; // fetched together with the table entries
@@ -160,7 +168,7 @@ __global__ __launch_bounds__(256) void page_write_kernel(PageWriteArgs a) {
             if (pos < 0) continue; // the sequence has no token yet at the present step
             src_tok = (size_t)b;
         }
-        const int64_t page = a.indices[a.indptr[b] + pos / (int)a.page_size];
+        const int64_t page = no_page ? -1 : a.indices[a.indptr[b] + pos / (int)a.page_size];
         const int slot = pos % (int)a.page_size;
 
         if (a.rope) {

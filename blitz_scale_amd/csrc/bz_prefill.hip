@@ -57,11 +57,9 @@ struct PrefillPlan {
     uint32_t batch_size = 0, num_qo_heads = 0, num_kv_heads = 0, head_dim = 0, num_items = 0;
     uint32_t total_tokens = 0, max_len = 0;
     const PrefillItem* items_d = nullptr;
-    // cos / sin of position * frequency for every position a request of this batch has (float workspace),
-    // filled by the first attention call that rotates q after a plan(), for the RoPE base of that call
+    // cos / sin of position * frequency for every position a request of this batch has (float workspace), written by
+    // every attention call that rotates q, on its own stream, in front of the attention kernel
     float* rope_table = nullptr; // [32 couples of pairs][max_len] x (cos, sin, cos, sin); nullptr: the float workspace has no room
-    float rope_table_theta = 0.f;
-    bool rope_table_valid = false;
     std::vector<PrefillItem> h_items; // host copy of the last job list (kept between calls)
     void* staging = nullptr;
     size_t staging_bytes = 0;
@@ -942,7 +940,6 @@ extern "C" int bz_prefill_plan(bz_prefill_plan_t* plan_, void* float_buffer, siz
     // the float workspace holds the angle table of the q rotation when it has room for it (512 bytes per position)
     p->rope_table = (float_buffer && (size_t)p->max_len * 512 <= float_buffer_bytes && (uintptr_t)float_buffer % 16 == 0)
                         ? (float*)float_buffer : nullptr;
-    p->rope_table_valid = false;
     p->planned = true;
     return 0;
 }
@@ -994,12 +991,12 @@ extern "C" int bz_batch_prefill_ragged(bz_prefill_plan_t* plan_, void* q, const 
     if (rope_mode != BZ_ROPE_NONE) {
         const float theta = rope_theta > 0.f ? rope_theta : 1e4f;
         const RopeFreqs freqs = make_rope_freqs(128, theta);
-        if (p->rope_table && (!p->rope_table_valid || p->rope_table_theta != theta)) {
+        if (p->rope_table) {
+            // (every call: the workspace may be shared with other handlers between calls, calls may change streams,
+            // and a captured call must replay its own fill; a few microseconds)
             hipLaunchKernelGGL(rope_table_kernel, dim3((p->max_len + 255) / 256, 32), dim3(256), 0, s, (float4*)p->rope_table,
                                p->max_len, p->max_len, freqs);
             BZ_LAUNCH_CHECK();
-            p->rope_table_theta = theta;
-            p->rope_table_valid = true;
         }
         RopeRaggedArgs ra;
         ra.q = p->rope_table ? nullptr : q; // no room for the table: q is rotated in place instead

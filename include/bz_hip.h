@@ -188,9 +188,11 @@ int bz_decode_step(bz_decode_plan_t* plan, const void* q, int q_dtype, const voi
  * except that the split-K partial results go to a fixed device array inside the library
  * (BZ_DECODE_NOALLOC_SCRATCH_BYTES per GPU, held from module load to process exit) instead of the float
  * workspace given to bz_decode_plan; that workspace is not touched by this call.  The call itself performs
- * no allocation, free, copy or synchronisation: it only launches kernels on `stream`.
+ * no allocation, free, copy or synchronisation: it only launches kernels on `stream` (the array's address on
+ * the current GPU is looked up by bz_decode_plan), so it may be recorded into a HIP graph.
  * Limit: the plan's partial results must fit the array (8256 bytes per partial of the matrix-core kernel,
- * 4*(head_dim+1)*num_qo_heads per partial of the general kernel); otherwise BZ_ERR_WORKSPACE is returned
+ * 4*(head_dim+1)*num_qo_heads per partial of the general kernel; the rule is conservative: what either kernel
+ * would need for this plan, whichever the call ends up running); otherwise BZ_ERR_WORKSPACE is returned
  * before anything is launched.  All calls on one GPU share that GPU's array: calls that overlap in time on
  * one GPU (two streams, two threads) race; calls in stream order are safe, and nothing in the array has to
  * be cleared between them (every partial the combine reads is written by the same call first).

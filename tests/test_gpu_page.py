@@ -1,6 +1,7 @@
 """GPU parity: KV page writes (prefill store, decode append, fused RoPE, e4m3 quantisation).
 Placement and raw copies are bit-exact; rotated / quantised rows are compared value-wise because the
-device uses fused multiply-adds in the rotation (one storage step on rare elements)."""
+device's sincosf may differ from the host's in the last place (one storage step on rare elements; the rotation
+itself rounds every product and sum on its own on both sides)."""
 import numpy as np
 import pytest
 import torch
@@ -174,6 +175,38 @@ def test_store_prefill_drops_tokens_beyond_the_listed_pages():
     K.store_prefill_kv_cache(dev.pt, to_dev(k, dtype), to_dev(v, dtype), to_dev(ri.view(np.float32), 3).view(torch.int32))
     torch.cuda.synchronize()
     assert np.array_equal(to_host_bits(dev.pool), want)
+
+
+@pytest.mark.parametrize("with_q", [False, True])
+def test_store_prefill_rotates_in_place_also_what_it_cannot_cache(with_q):
+    """Tokens beyond the listed pages are not cached, but a store that rotates in place (rope = 2, or the fused
+    form with q) still rotates their rows: the attention call that follows must see the whole request rotated."""
+    rng = np.random.default_rng(66)
+    Hq, Hkv, D, P, dtype, theta = 4, 2, 128, 16, BZ_F16, 1e4
+    p, fill = _setup(67, [20, 40], Hq, Hkv, D, P, dtype, BZ_LAYOUT_HND, reserve_extra=0)  # 2 and 3 pages
+    ri = np.array([0, 20, 120], np.int32)                                                 # request 1 claims 100 tokens
+    q = wl.randn_bits(rng, (120, Hq, D), dtype)
+    k, v = wl.randn_bits(rng, (120, Hkv, D), dtype), wl.randn_bits(rng, (120, Hkv, D), dtype)
+    want = p.pool.copy()
+    ri_fit = np.array([0, 20, 68], np.int32)  # what fits: 3 pages x 16 slots of request 1
+    oracle.store_prefill_kv(p.oracle_kv(want), k[:68], v[:68], dtype, ri_fit, rope=True, rope_theta=theta)
+    want_k = oracle.rope_ragged(k, dtype, ri, Hkv, D, theta)
+    want_q = oracle.rope_ragged(q, dtype, ri, Hq, D, theta)
+    dev = DeviceDecode(p)
+    qd, kd, vd = to_dev(q, dtype), to_dev(k, dtype), to_dev(v, dtype)
+    rid = to_dev(ri.view(np.float32), 3).view(torch.int32)
+    if with_q:
+        K.store_prefill_kv_cache(dev.pt, kd, vd, rid, q=qd, num_qo_heads=Hq, rope=True, rope_theta=theta)
+    else:
+        K.store_prefill_kv_cache(dev.pt, kd, vd, rid, rope=2, rope_theta=theta)
+    torch.cuda.synchronize()
+    pairs = [(to_host_bits(dev.pool), want), (to_host_bits(kd), want_k)] + ([(to_host_bits(qd), want_q)] if with_q else [])
+    for g, w in pairs:
+        assert np.abs(wl.to_f32(g, dtype) - wl.to_f32(w, dtype)).max() <= 2.0 ** -8
+        assert (g != w).mean() < 2e-3
+    if not with_q:
+        assert np.array_equal(to_host_bits(qd), q)
+    assert np.array_equal(to_host_bits(vd), v)
 
 
 def test_store_prefill_rotates_k_in_place_without_q():

@@ -95,3 +95,40 @@ def test_rejects_plans_beyond_the_fixed_array():
     K.batch_decode_attention(dev.handler, dev.q, dev.pt, out, p.Hq, rope_mode=BZ_ROPE_NONE)  # the workspace form still works
     torch.cuda.synchronize()
     assert out.any()
+
+
+def test_recorded_into_a_hip_graph_and_replayed():
+    """The call only launches kernels, so it can be captured: three replays with new q contents, eager work and
+    synchronisations between them, each compared bit for bit with the same call launched eagerly."""
+    p = DecodeProblem(907, [5000, 17, 2049, 640, 1, 300], 32, 8, 128, 16, BZ_BF16)
+    dev = DeviceDecode(p)
+    info = dev.plan(1024)  # (bz_decode_plan looks the array up: nothing but launches is left to the call)
+    assert info["split_seqs"] >= 1
+    side = torch.cuda.Stream()
+    q = dev.q.clone()
+    out_g = torch.empty((p.B, p.Hq, p.D), dtype=torch.bfloat16, device="cuda")
+    out_e = torch.empty_like(out_g)
+
+    def call(out, stream):
+        K.batch_decode_attention_noalloc(dev.handler, q, dev.pt, out, p.Hq, rope_mode=BZ_ROPE_Q_ONLY, rope_theta=5e5,
+                                         stream=stream)
+
+    with torch.cuda.stream(side):
+        call(out_g, side.cuda_stream)  # warm-up on the capture stream, outside the capture
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        call(out_g, torch.cuda.current_stream().cuda_stream)
+    torch.cuda.synchronize()
+    g = torch.Generator(device="cuda")
+    g.manual_seed(907)
+    for _ in range(3):
+        q.copy_(torch.randn(q.shape, dtype=torch.float32, device="cuda", generator=g).to(q.dtype))
+        out_g.fill_(float("nan"))
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        call(out_e, None)
+        torch.cuda.synchronize()
+        assert not torch.isnan(out_g.float()).any()
+        assert torch.equal(out_g.view(torch.int16), out_e.view(torch.int16))
