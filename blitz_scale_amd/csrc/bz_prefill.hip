@@ -45,17 +45,20 @@ __device__ __forceinline__ void lds_direct_load16(const char* uniform_base, uint
 }
 
 struct PrefillItem { // one workgroup's job, in launch order
-    int32_t tok0; // global index of the request's first token
-    int32_t len;  // tokens in the request (0: padding entry, nothing to do)
-    int32_t q0;   // first q row of this tile, relative to the request
-    int32_t head; // q head
+    int32_t tok0;   // global index of the request's first q row
+    int32_t len;    // q rows of the request (0: padding entry, nothing to do)
+    int32_t q0;     // first q row of this tile, relative to the request
+    int32_t head;   // q head
+    int32_t kv0;    // global index of the request's first K/V row
+    int32_t kv_len; // K/V rows of the request (>= len); q row i sits at position kv_len - len + i
+    int32_t pad[2];
 };
 
 struct PrefillPlan {
     bool planned = false;
     bool bf16_head_tail = false; // bf16: probabilities as head + tail of bf16 instead of V widened to f16 (bz_prefill_plan_set_bf16_mode)
     uint32_t batch_size = 0, num_qo_heads = 0, num_kv_heads = 0, head_dim = 0, num_items = 0;
-    uint32_t total_tokens = 0, max_len = 0;
+    uint32_t total_tokens = 0, total_kv_tokens = 0, max_len = 0; // max_len: longest K/V length
     const PrefillItem* items_d = nullptr;
     // cos / sin of position * frequency for every position a request of this batch has (float workspace), written by
     // every attention call that rotates q, on its own stream, in front of the attention kernel
@@ -280,15 +283,18 @@ __global__ __launch_bounds__(256, 2) void prefill_kernel(PrefillArgs a, const ch
     const int Hq = (int)a.num_qo_heads, Hkv = (int)a.num_kv_heads;
     const int kvh = head / (Hq / Hkv);
     const int qn = lane & 31, h = lane >> 5;
-    const int L = it.len;
+    // Lq q rows attend to L K/V rows (L >= Lq); q row i of the request sits at position off + i: it sees, when
+    // causal, the tokens up to that position, and is rotated by that position.
+    const int L = it.kv_len, Lq = it.len, off = L - Lq;
     const int wave_q_lo = it.q0 + 32 * wv;
     const int q_pos = wave_q_lo + qn;
-    const int kv_limit = a.causal ? min(L, it.q0 + kBM) : L; // tokens any row of this workgroup can see
-    const int n = (kv_limit + kSN - 1) / kSN;                // tiles of the job
-    // tiles this wave computes (causal: up to its diagonal tile; none for rows past the end of the request)
-    const int n_w = wave_q_lo >= L ? 0 : (a.causal ? min(n, wave_q_lo / kSN + 1) : n);
-    const int t_diag = a.causal ? wave_q_lo / kSN : 0x7fffffff;
-    const int kv_max = a.causal ? min(q_pos, L - 1) : L - 1; // last token this row may see
+    const int kv_limit = a.causal ? min(L, off + it.q0 + kBM) : L; // tokens any row of this workgroup can see
+    const int n = (kv_limit + kSN - 1) / kSN;                      // tiles of the job
+    // tiles this wave computes (causal: up to the diagonal tile of its last row; none for rows past the end of the
+    // request); t_diag: the first tile in which one of its rows may have to be masked
+    const int n_w = wave_q_lo >= Lq ? 0 : (a.causal ? min(n, (off + wave_q_lo + 31) / kSN + 1) : n);
+    const int t_diag = a.causal ? (off + wave_q_lo) / kSN : 0x7fffffff;
+    const int kv_max = a.causal ? min(off + q_pos, L - 1) : L - 1; // last token this row may see
 
     // ---- global -> LDS staging: wave wv moves rows 8wv .. 8wv+7 of a tile, two instructions of four 256-byte
     // rows each for K and for V (chunk XOR patterns: see the kernel's header)
@@ -304,7 +310,7 @@ __global__ __launch_bounds__(256, 2) void prefill_kernel(PrefillArgs a, const ch
         kfast[i] = (uint32_t)(4 * i + r4) * row_stride + kcol[i] - (uint32_t)(i * 1024);
         vfast[i] = (uint32_t)(4 * i + r4) * row_stride + vcol - (uint32_t)(i * 1024);
     }
-    const size_t kv_row0 = ((size_t)it.tok0 * Hkv + kvh) * 256; // byte offset of the request's first K/V row
+    const size_t kv_row0 = ((size_t)it.kv0 * Hkv + kvh) * 256; // byte offset of the request's first K/V row
     const char* const k_wave = k_ptr + kv_row0 + (size_t)(8 * wv) * row_stride;
     const char* const v_wave = v_ptr + kv_row0 + (size_t)(8 * wv) * row_stride;
     const uint32_t m0_wave = lds0 + (uint32_t)(8 * wv * 256);
@@ -348,7 +354,7 @@ __global__ __launch_bounds__(256, 2) void prefill_kernel(PrefillArgs a, const ch
     uint4 qreg[8];
     uint4 cs[ROPE_Q ? 16 : 1];
     {
-        const size_t qtok = (size_t)it.tok0 + (size_t)min(q_pos, L - 1);
+        const size_t qtok = (size_t)it.tok0 + (size_t)min(q_pos, Lq - 1);
         const char* qrow = q_ptr + (qtok * Hq + head) * 256;
 #pragma unroll
         for (int ks = 0; ks < 8; ++ks) qreg[ks] = sp_load16(qrow + ks * 32 + h * 16);
@@ -356,7 +362,7 @@ __global__ __launch_bounds__(256, 2) void prefill_kernel(PrefillArgs a, const ch
             // d = 16 ks + 8 h + e (ks < 4) pairs with d + 64, which this lane holds at step ks + 4.  The table is
             // laid out couple of pairs by couple of pairs, so the 32 rows of a half-wave read 512 consecutive bytes
             // per load.
-            const float4* tab = a.rope_table + min(q_pos, L - 1);
+            const float4* tab = a.rope_table + (off + min(q_pos, Lq - 1));
 #pragma unroll
             for (int e = 0; e < 16; ++e) cs[e] = sp_load16(tab + (size_t)(8 * (e >> 2) + 4 * h + (e & 3)) * a.rope_pitch);
         }
@@ -461,7 +467,7 @@ __global__ __launch_bounds__(256, 2) void prefill_kernel(PrefillArgs a, const ch
 
     auto mask_tile = [&](int t, pf_f32x16& sc) __attribute__((always_inline)) {
         // element 4b+r of a score block is token 32t + 8b + 4h + r
-        if (t == t_diag || (t + 1) * kSN > L) {
+        if (t >= t_diag || (t + 1) * kSN > L) {
 #pragma unroll
             for (int i = 0; i < 16; ++i) {
                 const int kv = t * kSN + 8 * (i >> 2) + 4 * h + (i & 3);
@@ -702,7 +708,7 @@ __global__ __launch_bounds__(256, 2) void prefill_kernel(PrefillArgs a, const ch
     for (int ps = 0; ps < 8; ++ps) {
         const int row = 4 * ps + (lane >> 4);
         const int pos = wave_q_lo + row;
-        if (pos < L) {
+        if (pos < Lq) {
             const uint4 v = *reinterpret_cast<const uint4*>(o_lds + row * 256 + (((lane & 15) ^ (row & 15)) * 16));
             char* orow = (char*)a.out + (((size_t)it.tok0 + pos) * Hq + head) * 256;
             *reinterpret_cast<uint4*>(orow + (lane & 15) * 16) = v;
@@ -723,12 +729,14 @@ __global__ __launch_bounds__(256, 2) void prefill_kernel(PrefillArgs a, const ch
 #endif
 }
 
-// ---- in-place RoPE of ragged q and k rows (used when the caller asks the attention call itself to rotate)
+// ---- in-place RoPE of ragged rows, one token per workgroup (used when the caller asks the attention call itself to
+// rotate).  K rows sit at their index inside the request; q rows, when a request has more K/V rows than q rows, at
+// that index plus the difference (`longer`: the K/V index of the batch, given for q rows only).
 struct RopeRaggedArgs {
-    void* q;
-    void* k;
-    const int32_t* indptr;
-    uint32_t batch_size, num_qo_heads, num_kv_heads;
+    void* rows;
+    const int32_t* indptr; // ragged index of `rows`
+    const int32_t* longer; // nullptr, or the ragged index whose request lengths set the offset of the positions
+    uint32_t batch_size, num_heads;
     RopeFreqs freqs;
 };
 
@@ -748,7 +756,8 @@ __global__ __launch_bounds__(256) void rope_ragged_kernel(RopeRaggedArgs a) {
         s_b = lo;
     }
     __syncthreads();
-    const int pos = tok - a.indptr[s_b];
+    int pos = tok - a.indptr[s_b];
+    if (a.longer) pos += (a.longer[s_b + 1] - a.longer[s_b]) - (a.indptr[s_b + 1] - a.indptr[s_b]);
     if (threadIdx.x < 64) {
         float s, c;
         sincosf((float)pos * a.freqs.f[threadIdx.x], &s, &c);
@@ -757,11 +766,8 @@ __global__ __launch_bounds__(256) void rope_ragged_kernel(RopeRaggedArgs a) {
     }
     __syncthreads();
     const int lane8 = threadIdx.x & 7; // 8 lanes per row: 8 low-half and the 8 matching high-half elements each
-    const int nq = a.q ? (int)a.num_qo_heads : 0, nk = a.k ? (int)a.num_kv_heads : 0; // either may be left alone
-    const int rows = nq + nk;
-    for (int r = threadIdx.x >> 3; r < rows; r += 32) {
-        T* row = (r < nq) ? reinterpret_cast<T*>(a.q) + ((size_t)tok * a.num_qo_heads + r) * 128
-                          : reinterpret_cast<T*>(a.k) + ((size_t)tok * a.num_kv_heads + (r - nq)) * 128;
+    for (int r = threadIdx.x >> 3; r < (int)a.num_heads; r += 32) {
+        T* row = reinterpret_cast<T*>(a.rows) + ((size_t)tok * a.num_heads + r) * 128;
         Vec8<T> lo, hi;
         lo.load(row + lane8 * 8);
         hi.load(row + 64 + lane8 * 8);
@@ -829,9 +835,14 @@ static int build_prefill_items(PrefillPlan* p, const int32_t* qo_indptr_h, const
     if (num_kv_heads == 0 || num_qo_heads % num_kv_heads) return BZ_ERR_BAD_ARG;
     p->planned = false;
     if (head_dim != 128) return BZ_ERR_UNSUPPORTED;
-    // self-attention only: the reference passes the same array twice (src/layer/attn.h:175-187)
-    for (uint32_t b = 0; b <= batch_size; ++b)
-        if (qo_indptr_h[b] != kv_indptr_h[b]) return BZ_ERR_UNSUPPORTED;
+    // The reference passes the same array twice (src/layer/attn.h:175-187).  With two arrays a request has q rows
+    // for its last tokens only (a chunk of a prompt whose earlier K/V rows are given again): at least as many
+    // K/V rows as q rows.
+    if (qo_indptr_h[0] != 0 || kv_indptr_h[0] != 0) return BZ_ERR_BAD_ARG;
+    for (uint32_t b = 0; b < batch_size; ++b) {
+        if (kv_indptr_h[b + 1] < kv_indptr_h[b]) return BZ_ERR_BAD_ARG;
+        if (kv_indptr_h[b + 1] - kv_indptr_h[b] < qo_indptr_h[b + 1] - qo_indptr_h[b]) return BZ_ERR_UNSUPPORTED;
+    }
     // One entry per workgroup, in launch order.  Workgroups are dealt round-robin to the 8 XCDs, each
     // with its own L2, so launch index i runs on XCD i % 8.  Every (request, kv head) unit is given to one
     // XCD as a run of consecutive jobs: its q tiles (of all q heads of the group) then execute together on
@@ -842,8 +853,8 @@ static int build_prefill_items(PrefillPlan* p, const int32_t* qo_indptr_h, const
         if (qo_indptr_h[b + 1] < qo_indptr_h[b]) return BZ_ERR_BAD_ARG;
     std::vector<uint32_t> order(batch_size);
     for (uint32_t b = 0; b < batch_size; ++b) order[b] = b;
-    std::stable_sort(order.begin(), order.end(), [&](uint32_t x, uint32_t y) {
-        return qo_indptr_h[x + 1] - qo_indptr_h[x] > qo_indptr_h[y + 1] - qo_indptr_h[y];
+    std::stable_sort(order.begin(), order.end(), [&](uint32_t x, uint32_t y) { // (a tile's work goes with the K/V length)
+        return kv_indptr_h[x + 1] - kv_indptr_h[x] > kv_indptr_h[y + 1] - kv_indptr_h[y];
     });
     constexpr int kXcd = 8;
     std::vector<PrefillItem> per_xcd[kXcd];
@@ -864,12 +875,13 @@ static int build_prefill_items(PrefillPlan* p, const int32_t* qo_indptr_h, const
         for (uint32_t unit = 0; unit < num_kv_heads * parts; ++unit, ++pair)
             for (int32_t q0 = last_q0; q0 >= 0; q0 -= kBM)
                 for (uint32_t g = 0; g < per_part; ++g)
-                    per_xcd[pair % kXcd].push_back({qo_indptr_h[b], len, q0, (int32_t)(unit * per_part + g)});
+                    per_xcd[pair % kXcd].push_back({qo_indptr_h[b], len, q0, (int32_t)(unit * per_part + g), kv_indptr_h[b],
+                                                    kv_indptr_h[b + 1] - kv_indptr_h[b], {0, 0}});
     }
     size_t longest = 0;
     for (auto& v : per_xcd) longest = std::max(longest, v.size());
     std::vector<PrefillItem>& items = p->h_items;
-    items.assign(longest * kXcd, PrefillItem{0, 0, 0, 0});
+    items.assign(longest * kXcd, PrefillItem{0, 0, 0, 0, 0, 0, {0, 0}});
     for (int x = 0; x < kXcd; ++x)
         for (size_t k = 0; k < per_xcd[x].size(); ++k) items[k * kXcd + x] = per_xcd[x][k];
     return 0;
@@ -883,7 +895,7 @@ extern "C" int bz_prefill_plan_workspace(bz_prefill_plan_t* plan_, const int32_t
     if (rc) return rc;
     if (float_buffer_bytes) { // the angle table of the q rotation: 512 bytes per position of the longest request
         int32_t longest = 0;
-        for (uint32_t b = 0; b < batch_size; ++b) longest = std::max(longest, qo_indptr_h[b + 1] - qo_indptr_h[b]);
+        for (uint32_t b = 0; b < batch_size; ++b) longest = std::max(longest, kv_indptr_h[b + 1] - kv_indptr_h[b]);
         *float_buffer_bytes = (size_t)longest * 512;
     }
     if (int_buffer_bytes) *int_buffer_bytes = pf_align_up(p->h_items.size() * sizeof(PrefillItem), 256);
@@ -934,9 +946,10 @@ extern "C" int bz_prefill_plan(bz_prefill_plan_t* plan_, void* float_buffer, siz
     p->batch_size = batch_size; p->num_qo_heads = num_qo_heads; p->num_kv_heads = num_kv_heads;
     p->head_dim = head_dim;
     p->total_tokens = (uint32_t)qo_indptr_h[batch_size];
+    p->total_kv_tokens = (uint32_t)kv_indptr_h[batch_size];
     p->max_len = 0;
     for (uint32_t b = 0; b < batch_size; ++b)
-        p->max_len = std::max<uint32_t>(p->max_len, (uint32_t)(qo_indptr_h[b + 1] - qo_indptr_h[b]));
+        p->max_len = std::max<uint32_t>(p->max_len, (uint32_t)(kv_indptr_h[b + 1] - kv_indptr_h[b]));
     // the float workspace holds the angle table of the q rotation when it has room for it (512 bytes per position)
     p->rope_table = (float_buffer && (size_t)p->max_len * 512 <= float_buffer_bytes && (uintptr_t)float_buffer % 16 == 0)
                         ? (float*)float_buffer : nullptr;
@@ -998,17 +1011,18 @@ extern "C" int bz_batch_prefill_ragged(bz_prefill_plan_t* plan_, void* q, const 
                                p->max_len, p->max_len, freqs);
             BZ_LAUNCH_CHECK();
         }
-        RopeRaggedArgs ra;
-        ra.q = p->rope_table ? nullptr : q; // no room for the table: q is rotated in place instead
-        ra.k = rope_mode == BZ_ROPE_FULL ? k : nullptr;
-        ra.indptr = qo_indptr;
-        ra.batch_size = batch_size; ra.num_qo_heads = num_qo_heads; ra.num_kv_heads = num_kv_heads;
-        ra.freqs = freqs;
-        if (ra.q || ra.k) {
-            if (dtype == BZ_F16) hipLaunchKernelGGL((rope_ragged_kernel<f16_t>), dim3(p->total_tokens), dim3(256), 0, s, ra);
-            else hipLaunchKernelGGL((rope_ragged_kernel<bf16_t>), dim3(p->total_tokens), dim3(256), 0, s, ra);
-            BZ_LAUNCH_CHECK();
-        }
+        auto rotate_rows = [&](void* rows, const int32_t* indptr, const int32_t* longer, uint32_t heads, uint32_t tokens) {
+            RopeRaggedArgs ra;
+            ra.rows = rows; ra.indptr = indptr; ra.longer = longer;
+            ra.batch_size = batch_size; ra.num_heads = heads;
+            ra.freqs = freqs;
+            if (tokens == 0) return;
+            if (dtype == BZ_F16) hipLaunchKernelGGL((rope_ragged_kernel<f16_t>), dim3(tokens), dim3(256), 0, s, ra);
+            else hipLaunchKernelGGL((rope_ragged_kernel<bf16_t>), dim3(tokens), dim3(256), 0, s, ra);
+        };
+        if (rope_mode == BZ_ROPE_FULL) rotate_rows(k, kv_indptr, nullptr, num_kv_heads, p->total_kv_tokens);
+        if (!p->rope_table) rotate_rows(q, qo_indptr, kv_indptr, num_qo_heads, p->total_tokens); // no room for the table
+        BZ_LAUNCH_CHECK();
         rope_q = p->rope_table != nullptr;
     }
     PrefillArgs a;

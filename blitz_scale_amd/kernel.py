@@ -213,12 +213,13 @@ class BatchPrefillRaggedHandler:
         check(_lib.load().bz_prefill_plan_set_bf16_mode(self._h, mode), "Handler bf16 mode")
 
     def host_schedule(self):
-        """numpy copy [workgroups, 4] of the last job list: tok0, len (0 = padding), q0, head."""
+        """numpy copy [workgroups, 8] of the last job list: first q row and q rows of the request (0 = padding), first q
+        row of the tile, q head, first K/V row and K/V rows of the request, 0, 0."""
         data, n, k = C.c_void_p(), C.c_size_t(), C.c_uint32()
         check(_lib.load().bz_prefill_plan_host_schedule(self._h, C.byref(data), C.byref(n), C.byref(k)),
               "Handler schedule")
         if n.value == 0:
-            return np.zeros((0, 4), np.int32)
+            return np.zeros((0, 8), np.int32)
         buf = (C.c_int32 * (n.value * k.value)).from_address(data.value)
         return np.frombuffer(buf, np.int32).reshape(n.value, k.value).copy()
 

@@ -217,9 +217,11 @@ int bz_prefill_plan(bz_prefill_plan_t* plan, void* float_buffer, size_t float_bu
                     uint32_t page_size, void* stream);
 
 /* Host-only counterparts of bz_decode_plan_workspace / bz_decode_plan_host_schedule for the prefill plan:
- * the bytes of int_buffer the job list of this batch takes (the float workspace is not used), and the
- * host copy of the list, one record per workgroup in launch order {first token of the request, tokens of
- * the request (0 = padding entry), first q row of the tile inside the request, q head}.  No GPU call. */
+ * the bytes of int_buffer the job list of this batch takes and the bytes of float_buffer that hold the angle
+ * table of the in-register q rotation (512 per position of the longest request; optional, see
+ * bz_batch_prefill_ragged), and the host copy of the list, one record of 8 ints per workgroup in launch order
+ * {first q row of the request, q rows of the request (0 = padding entry), first q row of the tile inside the
+ * request, q head, first K/V row of the request, K/V rows of the request, 0, 0}.  No GPU call. */
 int bz_prefill_plan_workspace(bz_prefill_plan_t* plan, const int32_t* qo_indptr_h, const int32_t* kv_indptr_h,
                               uint32_t batch_size, uint32_t num_qo_heads, uint32_t num_kv_heads, uint32_t head_dim,
                               size_t* float_buffer_bytes, size_t* int_buffer_bytes);
@@ -238,9 +240,12 @@ int bz_prefill_plan_set_bf16_mode(bz_prefill_plan_t* plan, int mode);
 
 /*
  * batch_prefill_attention (src/kernel/attention.h:9-22, attention_prefill.cu:11-46): ragged
- * self-attention, q [N,Hq,D], k,v [N,Hkv,D], out [N,Hq,D], qo_indptr == kv_indptr (the only
- * way the reference calls it, src/layer/attn.h:175-187).  causal != 0 masks j > i.
- * rope_mode BZ_ROPE_NONE: q, k used as they are.  BZ_ROPE_Q_ONLY: q rows are rotated by their offset inside
+ * attention, q [Nq,Hq,D], k,v [Nkv,Hkv,D], out [Nq,Hq,D].  The reference passes one array as qo_indptr and
+ * kv_indptr (src/layer/attn.h:175-187): self-attention over each request.  With two arrays request b has
+ * q rows for its LAST qo_len_b tokens only and K/V rows for all kv_len_b >= qo_len_b of them (a chunk of a
+ * prompt attending to the whole prefix): q row i sits at position kv_len_b - qo_len_b + i.  causal != 0 masks
+ * the K/V rows behind a q row's position.  The device arrays must hold what the plan was made from.
+ * rope_mode BZ_ROPE_NONE: q, k used as they are.  BZ_ROPE_Q_ONLY: q rows are rotated by their position inside
  * the request in registers (q in memory stays as it is), k is expected rotated (bz_store_prefill_kv with
  * rope = 2 leaves it so).  BZ_ROPE_FULL, the reference's kRoPELlama: q as for BZ_ROPE_Q_ONLY, and the k rows
  * are rotated IN PLACE first (the caller's k buffer then holds rotated K for the page store that follows,

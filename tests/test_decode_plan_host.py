@@ -198,8 +198,10 @@ def test_prefill_job_list_invariants(lens, Hq, Hkv):
     h = K.BatchPrefillRaggedHandler()
     fb, ib = h.workspace(indptr, indptr, len(lens), Hq, Hkv, 128)
     items = h.host_schedule()
+    assert items.shape[1] == 8 and np.array_equal(items[:, 4:6], items[:, 0:2]) and not items[:, 6:].any()  # K/V range = q range here
+    items = items[:, :4]
     # float workspace: the angle table of the q rotation, 512 bytes per position of the longest request
-    assert fb == 512 * max(lens) and ib == (len(items) * 16 + 255) // 256 * 256 and len(items) % 8 == 0
+    assert fb == 512 * max(lens) and ib == (len(items) * 32 + 255) // 256 * 256 and len(items) % 8 == 0
     tok0_to_req = {int(indptr[b]): b for b in range(len(lens)) if lens[b] > 0}
     seen, column, last_q0 = set(), {}, {}
     first_seen_len = []

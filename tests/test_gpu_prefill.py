@@ -281,6 +281,77 @@ def test_c4_rope_store_then_attention_at_full_size():
     assert np.abs(got[rows] - ref_raw).max() <= 3e-3, float(np.abs(got[rows] - ref_raw).max())
 
 
+@pytest.mark.parametrize("kind", KINDS, ids=KIND_IDS)
+@pytest.mark.parametrize("causal", [True, False])
+@pytest.mark.parametrize("rope_mode,float_ws_bytes", [(BZ_ROPE_NONE, 1 << 20), (BZ_ROPE_Q_ONLY, 1 << 20), (BZ_ROPE_FULL, 1 << 20),
+                                                      (BZ_ROPE_FULL, 1 << 10)])
+def test_q_rows_for_the_last_tokens_of_a_request_only(kind, causal, rope_mode, float_ws_bytes):
+    """qo_indptr != kv_indptr (src/kernel/attention.h:9-22 carries both): every request brings K/V rows for all its
+    tokens and q rows for the last ones only -- a chunk of a prompt attending to the whole prefix.  q row i sits at
+    position kv_len - qo_len + i.  The result must be the rows of plain self-attention over the whole request that
+    belong to those tokens, which is what the checker computes (the other q rows of its input are never looked at)."""
+    dtype, theta, Hq, Hkv, D = kind[0], 1e4, 8, 2, 128
+    kv_lens = np.array([300, 64, 129, 1000, 33, 5, 200, 257])
+    q_lens = np.array([100, 64, 1, 37, 32, 5, 0, 130])  # offsets 200, 0, 128, 963 (not a multiple of a tile), 1, 0, -, 127
+    kv_indptr = np.concatenate([[0], np.cumsum(kv_lens)]).astype(np.int32)
+    qo_indptr = np.concatenate([[0], np.cumsum(q_lens)]).astype(np.int32)
+    rng = np.random.default_rng(260)
+    Nkv, Nq, B = int(kv_indptr[-1]), int(qo_indptr[-1]), len(kv_lens)
+    q_full = wl.randn_bits(rng, (Nkv, Hq, D), dtype)
+    k = wl.randn_bits(rng, (Nkv, Hkv, D), dtype)
+    v = wl.randn_bits(rng, (Nkv, Hkv, D), dtype)
+    rows = np.concatenate([np.arange(kv_indptr[b + 1] - q_lens[b], kv_indptr[b + 1]) for b in range(B)]).astype(np.int32)
+    q = q_full[rows]
+    k_rot = oracle.rope_ragged(k, dtype, kv_indptr, Hkv, D, theta)
+    k_in = k_rot if rope_mode == BZ_ROPE_Q_ONLY else k
+    float_ws = torch.empty(float_ws_bytes, dtype=torch.uint8, device="cuda")
+    int_ws = torch.empty(1 << 20, dtype=torch.uint8, device="cuda")
+    handler = K.BatchPrefillRaggedHandler()
+    if kind[1] is not None:
+        handler.set_bf16_mode(kind[1])
+    fb, ib = handler.workspace(qo_indptr, kv_indptr, B, Hq, Hkv, D)
+    assert fb == 512 * 1000 and ib <= int_ws.numel()
+    handler.plan(float_ws, float_ws.numel(), int_ws, int_ws.numel(), qo_indptr, kv_indptr, B, Hq, Hkv, D, 16)
+    qd, kd, vd = to_dev(q, dtype), to_dev(k_in, dtype), to_dev(v, dtype)
+    out = torch.full_like(qd, float("nan"))
+    K.batch_prefill_attention(handler, qd, torch.from_numpy(qo_indptr).cuda(), kd, vd, torch.from_numpy(kv_indptr).cuda(), out,
+                              B, Hq, Hkv, D, causal=causal, rope_mode=rope_mode, rope_theta=theta)
+    torch.cuda.synchronize()
+    got = wl.to_f32(to_host_bits(out), dtype)
+    assert not np.isnan(got).any()
+    assert np.array_equal(to_host_bits(vd), v)
+    k_after = to_host_bits(kd)
+    step = 2.0 ** -8 if dtype == BZ_F16 else 2.0 ** -5
+    if rope_mode == BZ_ROPE_FULL:  # K rotated in place, every row at its own index
+        assert np.abs(wl.to_f32(k_after, dtype) - wl.to_f32(k_rot, dtype)).max() <= step and (k_after != k_rot).mean() < 2e-3
+    else:
+        assert np.array_equal(k_after, k_in)
+    table_fits = float_ws_bytes >= 512 * 1000
+    if rope_mode == BZ_ROPE_NONE:
+        assert np.array_equal(to_host_bits(qd), q)
+        ref = oracle.batch_prefill_ragged(q_full, k, v, dtype, kv_indptr, Hq, Hkv, D, causal=causal, rows=rows, parallel=True)
+    elif table_fits:
+        assert np.array_equal(to_host_bits(qd), q)  # rotated in registers
+        q_fed = prefill_q_as_fed(q_full, dtype, kv_indptr, Hq, D, theta, prefill_angle_table(float_ws, 1000, D))
+        ref = oracle.batch_prefill_ragged(q_fed, k_after, v, dtype, kv_indptr, Hq, Hkv, D, causal=causal, sm_scale=LN2,
+                                          rows=rows, parallel=True)
+    else:  # no room for the table: q rotated in place, at the positions of its tokens
+        q_rot = oracle.rope_ragged(q_full, dtype, kv_indptr, Hq, D, theta)[rows]
+        q_after = to_host_bits(qd)
+        assert np.abs(wl.to_f32(q_after, dtype) - wl.to_f32(q_rot, dtype)).max() <= step and (q_after != q_rot).mean() < 2e-3
+        q_full_after = q_full.copy()
+        q_full_after[rows] = q_after
+        ref = oracle.batch_prefill_ragged(q_full_after, k_after, v, dtype, kv_indptr, Hq, Hkv, D, causal=causal, rows=rows,
+                                          parallel=True)
+    assert (np.abs(got - ref) <= kind_tol(ref, kind)).all(), np.abs(got - ref).max()
+
+
+def test_fewer_kv_rows_than_q_rows_is_refused():
+    h = K.BatchPrefillRaggedHandler()
+    with pytest.raises(K.BzError, match="Handler workspace"):
+        h.workspace(np.array([0, 10], np.int32), np.array([0, 9], np.int32), 1, 4, 4, 128)
+
+
 def test_prefill_error_codes():
     pf = Prefill(230, [5], 4, 4, 128, BZ_F16)
     qd = to_dev(pf.q, BZ_F16)
