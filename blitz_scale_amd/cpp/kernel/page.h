@@ -135,6 +135,17 @@ void append_decode_kv_cache(PageTable<DType, IdType>& page_table, SrcType* k_dat
              "AppendPagedKVCacheDecode");
 }
 
+/// The cached K rows of every sequence of the table rotated in place at their positions (inverse: the rotation
+/// taken off again): converts a cache that holds K as the projection left it -- the reference's convention, under
+/// which attention_decode.cu:35 rotates every cached row at every step -- to the rotated-K cache the decode calls
+/// here expect, once, at the speed of a copy.  No counterpart in the reference.
+template<typename DType, typename IdType>
+void rope_cached_k(PageTable<DType, IdType>& page_table, bool inverse = false, const AttentionOptions* options = nullptr) {
+    const AttentionOptions& o = options ? *options : page_table.opts();
+    const bz_paged_kv_t kv = page_table.c_view();
+    bz_throw(bz_rope_cached_k(&kv, o.rope_theta, inverse ? 1 : 0, o.stream), "ropeCachedK");
+}
+
 /// declared and never defined in the reference (src/kernel/page.h:72-73); here it is the token count
 template<typename DType, typename IdType>
 uint32_t cal_total_num_rows(const PageTable<DType, IdType>& page_table) {

@@ -343,6 +343,69 @@ static int fill_args(PageWriteArgs& a, const bz_paged_kv_t* kv, const void* k, c
     return 0;
 }
 
+// ---- one pass over the cached K rows of a page table: rotate them in place at their positions (direction +1) or
+// take the rotation off again (direction -1).  A cache that arrives with K as the projection left it -- the
+// reference's convention, whose decode call rotates every cached row at every step (attention_decode.cu:35) -- is
+// brought to this library's convention (K cached rotated, the decode kernels rotate q only) once, at the speed of
+// a copy, instead of paying for the rotation at every step; a cache that leaves for such a consumer is taken back.
+// Workgroup (b, c) takes pages c, c + gridDim.y, ... of sequence b: the angles of a page's slots go through LDS
+// (they are shared by the kv heads), eight lanes per row as in the page writes.
+struct RopeCachedArgs {
+    char* k_data;
+    const int32_t* indices;
+    const int32_t* indptr;
+    const int32_t* last_page_len;
+    uint64_t stride_page, stride_n, stride_h;
+    uint32_t page_size, num_kv_heads;
+    float direction;
+    RopeFreqs freqs;
+};
+
+template <typename PT, int D>
+__global__ __launch_bounds__(256) void rope_cached_k_kernel(RopeCachedArgs a) {
+    extern __shared__ float2 s_cs[]; // [slot][pair]
+    constexpr int LANES = D / 16;
+    const int b = blockIdx.x;
+    const int ip0 = a.indptr[b], np = a.indptr[b + 1] - ip0;
+    if (np <= 0) return;
+    const int P = (int)a.page_size, Hkv = (int)a.num_kv_heads;
+    const int lane = threadIdx.x % LANES;
+    for (int pg = blockIdx.y; pg < np; pg += gridDim.y) {
+        const int slots = pg + 1 < np ? P : min(max(a.last_page_len[b], 0), P);
+        const int64_t page = a.indices[ip0 + pg];
+        __syncthreads(); // the previous page's angles are no longer read
+        for (int i = threadIdx.x; i < slots * (D / 2); i += 256) {
+            float sn, cs;
+            sincosf((float)(pg * P + i / (D / 2)) * a.freqs.f[i % (D / 2)], &sn, &cs);
+            s_cs[i] = make_float2(cs, a.direction * sn);
+        }
+        __syncthreads();
+        for (int r = threadIdx.x / LANES; r < slots * Hkv; r += 256 / LANES) {
+            const int slot = r / Hkv, h = r % Hkv;
+            PT* row = reinterpret_cast<PT*>(a.k_data) +
+                      ((size_t)page * a.stride_page + (size_t)slot * a.stride_n + (size_t)h * a.stride_h);
+            Vec8<PT> lo, hi;
+            lo.load(row + lane * 8);
+            hi.load(row + D / 2 + lane * 8);
+            float x[8], y[8];
+            lo.to_float(x);
+            hi.to_float(y);
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                const float2 cs = s_cs[slot * (D / 2) + lane * 8 + e];
+                float xr, yr;
+                rope_pair(x[e], y[e], cs.x, cs.y, xr, yr);
+                x[e] = xr;
+                y[e] = yr;
+            }
+            lo.from_float(x);
+            hi.from_float(y);
+            lo.store(row + lane * 8);
+            hi.store(row + D / 2 + lane * 8);
+        }
+    }
+}
+
 __global__ void steps_ahead_advance_kernel(int32_t* steps_ahead) {
     const int32_t v = *steps_ahead;
     if (v > 0) *steps_ahead = v - 1;
@@ -385,6 +448,35 @@ extern "C" int bz_append_decode_kv(const bz_paged_kv_t* kv, const void* k, const
     if (rc) return rc;
     return launch_page_write<false>(a, src_dtype, kv->kv_dtype, (int)kv->head_dim, kv->batch_size,
                                     (hipStream_t)stream);
+}
+
+extern "C" int bz_rope_cached_k(const bz_paged_kv_t* kv, float rope_theta, int inverse, void* stream) {
+    if (!kv || !kv->k_data || !kv->indices || !kv->indptr || !kv->last_page_len) return BZ_ERR_BAD_ARG;
+    if (kv->stride_n % 8 || kv->stride_h % 8 || kv->stride_page % 8 || kv->page_size == 0) return BZ_ERR_BAD_ARG;
+    if (kv->kv_dtype != BZ_F16 && kv->kv_dtype != BZ_BF16) return BZ_ERR_UNSUPPORTED; // (e4m3 rows would be requantised)
+    const int D = (int)kv->head_dim;
+    if (D != 128 && D != 64) return BZ_ERR_UNSUPPORTED;
+    const size_t lds = (size_t)kv->page_size * (D / 2) * sizeof(float2);
+    if (lds > 64 * 1024) return BZ_ERR_UNSUPPORTED; // page_size <= 128 (head_dim 128) / 256 (head_dim 64)
+    if (kv->batch_size == 0) return 0;
+    RopeCachedArgs a;
+    a.k_data = (char*)kv->k_data;
+    a.indices = kv->indices; a.indptr = kv->indptr; a.last_page_len = kv->last_page_len;
+    a.stride_page = kv->stride_page; a.stride_n = kv->stride_n; a.stride_h = kv->stride_h;
+    a.page_size = kv->page_size; a.num_kv_heads = kv->num_kv_heads;
+    a.direction = inverse ? -1.0f : 1.0f;
+    a.freqs = make_rope_freqs(D, rope_theta > 0.f ? rope_theta : 1e4f);
+    const dim3 grid(kv->batch_size, 32);
+    hipStream_t s = (hipStream_t)stream;
+    if (kv->kv_dtype == BZ_F16) {
+        if (D == 128) hipLaunchKernelGGL((rope_cached_k_kernel<f16_t, 128>), grid, dim3(256), lds, s, a);
+        else hipLaunchKernelGGL((rope_cached_k_kernel<f16_t, 64>), grid, dim3(256), lds, s, a);
+    } else {
+        if (D == 128) hipLaunchKernelGGL((rope_cached_k_kernel<bf16_t, 128>), grid, dim3(256), lds, s, a);
+        else hipLaunchKernelGGL((rope_cached_k_kernel<bf16_t, 64>), grid, dim3(256), lds, s, a);
+    }
+    BZ_LAUNCH_CHECK();
+    return 0;
 }
 
 // ---- pool helpers -----------------------------------------------------------------------------

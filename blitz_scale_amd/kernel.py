@@ -296,6 +296,14 @@ def append_decode_kv_cache(page_table, k_data, v_data, *, q=None, num_qo_heads=0
     check(rc, "AppendPagedKVCacheDecode")
 
 
+def rope_cached_k(page_table, *, rope_theta=1e4, inverse=False, stream=None):
+    """Rotate (or un-rotate) the cached K rows of every sequence of the table in place: a cache filled under the
+    reference's raw-K convention (kRoPELlama at every decode call, src/kernel/attention_decode.cu:35) converted once
+    to the rotated-K convention of the fast decode path, or back.  No counterpart in the reference."""
+    s = page_table.as_struct()
+    check(_lib.load().bz_rope_cached_k(C.byref(s), rope_theta, int(inverse), _stream(stream)), "ropeCachedK")
+
+
 def steps_ahead_advance(steps_ahead, *, stream=None):
     """End of a decode step under a page table that runs ahead of the present: counter -= 1, not below 0."""
     check(_lib.load().bz_steps_ahead_advance(_ptr(steps_ahead), _stream(stream)), "stepsAheadAdvance")

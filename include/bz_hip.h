@@ -289,6 +289,16 @@ int bz_append_decode_kv(const bz_paged_kv_t* kv, const void* k, const void* v, i
  * by one, not below zero.  One tiny launch on `stream`, recordable into a HIP graph. */
 int bz_steps_ahead_advance(int32_t* steps_ahead, void* stream);
 
+/* Rotate (inverse == 0) or un-rotate (inverse != 0) the cached K rows of every sequence of the table in place, row t
+ * of a sequence at position t: one pass at the speed of a copy.  The reference caches K as the projection left
+ * it and rotates every cached row inside every decode call (kRoPELlama, src/kernel/attention_decode.cu:35); this
+ * library caches K rotated and rotates q only.  A cache filled under the reference's convention (e.g. pages received
+ * from a reference instance) is converted once with this call and then served by the fast decode path
+ * (BZ_ROPE_Q_ONLY); inverse takes a cache back before it leaves for such a consumer.  Forward then inverse restores
+ * the rows to within one rounding of the storage type.  f16 / bf16 pools, head_dim 64 or 128, page_size <= 128
+ * (head_dim 128).  BZ_ROPE_FULL of bz_batch_decode remains for caches that must stay raw. */
+int bz_rope_cached_k(const bz_paged_kv_t* kv, float rope_theta, int inverse, void* stream);
+
 /* ---------------------------------------------------------------------------------------
  * element-wise kernels of src/layer's call sites
  * ------------------------------------------------------------------------------------- */

@@ -235,3 +235,47 @@ def test_store_prefill_rotates_k_in_place_without_q():
                                                                indices=p.indices, indptr=p.indptr, stride_page=p.stride_page,
                                                                stride_n=p.stride_n, stride_h=p.stride_h))())(2)
     assert np.array_equal(K0, wl.to_f32(got_k, dtype).reshape(-1, Hkv, D)[ri[2]:ri[3]])
+
+
+@pytest.mark.parametrize("dtype,D,P,layout", [(BZ_F16, 128, 16, BZ_LAYOUT_HND), (BZ_BF16, 128, 64, BZ_LAYOUT_NHD),
+                                              (BZ_F16, 64, 8, BZ_LAYOUT_HND)])
+def test_raw_k_cache_converted_once_then_served_by_the_fast_decode_path(dtype, D, P, layout):
+    """A cache that holds K as the projection left it (the reference's convention: kRoPELlama inside every decode
+    call, src/kernel/attention_decode.cu:35) is rotated in place once; decode with BZ_ROPE_Q_ONLY over it then gives
+    the checker's kRoPELlama result on the raw cache.  V, the unused slots and the pages of no sequence are not
+    touched; the inverse pass restores the raw rows to within one rounding."""
+    from blitz_scale_amd._lib import BZ_F32, BZ_ROPE_FULL, BZ_ROPE_Q_ONLY
+    theta = 5e5
+    p = DecodeProblem(70, [1, 17, 300, 0, 2049, 64, 1000], 8, 2, D, P, dtype, layout=layout)
+    ref = oracle.batch_decode(p.q, p.dtype, p.oracle_kv(), p.Hq, rope_mode=oracle.ROPE_FULL, rope_theta=theta, parallel=True)
+    dev = DeviceDecode(p)
+    dev.plan(1024)
+    K.rope_cached_k(dev.pt, rope_theta=theta)
+    torch.cuda.synchronize()
+    pool_rot = to_host_bits(dev.pool)
+    # the checker's rotation of the same rows: gather every sequence's K, rotate, compare where the pool changed
+    want = p.pool.copy()
+    k_rows = np.zeros(p.pool.size, bool)  # the elements of cached K rows: everything else must stay as it is
+    for b in range(p.B):
+        n = int(p.ctx[b])
+        if n == 0:
+            continue
+        Kb, _ = p.gather_kv(b)  # fp32 [n, Hkv, D]
+        rot = oracle.rope_ragged(wl.to_bits(Kb, dtype), dtype, np.array([0, n], np.int32), p.Hkv, D, theta)
+        for t in range(n):
+            page = int(p.indices[p.indptr[b] + t // P])
+            for h in range(p.Hkv):
+                off = page * p.stride_page + (t % P) * p.stride_n + h * p.stride_h
+                want[off:off + D] = rot[t, h]
+                k_rows[off:off + D] = True
+    assert np.abs(wl.to_f32(pool_rot, dtype) - wl.to_f32(want, dtype)).max() <= (2.0 ** -8 if dtype == BZ_F16 else 2.0 ** -5)
+    assert (pool_rot != want).mean() < 2e-3
+    assert np.array_equal(pool_rot[~k_rows], p.pool[~k_rows])  # V halves, unused slots, pages of no sequence
+    got = dev.decode(BZ_F32, BZ_ROPE_Q_ONLY, theta)
+    assert np.abs(got - ref).max() <= 2e-3, float(np.abs(got - ref).max())
+    K.rope_cached_k(dev.pt, rope_theta=theta, inverse=True)
+    torch.cuda.synchronize()
+    back = to_host_bits(dev.pool)
+    step = np.maximum(np.abs(wl.to_f32(p.pool, dtype)), 1.0) * (2.0 ** -9 if dtype == BZ_F16 else 2.0 ** -6)
+    assert (np.abs(wl.to_f32(back, dtype) - wl.to_f32(p.pool, dtype)) <= step).all()
+    assert np.array_equal(back[~k_rows], p.pool[~k_rows])
