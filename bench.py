@@ -33,7 +33,7 @@ def parse():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=None)
     ap.add_argument("--warmup", type=int, default=None)
-    ap.add_argument("--workload", default="C3", choices=["C2", "C3", "C4", "C5", "ENDS", "MIGRATE", "LAYERS"])
+    ap.add_argument("--workload", default="C3", choices=["C2", "C3", "C4", "C5", "ENDS", "MIGRATE", "LAYERS", "RAWK"])
     ap.add_argument("--layers", type=int, default=None, help="layer planes of the KV pool the steps cycle over")
     ap.add_argument("--seed", type=lambda s: int(s, 0), default=0x5EED)
     ap.add_argument("--sigma", type=float, default=1.0, help="sigma of the log-normal context lengths (C3)")
@@ -787,6 +787,98 @@ def bench_layers(args):
                          "kernel": "whole replayed step (launch-latency bound at this size, not a kernel figure)"}}
 
 
+def bench_rawk(args):
+    """A cache that holds K as the projection left it (the reference's convention, kRoPELlama inside every decode
+    call, src/kernel/attention_decode.cu:35): 128 sequences of 1024 tokens, Llama-3-8B heads, bf16.  Three figures:
+    the decode call that rotates every cached K row itself (BZ_ROPE_FULL), the one pass that converts the cache to
+    the rotated-K convention (bz_rope_cached_k), and the decode call over the converted cache (BZ_ROPE_Q_ONLY)."""
+    import numpy as np
+    import torch
+
+    import oracle
+    from blitz_scale_amd import kernel as K, workloads as wl
+    from blitz_scale_amd._lib import BZ_LAYOUT_HND, BZ_ROPE_FULL, BZ_ROPE_Q_ONLY
+
+    B, Hq, Hkv, D, P, ctx_len, theta = 128, 32, 8, 128, 16, 1024, 5e5
+    rng = np.random.default_rng(args.seed)
+    ctx = np.full(B, ctx_len)
+    pool_pages = B * ctx_len // P
+    indices, indptr, lpl = wl.page_table_for(ctx, P, pool_pages, rng)
+    stride_page, sn, sh = wl.strides(BZ_LAYOUT_HND, Hkv, P, D)
+    g = torch.Generator(device="cuda")
+    g.manual_seed(args.seed)
+    L = 4  # planes cycled so that no call finds its K/V in a cache
+    pool = torch.randn(L * pool_pages * stride_page, dtype=torch.bfloat16, device="cuda", generator=g)
+    raw0 = pool[:pool_pages * stride_page].clone()
+    q = torch.randn((B, Hq, D), dtype=torch.bfloat16, device="cuda", generator=g)
+    out = torch.empty((B, Hq, D), dtype=torch.float32, device="cuda")
+    pt = K.PageTable(B, P, Hkv, D, pool, layout=BZ_LAYOUT_HND)
+    pt.indices, pt.indptr, pt.last_page_len = indices, indptr, lpl
+    pt.upload()
+    float_ws = torch.empty(128 << 20, dtype=torch.uint8, device="cuda")
+    int_ws = torch.empty(8 << 20, dtype=torch.uint8, device="cuda")
+    handler = K.BlitzBatchDecodeHandler()
+    handler.plan(float_ws, float_ws.numel(), int_ws, int_ws.numel(), indptr, lpl, B, Hq, Hkv, D, P)
+    steps = args.steps or 40
+    warmup = args.warmup if args.warmup is not None else 8
+    kv_bytes = float(B * ctx_len * Hkv * D * 2 * 2)
+
+    def run(fn):
+        def step(i, e):
+            pt.set_layer(i % L, pool_pages)
+            if e is not None:
+                e[0].record()
+            fn()
+            if e is not None:
+                e[1].record()
+        _, ev = timed(step, steps, warmup)
+        return ev
+
+    full = run(lambda: K.batch_decode_attention(handler, q, pt, out, Hq, rope_mode=BZ_ROPE_FULL, rope_theta=theta))
+    pt.set_layer(0, pool_pages)
+    K.batch_decode_attention(handler, q, pt, out, Hq, rope_mode=BZ_ROPE_FULL, rope_theta=theta)
+    torch.cuda.synchronize()
+    out_full = out.clone()
+    # (a rotation keeps the magnitude of a row, so the pass can be timed over and over on the same planes)
+    conv = run(lambda: K.rope_cached_k(pt, rope_theta=theta))
+    pool[:pool_pages * stride_page].copy_(raw0)
+    pt.set_layer(0, pool_pages)
+    K.rope_cached_k(pt, rope_theta=theta)  # plane 0: the raw cache, converted once (the other planes only feed the timing)
+    q_only = run(lambda: K.batch_decode_attention(handler, q, pt, out, Hq, rope_mode=BZ_ROPE_Q_ONLY, rope_theta=theta))
+    pt.set_layer(0, pool_pages)
+    K.batch_decode_attention(handler, q, pt, out, Hq, rope_mode=BZ_ROPE_Q_ONLY, rope_theta=theta)
+    torch.cuda.synchronize()
+    res = {"metric": "raw_k_cache_decode_us_per_call", "value": pct(full)["mean"], "unit": "us/call", "n_gpus": 1, "steps": steps,
+           "warmup": warmup, "ms_per_step": round(float(full.mean()), 6), "higher_is_better": False, "scaling": "weak",
+           "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+           "config": {"workload": "RAWK: decode over a cache with K as projected (the reference's kRoPELlama convention), "
+                                  "128 sequences x 1024 tokens, 32/8 heads, head_dim 128, page 16"},
+           "decode_rope_full_us": pct(full), "convert_cache_once_us": pct(conv), "decode_q_only_after_conversion_us": pct(q_only),
+           "GB_per_s": {"decode_rope_full": round(kv_bytes / float(full.mean()) / 1e6, 1),
+                        "convert_cache_once (K read + written)": round(kv_bytes / float(conv.mean()) / 1e6, 1),
+                        "decode_q_only_after_conversion": round(kv_bytes / float(q_only.mean()) / 1e6, 1)},
+           "max_abs_diff_between_the_two_routes": float((out - out_full).abs().max()),
+           "roofline": {"bound": "hbm", "achieved": round(kv_bytes / float(full.mean()) / 1e6, 1), "peak": HBM_PEAK_GBPS,
+                        "unit": "GB/s", "frac": round(kv_bytes / float(full.mean()) / 1e6 / HBM_PEAK_GBPS, 4), "traffic": None,
+                        "kernel": "bz_batch_decode with BZ_ROPE_FULL (general kernel, angles from a table); K and V bytes of "
+                                  "the batch over the call's duration (torch events)"}}
+    if not args.no_cpu_baseline:
+        sb = 16
+        plane0 = raw0.view(torch.int16).cpu().numpy().view(np.uint16)
+        kv = oracle.PagedKV(plane0, plane0[stride_page // 2:], indices[:int(indptr[sb])], indptr[:sb + 1], lpl[:sb], P, Hkv, D,
+                            stride_page, sn, sh, oracle.BF16)
+        qh = q.view(torch.int16).cpu().numpy().view(np.uint16)
+        t0 = time.perf_counter()
+        ref = oracle.batch_decode(qh[:sb], oracle.BF16, kv, Hq, rope_mode=oracle.ROPE_FULL, rope_theta=theta, parallel=True)
+        cpu_s = time.perf_counter() - t0
+        res["max_abs_err_vs_cpu"] = {"decode_rope_full": float(np.abs(out_full[:sb].cpu().numpy() - ref).max()),
+                                     "convert_then_q_only": float(np.abs(out[:sb].cpu().numpy() - ref).max())}
+        res["cpu_baseline"] = {"value": round(cpu_s * B / sb * 1e6, 1), "unit": "us/call", "cores": oracle.num_threads(True),
+                               "kind": "port", "sample": f"kRoPELlama decode of the first {sb} of {B} sequences, scaled by {B // sb}x",
+                               "host_cpus": os.cpu_count()}
+    return res
+
+
 def main():
     args = parse()
     import torch
@@ -806,6 +898,8 @@ def main():
         res = bench_migrate(args)
     elif args.workload == "LAYERS":
         res = bench_layers(args)
+    elif args.workload == "RAWK":
+        res = bench_rawk(args)
     else:
         res = bench_prefill(args) if args.workload == "C4" else bench_decode(args, args.workload)
     print(json.dumps(res))
