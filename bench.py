@@ -33,7 +33,7 @@ def parse():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=None)
     ap.add_argument("--warmup", type=int, default=None)
-    ap.add_argument("--workload", default="C3", choices=["C2", "C3", "C4", "C5", "ENDS", "MIGRATE", "LAYERS", "RAWK"])
+    ap.add_argument("--workload", default="C3", choices=["C2", "C3", "C4", "C5", "ENDS", "MIGRATE", "LAYERS", "RAWK", "MFMA_CEILING"])
     ap.add_argument("--layers", type=int, default=None, help="layer planes of the KV pool the steps cycle over")
     ap.add_argument("--seed", type=lambda s: int(s, 0), default=0x5EED)
     ap.add_argument("--sigma", type=float, default=1.0, help="sigma of the log-normal context lengths (C3)")
@@ -879,8 +879,43 @@ def bench_rawk(args):
     return res
 
 
+def bench_mfma_ceiling(args):
+    """What the matrix pipes sustain on this GPU without any memory traffic (blitz_scale_amd/probes/mfma_ceiling.hip,
+    a stand-alone program run here as a child process): the yardstick beside the data sheet's 2.5 PFLOP/s for the
+    prefill kernel's figure."""
+    import re
+    import subprocess
+    exe = os.path.join(ROOT, "blitz_scale_amd", "probes", "mfma_ceiling")
+    if not os.path.exists(exe):
+        sys.exit("bench.py: blitz_scale_amd/probes/mfma_ceiling is not built (python -c 'import __graft_entry__ as g; g.build()')")
+    t0 = time.perf_counter()
+    out = subprocess.run([exe], capture_output=True, text=True, timeout=600)
+    if out.returncode != 0:
+        sys.exit("bench.py: the probe failed:\n" + out.stdout + out.stderr)
+    rows = {}
+    for line in out.stdout.splitlines():
+        m = re.match(r"(.*?)\s+([\d.]+) ms\s+([\d.]+) TFLOP/s\s+clock (\d+) MHz\s+pipe use (\d+) %", line)
+        if m:  # the program runs every variant twice: the second pass is the settled one
+            rows[m.group(1).strip()] = {"TFLOP_per_s": float(m.group(3)), "clock_MHz": int(m.group(4)),
+                                        "pipe_use_at_that_clock_pct": int(m.group(5))}
+    key = "+ LDS every instruction + exp, pack, dot2"
+    return {"metric": "mfma_ceiling_tflops", "value": rows[key]["TFLOP_per_s"], "unit": "TFLOP/s", "n_gpus": 1, "steps": 1,
+            "warmup": 1, "ms_per_step": round((time.perf_counter() - t0) * 1e3, 1), "higher_is_better": True, "scaling": "weak",
+            "vs_baseline": None, "dtype": "f16", "data": "synthetic",
+            "config": {"workload": "MFMA_CEILING: v_mfma_f32_32x32x16_f16 at full rate, 2 waves per SIMD on all 256 CUs, no "
+                                   "memory traffic; variants add what attention needs beside each matrix instruction"},
+            "variants": rows,
+            "roofline": {"bound": "mfma", "achieved": rows[key]["TFLOP_per_s"], "peak": MFMA_PEAK_TFLOPS, "unit": "TFLOP/s",
+                         "frac": round(rows[key]["TFLOP_per_s"] / MFMA_PEAK_TFLOPS, 4), "traffic": None,
+                         "kernel": "probe loop with one LDS operand read, one exponential, half a pack and half a row-sum "
+                                   "instruction per matrix instruction (`value`); the other variants are in `variants`"}}
+
+
 def main():
     args = parse()
+    if args.workload == "MFMA_CEILING":  # (a child process does the GPU work: nothing here touches the GPU before it)
+        print(json.dumps(bench_mfma_ceiling(args)))
+        return
     import torch
     from blitz_scale_amd import _lib
     _lib.load()  # fails loudly if the HIP library is not built

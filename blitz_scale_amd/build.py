@@ -68,6 +68,22 @@ def build(verbose=True, jobs=8):
     return LIB_PATH
 
 
+PROBE_SRC = os.path.join(HERE, "probes", "mfma_ceiling.hip")
+PROBE_BIN = os.path.join(HERE, "probes", "mfma_ceiling")
+
+
+def build_probes(verbose=True):
+    """The stand-alone measurement program behind `bench.py --workload MFMA_CEILING` (no part of the library)."""
+    cmd = [hipcc(), *[f for f in HIPCC_FLAGS if f != "-fPIC"], PROBE_SRC, "-o", PROBE_BIN]
+    if verbose:
+        print(" ".join(cmd), flush=True)
+    out = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    text = "\n".join(l for l in out.stdout.splitlines() if "packed-fp32-ops" not in l)
+    if out.returncode != 0:
+        raise RuntimeError("hipcc failed on the probe:\n" + text)
+    return PROBE_BIN
+
+
 def _drain(procs):
     failed = []
     for src, p in procs:
