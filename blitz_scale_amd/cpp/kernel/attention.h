@@ -7,10 +7,13 @@
 
 namespace blitz::kernel {
 
-/// src/kernel/attention.h:9-22.  Ragged causal self-attention over q [N,Hq,D], k,v [N,Hkv,D].
+/// src/kernel/attention.h:9-22.  Ragged causal attention over q [Nq,Hq,D], k,v [Nkv,Hkv,D]: self-attention when
+/// qo_indptr and kv_indptr are the same array (the reference's only use); with two arrays a request brings q rows
+/// for its last tokens only and K/V rows for all of them (what plan() was given must match).
 /// rope_mode < 0 takes handler.options.prefill_rope_mode, whose default BZ_ROPE_FULL is the reference's
-/// kRoPELlama (attention_prefill.cu:38): q and k rows are rotated by their offset inside the request, IN
-/// PLACE in the caller's buffers, before the contraction; k then holds what the cache must hold, and
+/// kRoPELlama (attention_prefill.cu:38): q rows are rotated by their position inside the request in registers (in
+/// place only when the float workspace has no room for the angle table), k rows IN PLACE in the caller's buffer,
+/// before the contraction; k then holds what the cache must hold, and
 /// store_prefill_kv_cache that follows (src/layer/attn.h:188-193) must not rotate it again (its default).
 /// BZ_ROPE_NONE: q and k are used as they are (they were rotated while the pages were written).
 template<typename DType, typename IdType>

@@ -1,6 +1,7 @@
-// Ragged (causal) prefill self-attention on the gfx950 matrix cores: replaces
+// Ragged (causal) prefill attention on the gfx950 matrix cores: replaces
 // src/kernel/attention_prefill.cu and the prefill half of flashinfer_types.cu of the BlitzScale
-// worker.  head_dim 128, f16 or bf16, any number of q heads per kv head.
+// worker.  head_dim 128, f16 or bf16, any number of q heads per kv head; self-attention over each request, or
+// q rows for the last tokens of a request only over K/V rows for all of them (distinct ragged indices).
 //
 // One workgroup of 4 waves takes 128 consecutive q rows of one (request, q head); wave w owns rows
 // 32w..32w+31.  K/V tiles of 32 tokens travel global -> LDS four tiles deep and are shared by the four
