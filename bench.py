@@ -54,6 +54,9 @@ def parse():
     ap.add_argument("--prefill-dtype", default="f16", choices=["f16", "bf16", "bf16-head-tail"],
                     help="C4: storage type of q, k, v and the output; bf16 runs the second product in f16 with V widened in "
                          "LDS, bf16-head-tail with the probabilities as two bf16 operands (any range of V)")
+    ap.add_argument("--prefill-lens", default=None,
+                    help="C4: comma-separated prompt lengths instead of the configuration's 16 x U[128, 4096] (diagnostic; "
+                         "the workload name says so)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also launch a few plain device copies of 1 GiB (reference point for rocprofv3 --pmc byte counters)")
     args = ap.parse_args()
@@ -422,6 +425,9 @@ def bench_prefill(args):
     B, Hq, Hkv, D, P, theta = cfg["batch"], cfg["Hq"], cfg["Hkv"], cfg["D"], cfg["P"], cfg["rope_theta"]
     rng = np.random.default_rng(args.seed)
     lens = wl.ctx_lens_for(cfg, rng)
+    if args.prefill_lens:
+        lens = np.array([int(x) for x in args.prefill_lens.split(",")], dtype=lens.dtype)
+        B = len(lens)
     indptr = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
     N = int(indptr[-1])
     # page table with the reference's len+1 reservation, seeded page placement
@@ -477,9 +483,11 @@ def bench_prefill(args):
         "metric": "ragged_causal_prefill_ms_per_step", "value": round(ms_per_step, 4), "unit": "ms/step",
         "n_gpus": 1, "steps": steps, "warmup": warmup, "ms_per_step": round(ms_per_step, 6),
         "higher_is_better": False, "scaling": "weak", "vs_baseline": None, "dtype": args.prefill_dtype, "data": "synthetic",
-        "config": {"workload": "C4: Llama-2-13B-shaped ragged causal prefill with RoPE + KV page store, one layer per step",
+        "config": {"workload": "C4: Llama-2-13B-shaped ragged causal prefill with RoPE + KV page store, one layer per step"
+                               if not args.prefill_lens else
+                               f"C4 heads and flow with prompt lengths {args.prefill_lens} (diagnostic, not the configuration's)",
                    "batch": B, "num_qo_heads": Hq, "num_kv_heads": Hkv, "head_dim": D, "page_size": P,
-                   "lens": "uniform[128,4096]", "tokens": N, "pool_pages": pool_pages, "rope_theta": theta,
+                   "lens": "uniform[128,4096]" if not args.prefill_lens else args.prefill_lens, "tokens": N, "pool_pages": pool_pages, "rope_theta": theta,
                    "q_rotated_by": args.q_rope,
                    "seed": hex(args.seed)},
         "tokens_per_s": round(N / (ms_per_step * 1e-3), 1),
