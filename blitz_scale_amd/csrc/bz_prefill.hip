@@ -369,12 +369,23 @@ __global__ __launch_bounds__(256, 2) void prefill_kernel(PrefillArgs a, const ch
         }
     }
     int copies = 0; // tile copies issued so far
+    if (L >= kSNK * kSN) {
+        // the common case: the first tiles all exist and are whole (kv_limit >= 128 as well, so n >= 4)
 #pragma unroll
-    for (int i = -kSNK; i < 0; ++i) {
-        if (i + kSNK < n) { issue_k(i + kSNK, i + kSNK); ++copies; }
-        if (i + kSNV - 1 >= 0 && i + kSNV - 1 < n) { issue_v(i + kSNV - 1, i + kSNV - 1); ++copies; }
+        for (int i = -kSNK; i < 0; ++i) {
+            issue_k_fast(i + kSNK, i + kSNK);
+            if (i + kSNV - 1 >= 0) issue_v_fast(i + kSNV - 1, i + kSNV - 1);
+        }
+        copies = kSNK + kSNV - 1;
+        sp_wait_copies(kSNK + kSNV - 1); // the q rows (and the angles) are here
+    } else {
+#pragma unroll
+        for (int i = -kSNK; i < 0; ++i) {
+            if (i + kSNK < n) { issue_k(i + kSNK, i + kSNK); ++copies; }
+            if (i + kSNV - 1 >= 0 && i + kSNV - 1 < n) { issue_v(i + kSNV - 1, i + kSNV - 1); ++copies; }
+        }
+        sp_wait_copies(copies);
     }
-    sp_wait_copies(copies); // the q rows (and the angles) are here
 #pragma unroll
     for (int ks = 0; ks < 8; ++ks) sp_loads_arrived(qreg[ks]);
     if constexpr (ROPE_Q) {
@@ -391,9 +402,10 @@ __global__ __launch_bounds__(256, 2) void prefill_kernel(PrefillArgs a, const ch
                 float x0, y0, x1, y1;
                 rope_pair(M::lo(xw), M::lo(yw), c0.x, c0.y, x0, y0);
                 rope_pair(M::hi(xw), M::hi(yw), c1.x, c1.y, x1, y1);
-                // (the softmax scale rides on the one rounding of the rotated row, see the kernel's header)
-                pf_u4(qreg[ks], w) = M::pack2(x0 * a.sm_scale_log2, x1 * a.sm_scale_log2);
-                pf_u4(qreg[ks + 4], w) = M::pack2(y0 * a.sm_scale_log2, y1 * a.sm_scale_log2);
+                // (the softmax scale rides on the one rounding of the rotated row, see the kernel's header: the
+                // table holds cos and sin times sm_scale * log2(e))
+                pf_u4(qreg[ks], w) = M::pack2(x0, x1);
+                pf_u4(qreg[ks + 4], w) = M::pack2(y0, y1);
             }
     }
 
@@ -791,14 +803,15 @@ __global__ __launch_bounds__(256) void rope_ragged_kernel(RopeRaggedArgs a) {
 }
 
 // cos / sin table for the q rotation inside the attention kernel: table[i / 2][pos] = (cos, sin) of pair i (even)
-// and of pair i + 1 at that position
-__global__ __launch_bounds__(256) void rope_table_kernel(float4* table, uint32_t positions, uint32_t pitch, RopeFreqs freqs) {
+// and of pair i + 1 at that position, each times `scale` (sm_scale * log2(e): the rotated rows come out scaled)
+__global__ __launch_bounds__(256) void rope_table_kernel(float4* table, uint32_t positions, uint32_t pitch, RopeFreqs freqs,
+                                                         float scale) {
     const uint32_t pos = blockIdx.x * 256 + threadIdx.x, i = 2 * blockIdx.y;
     if (pos >= positions) return;
     float s0, c0, s1, c1;
     sincosf((float)pos * freqs.f[i], &s0, &c0);
     sincosf((float)pos * freqs.f[i + 1], &s1, &c1);
-    table[(size_t)blockIdx.y * pitch + pos] = make_float4(c0, s0, c1, s1);
+    table[(size_t)blockIdx.y * pitch + pos] = make_float4(c0 * scale, s0 * scale, c1 * scale, s1 * scale);
 }
 
 static inline size_t pf_align_up(size_t x, size_t a) { return (x + a - 1) / a * a; }
@@ -1008,8 +1021,9 @@ extern "C" int bz_batch_prefill_ragged(bz_prefill_plan_t* plan_, void* q, const 
         if (p->rope_table) {
             // (every call: the workspace may be shared with other handlers between calls, calls may change streams,
             // and a captured call must replay its own fill; a few microseconds)
+            const float scale = (sm_scale > 0.f ? sm_scale : 1.0f / sqrtf((float)head_dim)) * 1.4426950408889634f;
             hipLaunchKernelGGL(rope_table_kernel, dim3((p->max_len + 255) / 256, 32), dim3(256), 0, s, (float4*)p->rope_table,
-                               p->max_len, p->max_len, freqs);
+                               p->max_len, p->max_len, freqs, scale);
             BZ_LAUNCH_CHECK();
         }
         auto rotate_rows = [&](void* rows, const int32_t* indptr, const int32_t* longer, uint32_t heads, uint32_t tokens) {

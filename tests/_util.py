@@ -109,30 +109,31 @@ def prefill_angle_table(float_ws, max_len, D=128):
 
 def prefill_q_as_fed(q_bits, dtype, indptr, Hq, D, theta, table, sm_scale=None):
     """The q rows as the prefill kernel feeds them to the matrix cores when it rotates them itself
-    (BZ_ROPE_Q_ONLY / BZ_ROPE_FULL): rotated at their offset inside the request with the angles of the device's own
-    table (`table`, from prefill_angle_table: the device's sincosf may differ from the host's in the last place, and
-    one such difference, rounded the other way and multiplied by logits of +-40, is visible in the output),
-    multiplied by sm_scale * log2(e) and rounded ONCE to the storage type -- every step an IEEE fp32 operation in
-    the kernel's order, so the bits are the kernel's.  Attention over these rows with sm_scale = ln 2
-    (exp(s ln 2) = 2^s) and no further rotation of q is what the kernel computes, so the comparison needs no
-    allowance for that rounding.  The table itself is held against the host's sincos (two units in the last place)."""
+    (BZ_ROPE_Q_ONLY / BZ_ROPE_FULL): rotated at their offset inside the request with the entries of the device's own
+    table (`table`, from prefill_angle_table: cos and sin times sm_scale * log2(e); the device's sincosf may differ from
+    the host's in the last place, and one such difference, rounded the other way and multiplied by logits of +-40, is
+    visible in the output) and rounded ONCE to the storage type -- every step an IEEE fp32 operation in the kernel's
+    order, so the bits are the kernel's.  Attention over these rows with sm_scale = ln 2 (exp(s ln 2) = 2^s) and no
+    further rotation of q is what the kernel computes, so the comparison needs no allowance for that rounding.  The
+    table itself is held against the host's sincos (two units in the last place)."""
     q = wl.to_f32(q_bits, dtype)
     N = q.shape[0]
     indptr = np.asarray(indptr)
     pos = np.arange(N) - np.repeat(indptr[:-1], np.diff(indptr))
     f = oracle.rope_freqs(D, theta)
     ang = pos[None, :].astype(np.float32) * f[:, None]  # [pairs][tokens], one fp32 multiply as on the device
+    if sm_scale is None:
+        sm_scale = np.float32(1.0) / np.sqrt(np.float32(D))
+    scale = np.float32(np.float32(sm_scale) * np.float32(1.4426950408889634))
     c, s_ = table[:, pos, 0], table[:, pos, 1]
-    assert np.abs(c - np.cos(ang.astype(np.float64))).max() <= 2.0 ** -22 and np.abs(s_ - np.sin(ang.astype(np.float64))).max() <= 2.0 ** -22
+    tol = 2.0 ** -22 * float(scale)
+    assert np.abs(c - np.cos(ang.astype(np.float64)) * float(scale)).max() <= tol
+    assert np.abs(s_ - np.sin(ang.astype(np.float64)) * float(scale)).max() <= tol
     c, s_ = c.T[:, None, :], s_.T[:, None, :]            # [tokens][1][pairs]
     x, y = q[:, :, : D // 2], q[:, :, D // 2:]
     xr = (x * c).astype(np.float32) - (y * s_).astype(np.float32)
     yr = (y * c).astype(np.float32) + (x * s_).astype(np.float32)
-    if sm_scale is None:
-        sm_scale = np.float32(1.0) / np.sqrt(np.float32(D))
-    scale = np.float32(np.float32(sm_scale) * np.float32(1.4426950408889634))
-    out = np.concatenate([xr, yr], axis=2).astype(np.float32) * scale
-    return wl.to_bits(out.astype(np.float32), dtype)
+    return wl.to_bits(np.concatenate([xr, yr], axis=2).astype(np.float32), dtype)
 
 
 LN2 = float(np.float32(0.6931471805599453))
