@@ -263,3 +263,56 @@ def test_wire_random_shapes(case):
     torch.cuda.synchronize()
     oracle.kv_pages_unpack(dst_bits, dtype, max_pages, sp, dst_ids, start, cnt, want)
     assert np.array_equal(to_host_bits(dst), dst_bits), case
+
+
+@pytest.mark.parametrize("case", range(18))
+def test_prefill_random_shapes_with_q_rows_for_the_last_tokens(case):
+    """Distinct ragged indices (src/kernel/attention.h:9-22 carries both): every request has K/V rows for all its tokens
+    and q rows for a random number of its last ones (none to all), in every RoPE mode and storage type, causal or not.
+    The result must be those rows of self-attention over the whole request, which is what the checker computes."""
+    from blitz_scale_amd._lib import BZ_PREFILL_BF16_HEAD_TAIL, BZ_PREFILL_BF16_WIDEN_V
+    from _gpu import to_dev, to_host_bits
+    from _util import prefill_angle_table, prefill_q_as_fed
+    rng = np.random.default_rng(9900 + case)
+    B = int(rng.integers(1, 6))
+    dtype, mode = [(BZ_F16, None), (BZ_BF16, BZ_PREFILL_BF16_WIDEN_V), (BZ_BF16, BZ_PREFILL_BF16_HEAD_TAIL)][case % 3]
+    Hkv = int(rng.choice([1, 2, 4]))
+    Hq = Hkv * int(rng.choice([1, 2, 4, 8]))
+    D = 128
+    kv_lens = rng.integers(1, int(rng.choice([40, 130, 300, 700])) + 1, B)
+    q_lens = np.array([int(rng.integers(0, l + 1)) for l in kv_lens])
+    q_lens[int(rng.integers(0, B))] = max(1, int(q_lens.max()))  # at least one q row in the batch
+    q_lens = np.minimum(q_lens, kv_lens)
+    causal = bool(rng.random() < 0.7)
+    rope_mode = [BZ_ROPE_NONE, BZ_ROPE_Q_ONLY, BZ_ROPE_FULL][(case // 3) % 3]
+    theta = float(rng.choice([1e4, 5e5]))
+    kvp = np.concatenate([[0], np.cumsum(kv_lens)]).astype(np.int32)
+    qop = np.concatenate([[0], np.cumsum(q_lens)]).astype(np.int32)
+    Nkv = int(kvp[-1])
+    q_full = wl.randn_bits(rng, (Nkv, Hq, D), dtype)
+    k = wl.randn_bits(rng, (Nkv, Hkv, D), dtype)
+    v = wl.randn_bits(rng, (Nkv, Hkv, D), dtype)
+    rows = np.concatenate([np.arange(kvp[b + 1] - q_lens[b], kvp[b + 1]) for b in range(B)]).astype(np.int32)
+    k_in = oracle.rope_ragged(k, dtype, kvp, Hkv, D, theta) if rope_mode == BZ_ROPE_Q_ONLY else k
+    fws = torch.empty(1 << 20, dtype=torch.uint8, device="cuda")
+    iws = torch.empty(1 << 20, dtype=torch.uint8, device="cuda")
+    h = K.BatchPrefillRaggedHandler()
+    if mode is not None:
+        h.set_bf16_mode(mode)
+    h.plan(fws, fws.numel(), iws, iws.numel(), qop, kvp, B, Hq, Hkv, D, 16)
+    qd, kd, vd = to_dev(q_full[rows], dtype), to_dev(k_in, dtype), to_dev(v, dtype)
+    out = torch.full_like(qd, float("nan"))
+    K.batch_prefill_attention(h, qd, torch.from_numpy(qop).cuda(), kd, vd, torch.from_numpy(kvp).cuda(), out, B, Hq, Hkv, D,
+                              causal=causal, rope_mode=rope_mode, rope_theta=theta)
+    torch.cuda.synchronize()
+    got = wl.to_f32(to_host_bits(out), dtype)
+    assert not np.isnan(got).any()
+    k_after = to_host_bits(kd)
+    if rope_mode == BZ_ROPE_NONE:
+        ref = oracle.batch_prefill_ragged(q_full, k, v, dtype, kvp, Hq, Hkv, D, causal=causal, rows=rows, parallel=True)
+    else:
+        q_fed = prefill_q_as_fed(q_full, dtype, kvp, Hq, D, theta, prefill_angle_table(fws, int(kv_lens.max()), D))
+        ref = oracle.batch_prefill_ragged(q_fed, k_after, v, dtype, kvp, Hq, Hkv, D, causal=causal, sm_scale=LN2, rows=rows,
+                                          parallel=True)
+    tol = ulp_tol(ref, dtype, before_rounding=PREFILL_BF16_WIDEN_V_ERR if mode == BZ_PREFILL_BF16_WIDEN_V else 0.0)
+    assert (np.abs(got - ref) <= tol).all(), (case, float(np.abs(got - ref).max()))
