@@ -82,3 +82,22 @@ def test_argument_errors_are_reported_before_anything_touches_a_gpu():
                                 None) == _lib.BZ_ERR_UNSUPPORTED
     assert lib.bz_kv_pages_pack(fake, 100, None, fake, 4, 0, 2, fake, _lib.BZ_E4M3, None, None,
                                 None) == _lib.BZ_ERR_BAD_ARG
+    # the cached-K conversion: table pointers cleared -> bad argument; an e4m3 pool would be requantised -> unsupported
+    assert lib.bz_rope_cached_k(C.byref(kv), 1e4, 0, None) == _lib.BZ_ERR_BAD_ARG
+    ids = (C.c_int32 * 8)()
+    kv.indices = kv.indptr = kv.last_page_len = C.addressof(ids)
+    assert lib.bz_rope_cached_k(C.byref(kv), 1e4, 0, None) == _lib.BZ_ERR_UNSUPPORTED
+    assert lib.bz_rope_cached_k(None, 1e4, 0, None) == _lib.BZ_ERR_BAD_ARG
+    # prefill plan: the bf16 mode is one of the two named ones; fewer K/V rows than q rows is refused on the host
+    pplan = lib.bz_prefill_plan_create()
+    try:
+        assert lib.bz_prefill_plan_set_bf16_mode(pplan, 2) == _lib.BZ_ERR_BAD_ARG
+        assert lib.bz_prefill_plan_set_bf16_mode(pplan, _lib.BZ_PREFILL_BF16_HEAD_TAIL) == 0
+        qo, kvp = (C.c_int32 * 2)(0, 10), (C.c_int32 * 2)(0, 9)
+        fb, ib = C.c_size_t(), C.c_size_t()
+        assert lib.bz_prefill_plan_workspace(pplan, qo, kvp, 1, 4, 4, 128, C.byref(fb), C.byref(ib)) == _lib.BZ_ERR_UNSUPPORTED
+        kvp[1] = 30
+        assert lib.bz_prefill_plan_workspace(pplan, qo, kvp, 1, 4, 4, 128, C.byref(fb), C.byref(ib)) == 0
+        assert fb.value == 30 * 512 and ib.value == 256  # the angle table covers the K/V length; one job of 32 bytes
+    finally:
+        lib.bz_prefill_plan_destroy(pplan)

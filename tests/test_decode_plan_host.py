@@ -241,3 +241,30 @@ def test_prefill_job_list_invariants(lens, Hq, Hkv):
     # a head size the kernel does not cover is refused on the host
     with pytest.raises(K.BzError):
         h.workspace(indptr, indptr, len(lens), Hq, Hkv, 64)
+
+
+def test_prefill_job_list_with_distinct_q_and_kv_lengths():
+    """qo_indptr != kv_indptr: a job covers 128 q rows of the request's last qo_len tokens and carries the request's
+    K/V range; requests are ordered by their K/V length (what a tile's work goes with); no q rows, no jobs."""
+    kv_lens = np.array([300, 64, 1000, 40], np.int64)
+    q_lens = np.array([130, 64, 0, 1], np.int64)
+    qo = np.concatenate([[0], np.cumsum(q_lens)]).astype(np.int32)
+    kv = np.concatenate([[0], np.cumsum(kv_lens)]).astype(np.int32)
+    h = K.BatchPrefillRaggedHandler()
+    fb, ib = h.workspace(qo, kv, 4, 8, 2, 128)
+    items = h.host_schedule()
+    assert fb == 512 * 1000  # the angle table covers the longest K/V length
+    live = items[items[:, 1] > 0]
+    want = {(b, hd, q0) for b in range(4) for hd in range(8) for q0 in range(0, int(q_lens[b]), 128)}
+    seen = set()
+    for tok0, ln, q0, head, kv0, kv_len, _, _ in live:
+        b = int(np.searchsorted(qo[1:], tok0, side="right"))
+        while q_lens[b] == 0:
+            b += 1
+        assert tok0 == qo[b] and ln == q_lens[b] and kv0 == kv[b] and kv_len == kv_lens[b]
+        seen.add((b, int(head), int(q0)))
+    assert seen == want and len(live) == len(want)
+    first = [int(r[5]) for r in live[::1] if r[2] == (r[1] - 1) // 128 * 128 and r[3] == 0]
+    assert first[0] == 300  # among the requests with q rows, the longest K/V range is dealt first
+    with pytest.raises(K.BzError):
+        h.workspace(kv, qo, 4, 8, 2, 128)  # fewer K/V rows than q rows
