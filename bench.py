@@ -1,6 +1,6 @@
 """Benchmark of the paged-attention compute path on one MI355X.  Prints ONE JSON line.
 
-Default workload (the headline, BASELINE config 3): Llama-3-8B-shaped GQA paged decode, bf16, batch
+Default workload (the headline, benchmark configuration 3): Llama-3-8B-shaped GQA paged decode, bf16, batch
 128, 32/8 heads, head_dim 128, page_size 16, log-normal contexts.  A step is one layer's decode-time
 attention block over the whole batch: the KV append of the new token (K rotated) and the batch decode
 over the paged KV cache (src/layer/attn.h:196-203 of the reference), issued as the library's one-call

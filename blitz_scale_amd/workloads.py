@@ -101,7 +101,7 @@ def lognormal_ctx(rng, batch, mean=1024.0, sigma=1.0, lo=64, hi=8192):
     return np.clip(np.rint(np.exp(mu + sigma * z)), lo, hi).astype(np.int64)
 
 
-# ---- the benchmark configurations (BASELINE.json `configs`, in order) -----------------------
+# ---- the benchmark configurations (the target file's `configs`, in order) -----------------------
 CONFIGS = {
     "C1": dict(kind="decode", dtype=BZ_F16, kv_dtype=BZ_F16, batch=4, Hq=4, Hkv=4, D=64, P=16, pool_pages=64,
                ctx=[17, 64, 130, 255], rope_theta=None),

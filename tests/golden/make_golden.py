@@ -1,4 +1,4 @@
-"""Writes tests/golden/c1_decode.npz: BASELINE config 1 (fp16, batch 4, 4/4 heads, D 64, P 16,
+"""Writes tests/golden/c1_decode.npz: benchmark configuration 1 (fp16, batch 4, 4/4 heads, D 64, P 16,
 ctx {17,64,130,255}, 64-page pool, scale 1/8, no RoPE) generated from the seeded workload generator,
 with the CPU checker's fp32 output and digests of the input bits.  The reference holds no numeric
 vectors for this path, so this fixture pins the generator and the checker against drift; the GPU

@@ -1,4 +1,4 @@
-"""The committed fixture of BASELINE config 1 pins the workload generator and the checker (CPU) and
+"""The committed fixture of benchmark configuration 1 pins the workload generator and the checker (CPU) and
 the HIP path (GPU) to the same numbers."""
 import os
 import sys

@@ -51,7 +51,7 @@ def _check_one(p, split_tokens, rope_mode, theta, f32_tol, ref, ref_lse):
 
 
 def test_c1_plumbing_config():
-    """BASELINE config 1: fp16, batch 4, 4/4 heads, D 64, P 16, ctx {17,64,130,255}, 64-page pool, no RoPE."""
+    """benchmark configuration 1: fp16, batch 4, 4/4 heads, D 64, P 16, ctx {17,64,130,255}, 64-page pool, no RoPE."""
     cfg = wl.CONFIGS["C1"]
     p = DecodeProblem(wl.DEFAULT_SEED, cfg["ctx"], cfg["Hq"], cfg["Hkv"], cfg["D"], cfg["P"], cfg["dtype"],
                       pool_pages=cfg["pool_pages"])

@@ -1,4 +1,4 @@
-"""GPU parity at the FULL batch sizes of BASELINE configs 2 and 5 (and one whole request of config 4).
+"""GPU parity at the FULL batch sizes of benchmark configurations 2 and 5 (and one whole request of config 4).
 
 At these sizes the checker would take minutes over the whole batch, so the HIP path runs the full batch (the
 planner regime of thousands of wave slots, the instantiation with hinted loads, megabytes of tile records) and

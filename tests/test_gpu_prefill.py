@@ -188,7 +188,7 @@ def test_prefill_then_store_then_decode_is_consistent():
 @pytest.mark.parametrize("batch", [4, 16])
 def test_c4_shape_sampled_rows(batch):
     """Llama-2-13B-shaped prefill (40/40 heads, D 128, f16, lengths U[128,4096], causal); batch 16 is the
-    full BASELINE config 4.  The checker evaluates a seeded sample of rows (all heads) plus the first and
+    full benchmark configuration 4.  The checker evaluates a seeded sample of rows (all heads) plus the first and
     last row of every request."""
     cfg = wl.CONFIGS["C4"]
     rng = np.random.default_rng(wl.DEFAULT_SEED)
@@ -204,7 +204,7 @@ def test_c4_shape_sampled_rows(batch):
 
 
 def test_c4_one_whole_request_of_full_length():
-    """BASELINE config 4 at full size (16 prompts, 40/40 heads): EVERY row of the longest request (all heads)
+    """benchmark configuration 4 at full size (16 prompts, 40/40 heads): EVERY row of the longest request (all heads)
     against the checker, i.e. every causal length from 1 to the request's end through every q tile and wave."""
     cfg = wl.CONFIGS["C4"]
     rng = np.random.default_rng(wl.DEFAULT_SEED)
@@ -221,7 +221,7 @@ def test_c4_one_whole_request_of_full_length():
 
 
 def test_c4_rope_store_then_attention_at_full_size():
-    """BASELINE config 4 as the layer runs it (src/layer/attn.h:173-193 with this library's order of calls), at full
+    """benchmark configuration 4 as the layer runs it (src/layer/attn.h:173-193 with this library's order of calls), at full
     size: 16 prompts U[128,4096], 40/40 heads, f16, RoPE theta 1e4, page size 16, seeded page placement with the
     reference's len+1 reservation.  store_prefill_kv_cache(rope = 2) rotates K into the pages and in the caller's
     rows, batch_prefill_attention(BZ_ROPE_Q_ONLY) rotates q in registers.  Checked: the pool against the checker's
