@@ -604,98 +604,70 @@ __global__ __launch_bounds__(256, 2) void prefill_kernel(PrefillArgs a, const ch
     // ---- the steady state: every tile touched exists, is whole and needs no mask.  SL = j % 4 is the slot of
     // K(j) and of V(j), a compile-time constant (the loop is unrolled by four), so that LDS addresses are one
     // register plus an immediate and the copies' LDS targets are constants as well.
-    int kj = 0, vj = 0; // j % kSNK, j % kSNV (used by `generic`)
     const char* k_next = k_wave + (size_t)kSNK * tile_stride;       // K(j + kSNK)
     const char* v_next = v_wave + (size_t)(kSNV - 1) * tile_stride; // V(j + kSNV - 1)
-    // COND: the copies and the count of copies in flight are looked at (the last few tiles of a job), otherwise
-    // the tiles copied are known to exist and to be whole.
-    auto full = [&](int j, auto par_c, auto sl_c, auto cond_c) __attribute__((always_inline)) {
+    auto full = [&](int j, auto par_c, auto sl_c) __attribute__((always_inline)) {
         constexpr int PAR = decltype(par_c)::value, SL = decltype(sl_c)::value;
-        constexpr bool COND = decltype(cond_c)::value;
-        if (!COND) {
-            sp_wait_copies(sp_copies_behind_steady(V_F16)); // K(j+2) and V(j) have landed (V_F16: V(j+1) too)
-            sp_barrier();
-            lds_direct_load16x2(k_next, kfast[0], kfast[1], m0_wave + (uint32_t)(SL * kSTile));
-            lds_direct_load16x2(v_next, vfast[0], vfast[1], m0_wave + (uint32_t)((kSNK + (SL + kSNV - 1) % kSNV) * kSTile));
-            k_next += tile_stride;
-            v_next += tile_stride;
-        } else {
-            // behind K(j+2): V(j+1), K(j+3), V(j+2), of which only K(j+3) may be missing here
-            sp_wait_copies((V_F16 ? 1 : 2) + (j + 3 < n ? 1 : 0));
-            sp_barrier();
-            if (j + kSNK < n) issue_k(j + kSNK, SL);
-            if (j + kSNV - 1 < n) issue_v(j + kSNV - 1, (SL + kSNV - 1) % kSNV);
-        }
+        sp_wait_copies(sp_copies_behind_steady(V_F16)); // K(j+2) and V(j) have landed (V_F16: V(j+1) too)
+        sp_barrier();
+        lds_direct_load16x2(k_next, kfast[0], kfast[1], m0_wave + (uint32_t)(SL * kSTile));
+        lds_direct_load16x2(v_next, vfast[0], vfast[1], m0_wave + (uint32_t)((kSNK + (SL + kSNV - 1) % kSNV) * kSTile));
+        k_next += tile_stride;
+        v_next += tile_stride;
         if (V_F16) widen_v((SL + 1) % kSNV); // V(j+1), first read after the next barrier
         first_half(par_c, std::true_type{}, std::true_type{}, k_at((SL + 1) % kSNK), v_at(SL));
         if (__any(!(psum < 32768.0f))) move_maximum(s[PAR], s[PAR ^ 1]);
         l_run += psum;
         second_half(std::true_type{}, v_at(SL), k_at((SL + 2) % kSNK));
     };
-    // ---- the same with every condition checked.  The operand reads are issued by every wave, also one that has
-    // nothing to compute, so that the registers have one definition per iteration.
-    auto generic = [&](int j, auto par_c) __attribute__((always_inline)) {
-        constexpr int PAR = decltype(par_c)::value;
+    // ---- the same with every condition checked (the slots are still compile-time constants: j % 4 == SL).  The operand
+    // reads are issued by every wave, also one that has nothing to compute, so that the registers have one definition
+    // per iteration.
+    auto generic = [&](int j, auto par_c, auto sl_c) __attribute__((always_inline)) {
+        constexpr int PAR = decltype(par_c)::value, SL = decltype(sl_c)::value;
         const bool has_cur = j < n_w, has_next = j + 1 < n_w;
         sp_wait_copies(sp_copies_behind(j, n, V_F16));
         sp_barrier();
-        if (j + kSNK < n) issue_k(j + kSNK, kj);
-        if (j + kSNV - 1 < n) issue_v(j + kSNV - 1, sp_wrap(vj + kSNV - 1, kSNV));
-        if (V_F16 && j + 1 < n) widen_v(sp_wrap(vj + 1, kSNV));
-        const uint32_t k1 = k_at(sp_wrap(kj + 1, kSNK)), k2 = k_at(sp_wrap(kj + 2, kSNK));
-        if (has_next) first_half(par_c, std::true_type{}, std::true_type{}, k1, v_at(vj));
-        else first_half(par_c, std::false_type{}, std::true_type{}, k1, v_at(vj)); // (harmless without a tile: p of stale scores, never used)
+        if (j + kSNK < n) issue_k(j + kSNK, SL);
+        if (j + kSNV - 1 < n) issue_v(j + kSNV - 1, (SL + kSNV - 1) % kSNV);
+        if (V_F16 && j + 1 < n) widen_v((SL + 1) % kSNV);
+        const uint32_t k1 = k_at((SL + 1) % kSNK), k2 = k_at((SL + 2) % kSNK);
+        if (has_next) first_half(par_c, std::true_type{}, std::true_type{}, k1, v_at(SL));
+        else first_half(par_c, std::false_type{}, std::true_type{}, k1, v_at(SL)); // (harmless without a tile: p of stale scores, never used)
         if (has_cur) {
             if (__any(!(psum < 32768.0f))) move_maximum(s[PAR], s[PAR ^ 1]);
             l_run += psum;
             if (has_next) mask_tile(j + 1, s[PAR ^ 1]);
-            second_half(std::true_type{}, v_at(vj), k2);
+            second_half(std::true_type{}, v_at(SL), k2);
         } else {
-            second_half(std::false_type{}, v_at(vj), k2);
+            second_half(std::false_type{}, v_at(SL), k2);
         }
-        kj = sp_wrap(kj + 1, kSNK);
-        vj = sp_wrap(vj + 1, kSNV);
     };
-    // full needs: tiles j .. j+2 computed by this wave and tile j+1 unmasked; without COND also the tiles it copies
-    // whole and in range
-    const int j_cond = min(n_w - 2, t_diag - 1);
-    const int j_full = min(j_cond, min(L / kSN, n) - kSNK);
+    // full needs: tiles j .. j+2 computed by this wave, tile j+1 unmasked, and the tiles it copies whole and in range
+    const int j_full = min(min(n_w - 2, t_diag - 1), min(L / kSN, n) - kSNK);
     const std::integral_constant<int, 0> c0{};
     const std::integral_constant<int, 1> c1{};
     const std::integral_constant<int, 2> c2{};
     const std::integral_constant<int, 3> c3{};
     int j = 0;
     for (; j + 3 < j_full; j += 4) {
-        full(j, c0, c0, std::false_type{});
-        full(j + 1, c1, c1, std::false_type{});
-        full(j + 2, c0, c2, std::false_type{});
-        full(j + 3, c1, c3, std::false_type{});
+        full(j, c0, c0);
+        full(j + 1, c1, c1);
+        full(j + 2, c0, c2);
+        full(j + 3, c1, c3);
     }
-    for (; j + 3 < j_cond; j += 4) {
-        full(j, c0, c0, std::true_type{});
-        full(j + 1, c1, c1, std::true_type{});
-        full(j + 2, c0, c2, std::true_type{});
-        full(j + 3, c1, c3, std::true_type{});
-    }
-    if (j < j_cond) { // (j is a multiple of four here: up to three more, slots known)
-        full(j, c0, c0, std::true_type{});
-        if (++j < j_cond) {
-            full(j, c1, c1, std::true_type{});
-            if (++j < j_cond) {
-                full(j, c0, c2, std::true_type{});
-                ++j;
+    BZ_PF_WG(4);
+    // the rest (j is a multiple of four): the last tiles of the job, the diagonal ones and everything ragged.  Nested,
+    // not one condition after the other: a tile's registers are then defined on one path only.
+    for (; j < n; j += 4) {
+        generic(j, c0, c0);
+        if (j + 1 < n) {
+            generic(j + 1, c1, c1);
+            if (j + 2 < n) {
+                generic(j + 2, c0, c2);
+                if (j + 3 < n) generic(j + 3, c1, c3);
             }
         }
-    }
-    kj = vj = j & 3;
-    BZ_PF_WG(4);
-    if ((j & 1) && j < n) {
-        generic(j, c1);
-        ++j;
-    }
-    for (; j < n; j += 2) { // (j is even here)
-        generic(j, std::integral_constant<int, 0>{});
-        if (j + 1 < n) generic(j + 1, std::integral_constant<int, 1>{});
     }
     sp_barrier(); // nobody reads a tile any more: the epilogue takes their place
     BZ_PF_WG(5);
