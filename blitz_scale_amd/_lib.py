@@ -68,6 +68,7 @@ SIGNATURES = {
     "bz_prefill_plan_workspace": (_i32, [_vp, _vp, _vp, _u32, _u32, _u32, _u32, C.POINTER(_sz), C.POINTER(_sz)]),
     "bz_prefill_plan_host_schedule": (_i32, [_vp, C.POINTER(_vp), C.POINTER(_sz), C.POINTER(_u32)]),
     "bz_prefill_plan_set_bf16_mode": (_i32, [_vp, _i32]),
+    "bz_prefill_plan_set_timing_events": (_i32, [_vp, _vp, _vp]),
     "bz_rope_cached_k": (_i32, [_vp, _f32, _i32, _vp]),
     "bz_batch_prefill_ragged": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i32, _u32, _u32, _u32, _u32, _i32, _i32,
                                        _f32, _f32, _vp]),

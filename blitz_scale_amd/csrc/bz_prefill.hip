@@ -68,6 +68,7 @@ struct PrefillPlan {
     void* staging = nullptr;
     size_t staging_bytes = 0;
     hipEvent_t upload_done = nullptr;
+    hipEvent_t time_start = nullptr, time_stop = nullptr; // optional: bracket the attention kernel's launch
 };
 
 struct PrefillArgs {
@@ -803,6 +804,14 @@ extern "C" int bz_prefill_plan_set_bf16_mode(bz_prefill_plan_t* plan_, int mode)
     return 0;
 }
 
+extern "C" int bz_prefill_plan_set_timing_events(bz_prefill_plan_t* plan_, void* start_event, void* stop_event) {
+    PrefillPlan* p = reinterpret_cast<PrefillPlan*>(plan_);
+    if (!p || ((start_event == nullptr) != (stop_event == nullptr))) return BZ_ERR_BAD_ARG;
+    p->time_start = (hipEvent_t)start_event;
+    p->time_stop = (hipEvent_t)stop_event;
+    return 0;
+}
+
 extern "C" void bz_prefill_plan_destroy(bz_prefill_plan_t* plan_) {
     PrefillPlan* p = reinterpret_cast<PrefillPlan*>(plan_);
     if (!p) return;
@@ -955,8 +964,10 @@ static int launch_prefill(const PrefillPlan* p, const PrefillArgs& a, const void
         BZ_CHECK_HIP(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, kSLds));
         attr_done.fetch_or(bit, std::memory_order_relaxed);
     }
+    if (p->time_start) BZ_CHECK_HIP(hipEventRecord(p->time_start, s));
     hipLaunchKernelGGL(kern, dim3(p->num_items), dim3(256), kSLds, s, a, (const char*)q, (const char*)k, (const char*)v);
     BZ_LAUNCH_CHECK();
+    if (p->time_stop) BZ_CHECK_HIP(hipEventRecord(p->time_stop, s));
     return 0;
 }
 

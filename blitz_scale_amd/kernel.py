@@ -208,6 +208,10 @@ class BatchPrefillRaggedHandler:
               "Handler workspace")
         return fb.value, ib.value
 
+    def set_timing_events(self, start=None, stop=None):
+        """hipEvent_t handles recorded right before / after the attention kernel's launch (None: off)."""
+        check(_lib.load().bz_prefill_plan_set_timing_events(self._h, start, stop), "Handler timing events")
+
     def set_bf16_mode(self, mode):
         """BZ_PREFILL_BF16_WIDEN_V (default) or BZ_PREFILL_BF16_HEAD_TAIL: see include/bz_hip.h."""
         check(_lib.load().bz_prefill_plan_set_bf16_mode(self._h, mode), "Handler bf16 mode")

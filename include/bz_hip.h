@@ -238,6 +238,11 @@ int bz_prefill_plan_host_schedule(const bz_prefill_plan_t* plan, const int32_t**
 #define BZ_PREFILL_BF16_HEAD_TAIL 1
 int bz_prefill_plan_set_bf16_mode(bz_prefill_plan_t* plan, int mode);
 
+/* Profiling aid, as bz_decode_plan_set_timing_events: two hipEvent_t handles recorded on the call's stream right
+ * before and right after the launch of the attention kernel of bz_batch_prefill_ragged (not around the kernels that
+ * rotate k or write the angle table in front of it).  Both NULL switches it off.  No counterpart in the reference. */
+int bz_prefill_plan_set_timing_events(bz_prefill_plan_t* plan, void* start_event, void* stop_event);
+
 /*
  * batch_prefill_attention (src/kernel/attention.h:9-22, attention_prefill.cu:11-46): ragged
  * attention, q [Nq,Hq,D], k,v [Nkv,Hkv,D], out [Nq,Hq,D].  The reference passes one array as qo_indptr and
