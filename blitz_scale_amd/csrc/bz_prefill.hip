@@ -255,6 +255,18 @@ __device__ unsigned long long bz_pf_wg[kPftMaxWg * 8];
 #else
 #define BZ_PF_WG(k) do { } while (0)
 #endif
+#ifdef BZ_PF_PHASES
+// Diagnostic build on top of BZ_PF_TIMING: the first and the last wave of every workgroup add up, over their
+// steady-state iterations, the shader clock spent in each part of an iteration (bz_pf_ph, read through
+// bz_pf_phase_table).  Reading the clock waits for the wave's outstanding LDS reads, so the parts are a little
+// longer than in the library proper.
+__device__ unsigned long long bz_pf_ph[kPftMaxWg * 2 * 8];
+#define BZ_PF_PH_START() do { __builtin_amdgcn_sched_barrier(0); ph_last = __builtin_amdgcn_s_memtime(); __builtin_amdgcn_sched_barrier(0); } while (0)
+#define BZ_PF_PH(k) do { __builtin_amdgcn_sched_barrier(0); const unsigned long long t_ = __builtin_amdgcn_s_memtime(); ph[k] += t_ - ph_last; ph_last = t_; __builtin_amdgcn_sched_barrier(0); } while (0)
+#else
+#define BZ_PF_PH_START() do { } while (0)
+#define BZ_PF_PH(k) do { } while (0)
+#endif
 
 // bf16 has two ways through the second contraction (the 8-bit significand of a bf16 probability alone would eat
 // the error budget).  SPLIT_P: the probabilities enter it as head + tail of bf16, two matrix instructions per step.
@@ -272,6 +284,9 @@ __global__ __launch_bounds__(256, 2) void prefill_kernel(PrefillArgs a, const ch
     constexpr bool QSCALED = ROPE_Q; // q carries sm_scale * log2(e)
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
 #ifdef BZ_PF_TIMING
+#ifdef BZ_PF_PHASES
+    unsigned long long ph[6] = {0, 0, 0, 0, 0, 0}, ph_last = 0;
+#endif
     unsigned long long pft[8];
     pft[0] = __builtin_amdgcn_s_memtime();
     pft[7] = __builtin_amdgcn_s_memrealtime();
@@ -609,17 +624,23 @@ __global__ __launch_bounds__(256, 2) void prefill_kernel(PrefillArgs a, const ch
     const char* v_next = v_wave + (size_t)(kSNV - 1) * tile_stride; // V(j + kSNV - 1)
     auto full = [&](int j, auto par_c, auto sl_c) __attribute__((always_inline)) {
         constexpr int PAR = decltype(par_c)::value, SL = decltype(sl_c)::value;
+        BZ_PF_PH_START();
         sp_wait_copies(sp_copies_behind_steady(V_F16)); // K(j+2) and V(j) have landed (V_F16: V(j+1) too)
+        BZ_PF_PH(0);
         sp_barrier();
+        BZ_PF_PH(1);
         lds_direct_load16x2(k_next, kfast[0], kfast[1], m0_wave + (uint32_t)(SL * kSTile));
         lds_direct_load16x2(v_next, vfast[0], vfast[1], m0_wave + (uint32_t)((kSNK + (SL + kSNV - 1) % kSNV) * kSTile));
         k_next += tile_stride;
         v_next += tile_stride;
         if (V_F16) widen_v((SL + 1) % kSNV); // V(j+1), first read after the next barrier
+        BZ_PF_PH(2);
         first_half(par_c, std::true_type{}, std::true_type{}, k_at((SL + 1) % kSNK), v_at(SL));
+        BZ_PF_PH(3);
         if (__any(!(psum < 32768.0f))) move_maximum(s[PAR], s[PAR ^ 1]);
         l_run += psum;
         second_half(std::true_type{}, v_at(SL), k_at((SL + 2) % kSNK));
+        BZ_PF_PH(4);
     };
     // ---- the same with every condition checked (the slots are still compile-time constants: j % 4 == SL).  The operand
     // reads are issued by every wave, also one that has nothing to compute, so that the registers have one definition
@@ -700,6 +721,13 @@ __global__ __launch_bounds__(256, 2) void prefill_kernel(PrefillArgs a, const ch
             *reinterpret_cast<uint4*>(orow + (lane & 15) * 16) = v;
         }
     }
+#ifdef BZ_PF_PHASES
+    if ((wv == 0 || wv == 3) && lane == 0 && blockIdx.x < kPftMaxWg) {
+        unsigned long long* dst = bz_pf_ph + ((size_t)blockIdx.x * 2 + (wv == 3 ? 1 : 0)) * 8;
+        for (int i = 0; i < 5; ++i) dst[i] = ph[i];
+        dst[5] = (unsigned long long)max(j_full, 0) / 4 * 4; // steady-state iterations of this wave
+    }
+#endif
 #ifdef BZ_PF_TIMING
     if (tid == 0 && blockIdx.x < kPftMaxWg) {
         pft[6] = __builtin_amdgcn_s_memtime();
@@ -707,7 +735,7 @@ __global__ __launch_bounds__(256, 2) void prefill_kernel(PrefillArgs a, const ch
         unsigned hw = 0, xcc = 0;
         asm volatile("s_getreg_b32 %0, hwreg(HW_REG_HW_ID)" : "=s"(hw));
         asm volatile("s_getreg_b32 %0, hwreg(HW_REG_XCC_ID)" : "=s"(xcc));
-        bz_pf_wg[blockIdx.x * 8 + 0] = ((unsigned long long)n << 32) | (unsigned)max(j_cond, 0);
+        bz_pf_wg[blockIdx.x * 8 + 0] = ((unsigned long long)n << 32) | (unsigned)max(j_full, 0);
         bz_pf_wg[blockIdx.x * 8 + 2] = ((unsigned long long)(xcc & 15) << 32) | hw; // (replaces the K0-landed stamp)
         for (int i = 1; i < 7; ++i) if (i != 2) bz_pf_wg[blockIdx.x * 8 + i] = pft[i] - pft[0];
         bz_pf_wg[blockIdx.x * 8 + 7] = ((__builtin_amdgcn_s_memrealtime() - pft[7]) << 40) | (pft[7] & 0xffffffffffull);
@@ -971,6 +999,13 @@ static int launch_prefill(const PrefillPlan* p, const PrefillArgs& a, const void
     return 0;
 }
 
+#ifdef BZ_PF_PHASES
+extern "C" int bz_pf_phase_table(unsigned long long* host, size_t count) {
+    if (count > sizeof(bz_pf_ph) / 8) count = sizeof(bz_pf_ph) / 8;
+    BZ_CHECK_HIP(hipMemcpyFromSymbol(host, HIP_SYMBOL(bz_pf_ph), count * 8, 0, hipMemcpyDeviceToHost));
+    return 0;
+}
+#endif
 #ifdef BZ_PF_TIMING
 // copies the table of the diagnostic build to the host: per workgroup 8 values (see prefill_kernel)
 extern "C" int bz_pf_wg_table(unsigned long long* host, size_t count) {
