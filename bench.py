@@ -300,14 +300,18 @@ def bench_decode(args, name):
             # host thread (tens of microseconds) is not counted into a region of a few milliseconds.
             torch.cuda.synchronize()
             t0 = time.perf_counter()
-            dev_ev[r][0].record()
             run_steps(steps)
-            dev_ev[r][1].record()
             done.record()
             while not done.query():
                 pass
             torch.cuda.synchronize()
             region_ms.append((time.perf_counter() - t0) * 1e3)
+        for r in range(regions):  # the same regions once more between two events on the stream (not part of `value`)
+            torch.cuda.synchronize()
+            dev_ev[r][0].record()
+            run_steps(steps)
+            dev_ev[r][1].record()
+        torch.cuda.synchronize()
         region_us = np.array(region_ms) / steps  # ms per step of each region; pct() scales to us
         device_us = np.array([a.elapsed_time(b) for a, b in dev_ev]) / steps
         ms_per_step = float(region_us.mean())
