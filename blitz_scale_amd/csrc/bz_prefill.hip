@@ -1029,14 +1029,13 @@ extern "C" int bz_batch_prefill_ragged(bz_prefill_plan_t* plan_, void* q, const 
     if (rope_mode < BZ_ROPE_NONE || rope_mode > BZ_ROPE_FULL) return BZ_ERR_BAD_ARG;
     if (((uintptr_t)q | (uintptr_t)k | (uintptr_t)v | (uintptr_t)out) % 16) return BZ_ERR_BAD_ARG;
     hipStream_t s = (hipStream_t)stream;
-    if (p->num_items == 0) return 0;
     // q is rotated in registers inside the attention kernel (angles from a table in the float workspace) and
     // stays as it is in memory; k, which every q tile of a request reads, is rotated once, in place, first.
     bool rope_q = rope_mode != BZ_ROPE_NONE;
     if (rope_mode != BZ_ROPE_NONE) {
         const float theta = rope_theta > 0.f ? rope_theta : 1e4f;
         const RopeFreqs freqs = make_rope_freqs(128, theta);
-        if (p->rope_table) {
+        if (p->rope_table && p->num_items > 0) {
             // (every call: the workspace may be shared with other handlers between calls, calls may change streams,
             // and a captured call must replay its own fill; a few microseconds)
             const float scale = (sm_scale > 0.f ? sm_scale : 1.0f / sqrtf((float)head_dim)) * 1.4426950408889634f;
@@ -1058,6 +1057,7 @@ extern "C" int bz_batch_prefill_ragged(bz_prefill_plan_t* plan_, void* q, const 
         BZ_LAUNCH_CHECK();
         rope_q = p->rope_table != nullptr;
     }
+    if (p->num_items == 0) return 0; // no q rows in the batch (K, if the call was to rotate it, has been rotated)
     PrefillArgs a;
     a.out = out;
     a.items = p->items_d;

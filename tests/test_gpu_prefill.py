@@ -346,6 +346,28 @@ def test_q_rows_for_the_last_tokens_of_a_request_only(kind, causal, rope_mode, f
     assert (np.abs(got - ref) <= kind_tol(ref, kind)).all(), np.abs(got - ref).max()
 
 
+def test_a_batch_without_q_rows_still_rotates_k():
+    """BZ_ROPE_FULL promises rotated k rows in the caller's buffer (the page store that follows copies them), also
+    when no request of the batch has a q row."""
+    rng = np.random.default_rng(270)
+    kv_lens, Hq, Hkv, D, dtype, theta = [5, 70], 4, 2, 128, BZ_F16, 1e4
+    kvp = np.concatenate([[0], np.cumsum(kv_lens)]).astype(np.int32)
+    qop = np.zeros(3, np.int32)
+    k, v = wl.randn_bits(rng, (75, Hkv, D), dtype), wl.randn_bits(rng, (75, Hkv, D), dtype)
+    fws = torch.empty(1 << 20, dtype=torch.uint8, device="cuda")
+    iws = torch.empty(1 << 20, dtype=torch.uint8, device="cuda")
+    h = K.BatchPrefillRaggedHandler()
+    h.plan(fws, fws.numel(), iws, iws.numel(), qop, kvp, 2, Hq, Hkv, D, 16)
+    qd = torch.zeros((1, Hq, D), dtype=torch.float16, device="cuda")  # (a valid pointer; no row is read)
+    kd, vd = to_dev(k, dtype), to_dev(v, dtype)
+    K.batch_prefill_attention(h, qd, torch.from_numpy(qop).cuda(), kd, vd, torch.from_numpy(kvp).cuda(), qd.clone(), 2, Hq, Hkv,
+                              D, causal=True, rope_mode=BZ_ROPE_FULL, rope_theta=theta)
+    torch.cuda.synchronize()
+    k_rot = oracle.rope_ragged(k, dtype, kvp, Hkv, D, theta)
+    got = to_host_bits(kd)
+    assert np.abs(wl.to_f32(got, dtype) - wl.to_f32(k_rot, dtype)).max() <= 2.0 ** -8 and (got != k_rot).mean() < 2e-3
+
+
 def test_fewer_kv_rows_than_q_rows_is_refused():
     h = K.BatchPrefillRaggedHandler()
     with pytest.raises(K.BzError, match="Handler workspace"):
