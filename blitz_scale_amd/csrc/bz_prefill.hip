@@ -870,8 +870,8 @@ static int build_prefill_items(PrefillPlan* p, const int32_t* qo_indptr_h, const
     // with its own L2, so launch index i runs on XCD i % 8.  Every (request, kv head) unit is given to one
     // XCD as a run of consecutive jobs: its q tiles (of all q heads of the group) then execute together on
     // that XCD and share the unit's K/V (up to 2 MiB for 4096 tokens) through that L2 instead of each
-    // fetching it from HBM.  Units go to the XCDs in turn, longest requests first and tiles from the last
-    // (most keys) to the first, so every XCD gets the same mix of work.
+    // fetching it from HBM.  Units go to the XCDs in turn, longest requests first, so every XCD gets the same
+    // mix of work.
     for (uint32_t b = 0; b < batch_size; ++b)
         if (qo_indptr_h[b + 1] < qo_indptr_h[b]) return BZ_ERR_BAD_ARG;
     std::vector<uint32_t> order(batch_size);
@@ -891,15 +891,26 @@ static int build_prefill_items(PrefillPlan* p, const int32_t* qo_indptr_h, const
     uint32_t parts = 1;
     while (parts < G && (G % parts || (uint64_t)live * num_kv_heads * parts < 2 * kXcd)) ++parts;
     const uint32_t per_part = G / parts;
+    // A workgroup and the one that shares its compute unit (32 launch positions later in the XCD's list)
+    // step through their units in the same order, so jobs of the same size meet and their phases coincide:
+    // both wait for copies at once, both want the matrix cores at once.  Every second unit of an XCD's list
+    // therefore runs its tiles from the first (fewest keys) to the last, which pairs long jobs with short
+    // ones.  The last two units of a list, and lists too short for the order to matter, keep most-keys-first,
+    // so that the XCD's work does not end on its longest jobs.
+    const uint32_t units_per_xcd = live * num_kv_heads * parts / kXcd; // (rounded down)
     for (uint32_t b : order) {
         const int32_t len = qo_indptr_h[b + 1] - qo_indptr_h[b];
         if (len == 0) continue;
         const int32_t last_q0 = (len - 1) / kBM * kBM;
-        for (uint32_t unit = 0; unit < num_kv_heads * parts; ++unit, ++pair)
-            for (int32_t q0 = last_q0; q0 >= 0; q0 -= kBM)
+        for (uint32_t unit = 0; unit < num_kv_heads * parts; ++unit, ++pair) {
+            const uint32_t nth = pair / kXcd; // the unit's place in its XCD's list
+            const bool ascending = (nth & 1) && units_per_xcd >= 6 && nth + 2 < units_per_xcd;
+            for (int32_t qi = last_q0; qi >= 0; qi -= kBM)
                 for (uint32_t g = 0; g < per_part; ++g)
-                    per_xcd[pair % kXcd].push_back({qo_indptr_h[b], len, q0, (int32_t)(unit * per_part + g), kv_indptr_h[b],
+                    per_xcd[pair % kXcd].push_back({qo_indptr_h[b], len, ascending ? last_q0 - qi : qi,
+                                                    (int32_t)(unit * per_part + g), kv_indptr_h[b],
                                                     kv_indptr_h[b + 1] - kv_indptr_h[b], {0, 0}});
+        }
     }
     size_t longest = 0;
     for (auto& v : per_xcd) longest = std::max(longest, v.size());

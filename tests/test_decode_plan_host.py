@@ -185,12 +185,15 @@ def test_fewer_compute_units_mean_fewer_longer_shares():
     (None, 40, 40),  # config 4: 16 prompts U[128, 4096], 40 heads
     ([512, 300, 2048, 77], 32, 8),  # grouped-query attention with enough units: whole groups stay together
     ([4096], 32, 4),                # ... and with too few: the group of 8 is cut into parts
+    ([700, 300, 300, 1200, 129, 128, 127], 16, 8),  # seven units per column, groups of two
 ])
 def test_prefill_job_list_invariants(lens, Hq, Hkv):
     """The prefill plan (replacement of BatchPrefillRaggedHandler::plan, src/kernel/flashinfer_types.cu:24-49):
     one job per (request, q head, 128-row q tile), each exactly once; the jobs of a (request, kv head) unit
-    sit in one column of the 8-wide launch order (one XCD, consecutive there), last tile first, the q heads
-    of the group side by side; longer requests come first; padding entries have length 0."""
+    sit in one column of the 8-wide launch order (one XCD, consecutive there), the q heads of the group side
+    by side, tiles from the last to the first -- or, for every second unit of a column of six or more units,
+    its last two excepted, from the first to the last; longer requests come first; padding entries have
+    length 0."""
     if lens is None:
         lens = np.random.default_rng(0x5EED).integers(128, 4097, 16)
     lens = np.asarray(lens, np.int64)
@@ -203,7 +206,7 @@ def test_prefill_job_list_invariants(lens, Hq, Hkv):
     # float workspace: the angle table of the q rotation, 512 bytes per position of the longest request
     assert fb == 512 * max(lens) and ib == (len(items) * 32 + 255) // 256 * 256 and len(items) % 8 == 0
     tok0_to_req = {int(indptr[b]): b for b in range(len(lens)) if lens[b] > 0}
-    seen, column, last_q0 = set(), {}, {}
+    seen, column, q0s = set(), {}, {}
     first_seen_len = []
     for i, (tok0, ln, q0, head) in enumerate(items):
         if ln == 0:
@@ -215,24 +218,34 @@ def test_prefill_job_list_invariants(lens, Hq, Hkv):
         seen.add(key)
         pair = (b, int(head))
         assert column.setdefault(pair, i % 8) == i % 8
-        if pair in last_q0:
-            assert q0 == last_q0[pair] - 128  # consecutive in its column, most keys first
-        else:
+        if pair not in q0s:
             first_seen_len.append(int(ln))
-        last_q0[pair] = int(q0)
+        q0s.setdefault(pair, []).append(int(q0))
     want = {(b, hd, q0) for b in range(len(lens)) for hd in range(Hq) for q0 in range(0, int(lens[b]), 128)}
     assert seen == want
-    assert all(v == 0 for v in last_q0.values())
+    # a unit's tiles are consecutive in its column: most keys first, or fewest keys first for the units named above
+    G = Hq // Hkv
+    live = int((lens > 0).sum())
+    parts = next(p for p in range(1, G + 1) if G % p == 0 and (live * Hkv * p >= 16 or p == G))
+    per_part = G // parts
+    units_per_col = live * Hkv * parts // 8
+    nth_in_col, n_ascending = {}, 0
+    for (b, hd), seq in q0s.items():  # (in order of first appearance)
+        unit = (b, hd - hd % per_part)
+        if unit not in nth_in_col:
+            nth_in_col[unit] = sum(1 for u in nth_in_col if column[u] == column[unit])
+        nth = nth_in_col[unit]
+        down = list(range((int(lens[b]) - 1) // 128 * 128, -1, -128))
+        ascending = nth % 2 == 1 and units_per_col >= 6 and nth + 2 < units_per_col
+        assert seq == (down[::-1] if ascending else down)
+        n_ascending += ascending
+    assert (n_ascending > 0) == (units_per_col >= 6)
     # pairs are dealt to the columns in turn, longest requests first: within one column lengths never grow
     for c in range(8):
         col = [int(ln) for (tok0, ln, q0, head) in items[c::8] if ln > 0]
         assert all(a >= b for a, b in zip(col, col[1:]))
     # grouped-query attention: the q heads of a kv head travel together (same column, same tile side by side)
     # unless that would leave fewer than two units per column, in which case the group is cut into equal parts
-    G = Hq // Hkv
-    live = int((lens > 0).sum())
-    parts = next(p for p in range(1, G + 1) if G % p == 0 and (live * Hkv * p >= 16 or p == G))
-    per_part = G // parts
     for (b, hd), c in column.items():
         assert c == column[(b, hd - hd % per_part)]
     # no column holds more than its share of units + 1
