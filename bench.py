@@ -55,8 +55,10 @@ def parse():
                     help="C4: storage type of q, k, v and the output; bf16 runs the second product in f16 with V widened in "
                          "LDS, bf16-head-tail with the probabilities as two bf16 operands (any range of V)")
     ap.add_argument("--prefill-lens", default=None,
-                    help="C4: comma-separated prompt lengths instead of the configuration's 16 x U[128, 4096] (diagnostic; "
-                         "the workload name says so)")
+                    help="C4: comma-separated prompt lengths instead of the configuration's 16 x U[128, 4096], `8x1024` for "
+                         "eight of 1024 (diagnostic; the workload name says so)")
+    ap.add_argument("--prefill-heads", default=None,
+                    help="C4: q heads/kv heads instead of the configuration's 40/40, e.g. 32/8 (diagnostic, as above)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also launch a few plain device copies of 1 GiB (reference point for rocprofv3 --pmc byte counters)")
     args = ap.parse_args()
@@ -118,6 +120,8 @@ def measured_traffic(name, args):
     """HBM bytes per launch of the dominant kernel, measured offline with rocprofv3 --pmc (profiles/*.md);
     only reported for the exact workload it was measured on."""
     if args.seed != 0x5EED or args.sigma != 1.0 or args.split_tokens != 2048 or args.page_size:
+        return None
+    if name == "C4" and (args.prefill_lens or args.prefill_heads or args.prefill_dtype != "f16"):
         return None
     try:
         with open(os.path.join(ROOT, "blitz_scale_amd", "measured_traffic.json")) as f:
@@ -430,8 +434,12 @@ def bench_prefill(args):
     rng = np.random.default_rng(args.seed)
     lens = wl.ctx_lens_for(cfg, rng)
     if args.prefill_lens:
-        lens = np.array([int(x) for x in args.prefill_lens.split(",")], dtype=lens.dtype)
+        lens = np.array([int(x.split("x")[-1]) for x in args.prefill_lens.split(",")
+                         for _ in range(int(x.split("x")[0]) if "x" in x else 1)], dtype=lens.dtype)
         B = len(lens)
+    if args.prefill_heads:
+        Hq, Hkv = (int(x) for x in args.prefill_heads.split("/"))
+    diagnostic = bool(args.prefill_lens or args.prefill_heads)
     indptr = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
     N = int(indptr[-1])
     # page table with the reference's len+1 reservation, seeded page placement
@@ -492,8 +500,9 @@ def bench_prefill(args):
         "n_gpus": 1, "steps": steps, "warmup": warmup, "ms_per_step": round(ms_per_step, 6),
         "higher_is_better": False, "scaling": "weak", "vs_baseline": None, "dtype": args.prefill_dtype, "data": "synthetic",
         "config": {"workload": "C4: Llama-2-13B-shaped ragged causal prefill with RoPE + KV page store, one layer per step"
-                               if not args.prefill_lens else
-                               f"C4 heads and flow with prompt lengths {args.prefill_lens} (diagnostic, not the configuration's)",
+                               if not diagnostic else
+                               f"C4's flow with prompt lengths {args.prefill_lens or 'as configured'} and {Hq}/{Hkv} heads "
+                               "(diagnostic, not the configuration's)",
                    "batch": B, "num_qo_heads": Hq, "num_kv_heads": Hkv, "head_dim": D, "page_size": P,
                    "lens": "uniform[128,4096]" if not args.prefill_lens else args.prefill_lens, "tokens": N, "pool_pages": pool_pages, "rope_theta": theta,
                    "q_rotated_by": args.q_rope,
