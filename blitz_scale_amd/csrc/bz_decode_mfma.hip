@@ -859,7 +859,7 @@ struct StepFinishArgs {
     uint32_t page_size, num_qo_heads, num_kv_heads, group, parts;
     int rope;
     float sm_scale_log2;
-    RopeFreqs freqs;
+    alignas(8) RopeFreqs freqs; // (read two at a time)
 };
 
 // Thread layout: 32 lanes per q head, four consecutive output dimensions per lane (16-byte loads of the partial
@@ -887,9 +887,26 @@ template <> __device__ __forceinline__ void store4<float>(float* p, const float*
 
 template <typename QT, typename PT, typename OT, int S, int HB>
 __global__ __launch_bounds__(32 * HB * S) void decode_step_finish_kernel(StepFinishArgs a) {
-    __shared__ float s_cos[64], s_sin[64];
-    const MfmaUnit u = a.units[blockIdx.x];
     const uint32_t t = threadIdx.x, hl = threadIdx.y, sl = threadIdx.z;
+    // Left to the compiler, the kernel's arguments are fetched a few at a time, each where it is first needed and
+    // each with a wait of its own: scalar round trips in a row before the first row is asked for.  The empty asm
+    // below needs a value made of all of them, so they are all asked for here, in one batch; the unit record and the
+    // step counter, whose indices pass through the same asm, make the second batch.
+    uint32_t early = (uint32_t)(uintptr_t)a.q ^ (uint32_t)(uintptr_t)a.k_new ^ (uint32_t)(uintptr_t)a.v_new ^
+                     (uint32_t)(uintptr_t)a.k_data ^ (uint32_t)(uintptr_t)a.v_data ^ (uint32_t)(uintptr_t)a.indices ^
+                     (uint32_t)(uintptr_t)a.units ^ (uint32_t)(uintptr_t)a.steps_ahead ^ (uint32_t)(uintptr_t)a.part_o ^
+                     (uint32_t)(uintptr_t)a.part_lse ^ (uint32_t)(uintptr_t)a.out ^ (uint32_t)(uintptr_t)a.lse ^
+                     (uint32_t)(uintptr_t)a.k_scale ^ (uint32_t)(uintptr_t)a.v_scale;
+    early ^= (uint32_t)a.stride_page ^ (uint32_t)a.stride_n ^ (uint32_t)a.stride_h ^ a.page_size ^ a.num_qo_heads ^
+             a.num_kv_heads ^ a.group ^ a.parts ^ (uint32_t)a.rope ^ __float_as_uint(a.sm_scale_log2);
+    uint32_t unit_i = blockIdx.x, zero = 0;
+    asm("" : "+s"(early), "+s"(unit_i), "+s"(zero));
+    const MfmaUnit u = a.units[unit_i];
+    const int ahead_raw = a.steps_ahead ? a.steps_ahead[zero] : 0;
+    // The angles of the new token's position: lane t of a head works out pairs 2t and 2t + 1, and the lanes of the
+    // head then pass them round (no LDS table, no workgroup barrier).  The two frequencies are asked for here, beside
+    // the unit record, not where they are used.
+    float2 freq2 = *reinterpret_cast<const float2*>(&a.freqs.f[2 * t]);
     const uint32_t g_raw = blockIdx.y * HB + hl;
     const bool head_live = g_raw < a.group;           // a group that is no multiple of HB leaves lanes idle
     const uint32_t g = head_live ? g_raw : a.group - 1;
@@ -903,7 +920,12 @@ __global__ __launch_bounds__(32 * HB * S) void decode_step_finish_kernel(StepFin
     // and the first four partial results of this slice.  (The sequence's length and its place in the page
     // list come with the unit record, from the host table the plan was made from, like the lengths the
     // decode kernel works with.)
-    const int ahead_raw = a.steps_ahead ? *a.steps_ahead : 0;
+    const int seq_len = u.seq_len - max(ahead_raw, 0);
+    // (the page of the newest token is asked for beside the rows, not where it is used: one dependent round trip less
+    // between the unit record and the append -- and by every workgroup, needed or not: a unit's sequence has pages,
+    // and a load under a condition would be waited for on the spot)
+    const bool appends = g_raw == 0 && sl == 0 && u.unit % (int)a.parts == 0; // one head's lanes per (sequence, kv head)
+    const int64_t page = a.indices[u.ip0 + max(seq_len - 1, 0) / (int)a.page_size];
     const QT* qrow = reinterpret_cast<const QT*>(a.q) + ((size_t)b * a.num_qo_heads + hq) * 128;
     const QT* krow = reinterpret_cast<const QT*>(a.k_new) + ((size_t)b * a.num_kv_heads + kvr) * 128;
     const QT* vrow = reinterpret_cast<const QT*>(a.v_new) + ((size_t)b * a.num_kv_heads + kvr) * 128;
@@ -927,13 +949,10 @@ __global__ __launch_bounds__(32 * HB * S) void decode_step_finish_kernel(StepFin
     float li0[NB];
     float4 oi0[NB];
     load_batch(NB * (int)sl, li0, oi0);
+    asm("" : "+v"(freq2.x), "+v"(freq2.y)); // (asked for at the top, kept in their registers: not fetched again where used)
 
-    const int seq_len = u.seq_len - max(ahead_raw, 0);
-    // (the page of the newest token is asked for here, with the loads above, not where it is used: one
-    // dependent round trip less between the unit record and the append)
-    const bool appends = g_raw == 0 && sl == 0 && u.unit % (int)a.parts == 0; // one head's lanes per (sequence, kv head)
-    const int64_t page = appends ? a.indices[u.ip0 + max(seq_len - 1, 0) / (int)a.page_size] : 0;
     OT* orow = reinterpret_cast<OT*>(a.out) + ((size_t)b * a.num_qo_heads + hq) * 128;
+    if (u.seq == INT32_MIN && early == 0x9e3779b9u) return; // (never: the test only keeps `early` in use)
     if (seq_len <= 0) { // no token at present: nothing to append, a zero row
         const OT z[4] = {StoreCvt<OT>::from(0.f), StoreCvt<OT>::from(0.f), StoreCvt<OT>::from(0.f), StoreCvt<OT>::from(0.f)};
         if (sl == 0 && head_live) store4(orow + d0, z);
@@ -949,17 +968,13 @@ __global__ __launch_bounds__(32 * HB * S) void decode_step_finish_kernel(StepFin
 #pragma unroll
         for (int e = 0; e < 4; ++e) { qd[e] = q_own[e]; kd[e] = k_own[e]; }
         if (a.rope) {
-            const uint32_t tid = t + 32 * (hl + HB * sl);
-            for (uint32_t i = tid; i < 64; i += 32 * HB * S) {
-                float sn0, cs0;
-                sincosf((float)pos * a.freqs.f[i], &sn0, &cs0);
-                s_cos[i] = cs0;
-                s_sin[i] = sn0;
-            }
-            __syncthreads();
+            float sn2[2], cs2[2];
+            sincosf((float)pos * freq2.x, &sn2[0], &cs2[0]);
+            sincosf((float)pos * freq2.y, &sn2[1], &cs2[1]);
+            const int src = (int)(i0 >> 1); // the lane of this head that holds pairs i0 and i0 + 1; the next one i0 + 2, i0 + 3
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
-                const float sn = s_sin[i0 + e], cs = s_cos[i0 + e];
+                const float sn = __shfl(sn2[e & 1], src + (e >> 1), 32), cs = __shfl(cs2[e & 1], src + (e >> 1), 32);
                 float xr, yr;
                 rope_pair(upper ? q_par[e] : q_own[e], upper ? q_own[e] : q_par[e], cs, sn, xr, yr);
                 qd[e] = upper ? yr : xr;
