@@ -37,6 +37,14 @@ HIPCC_FLAGS = [
 ]
 
 
+# bz_decode_mfma.hip: the first two pointers of a kernel's argument list arrive in registers with the wave
+# (kernel-argument preload of gfx950), which lets the finishing kernel of the decode step ask for its unit record at
+# once, while its other arguments are still being fetched.  A kernel whose first argument is a struct is unaffected.
+EXTRA_FLAGS = {
+    "bz_decode_mfma.hip": ["-mllvm", "-amdgpu-kernarg-preload-count=4"],
+}
+
+
 def hipcc():
     return os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 
@@ -53,7 +61,8 @@ def build(verbose=True, jobs=8):
             continue
         obj = os.path.join(obj_dir, src.replace(".hip", ".o"))
         objs.append(obj)
-        cmd = [hipcc(), *HIPCC_FLAGS, "-I", os.path.join(ROOT, "include"), "-I", os.path.join(HERE, "cpp", "kernel"),
+        cmd = [hipcc(), *HIPCC_FLAGS, *EXTRA_FLAGS.get(src, []), "-I", os.path.join(ROOT, "include"),
+               "-I", os.path.join(HERE, "cpp", "kernel"),
                "-c", path, "-o", obj]
         if verbose:
             print(" ".join(cmd), flush=True)

@@ -886,23 +886,22 @@ template <> __device__ __forceinline__ void store4<float>(float* p, const float*
 }
 
 template <typename QT, typename PT, typename OT, int S, int HB>
-__global__ __launch_bounds__(32 * HB * S) void decode_step_finish_kernel(StepFinishArgs a) {
+__global__ __launch_bounds__(32 * HB * S) void decode_step_finish_kernel(const MfmaUnit* __restrict__ units_p,
+                                                                         const int32_t* __restrict__ ahead_p, StepFinishArgs a) {
     const uint32_t t = threadIdx.x, hl = threadIdx.y, sl = threadIdx.z;
-    // Left to the compiler, the kernel's arguments are fetched a few at a time, each where it is first needed and
-    // each with a wait of its own: scalar round trips in a row before the first row is asked for.  The empty asm
-    // below needs a value made of all of them, so they are all asked for here, in one batch; the unit record and the
-    // step counter, whose indices pass through the same asm, make the second batch.
-    uint32_t early = (uint32_t)(uintptr_t)a.q ^ (uint32_t)(uintptr_t)a.k_new ^ (uint32_t)(uintptr_t)a.v_new ^
-                     (uint32_t)(uintptr_t)a.k_data ^ (uint32_t)(uintptr_t)a.v_data ^ (uint32_t)(uintptr_t)a.indices ^
-                     (uint32_t)(uintptr_t)a.units ^ (uint32_t)(uintptr_t)a.steps_ahead ^ (uint32_t)(uintptr_t)a.part_o ^
-                     (uint32_t)(uintptr_t)a.part_lse ^ (uint32_t)(uintptr_t)a.out ^ (uint32_t)(uintptr_t)a.lse ^
-                     (uint32_t)(uintptr_t)a.k_scale ^ (uint32_t)(uintptr_t)a.v_scale;
-    early ^= (uint32_t)a.stride_page ^ (uint32_t)a.stride_n ^ (uint32_t)a.stride_h ^ a.page_size ^ a.num_qo_heads ^
-             a.num_kv_heads ^ a.group ^ a.parts ^ (uint32_t)a.rope ^ __float_as_uint(a.sm_scale_log2);
-    uint32_t unit_i = blockIdx.x, zero = 0;
-    asm("" : "+s"(early), "+s"(unit_i), "+s"(zero));
-    const MfmaUnit u = a.units[unit_i];
-    const int ahead_raw = a.steps_ahead ? a.steps_ahead[zero] : 0;
+    // The two pointers in front of the argument block arrive in registers with the wave (kernel-argument preload of
+    // this target; the build asks for it), so the unit record and the step counter are asked for at once, while the
+    // rest of the arguments is still being fetched.  Those, left to the compiler, are fetched a few at a time, each
+    // where it is first needed and each with a wait of its own: scalar round trips in a row before the first row is
+    // asked for.  The empty asm below needs a value made of all of them, so they are all asked for here, in one batch.
+    const MfmaUnit u = units_p[blockIdx.x];
+    // (without a step counter the record's own padding, which is zero, is read in its place: a load under a condition
+    // would be waited for on the spot, before the arguments below are asked for)
+    const int ahead_raw = *(ahead_p ? ahead_p : &units_p[blockIdx.x].pad[0]);
+    asm volatile("" ::"s"(a.q), "s"(a.k_new), "s"(a.v_new), "s"(a.k_data), "s"(a.v_data), "s"(a.indices), "s"(a.part_o),
+                 "s"(a.part_lse), "s"(a.out), "s"(a.lse), "s"(a.k_scale), "s"(a.v_scale), "s"(a.stride_page),
+                 "s"(a.stride_n), "s"(a.stride_h), "s"(a.page_size), "s"(a.num_qo_heads), "s"(a.num_kv_heads),
+                 "s"(a.group), "s"(a.parts), "s"(a.rope), "s"(a.sm_scale_log2));
     // The angles of the new token's position: lane t of a head works out pairs 2t and 2t + 1, and the lanes of the
     // head then pass them round (no LDS table, no workgroup barrier).  The two frequencies are asked for here, beside
     // the unit record, not where they are used.
@@ -952,7 +951,6 @@ __global__ __launch_bounds__(32 * HB * S) void decode_step_finish_kernel(StepFin
     asm("" : "+v"(freq2.x), "+v"(freq2.y)); // (asked for at the top, kept in their registers: not fetched again where used)
 
     OT* orow = reinterpret_cast<OT*>(a.out) + ((size_t)b * a.num_qo_heads + hq) * 128;
-    if (u.seq == INT32_MIN && early == 0x9e3779b9u) return; // (never: the test only keeps `early` in use)
     if (seq_len <= 0) { // no token at present: nothing to append, a zero row
         const OT z[4] = {StoreCvt<OT>::from(0.f), StoreCvt<OT>::from(0.f), StoreCvt<OT>::from(0.f), StoreCvt<OT>::from(0.f)};
         if (sl == 0 && head_live) store4(orow + d0, z);
@@ -1151,20 +1149,20 @@ static int launch_step_finish(const DecodePlan* p, const StepFinishArgs& a, hipS
     const uint32_t G = a.group;
     if (p->mfma_unit_max_count <= 16) { // what large batches produce
         if (G >= 4)
-            hipLaunchKernelGGL((decode_step_finish_kernel<QT, PT, OT, 1, 4>), dim3(p->mfma_units, (G + 3) / 4), dim3(32, 4, 1), 0, s, a);
+            hipLaunchKernelGGL((decode_step_finish_kernel<QT, PT, OT, 1, 4>), dim3(p->mfma_units, (G + 3) / 4), dim3(32, 4, 1), 0, s, a.units, a.steps_ahead, a);
         else if (G >= 2)
-            hipLaunchKernelGGL((decode_step_finish_kernel<QT, PT, OT, 1, 2>), dim3(p->mfma_units, (G + 1) / 2), dim3(32, 2, 1), 0, s, a);
+            hipLaunchKernelGGL((decode_step_finish_kernel<QT, PT, OT, 1, 2>), dim3(p->mfma_units, (G + 1) / 2), dim3(32, 2, 1), 0, s, a.units, a.steps_ahead, a);
         else
-            hipLaunchKernelGGL((decode_step_finish_kernel<QT, PT, OT, 1, 1>), dim3(p->mfma_units, G), dim3(32, 1, 1), 0, s, a);
+            hipLaunchKernelGGL((decode_step_finish_kernel<QT, PT, OT, 1, 1>), dim3(p->mfma_units, G), dim3(32, 1, 1), 0, s, a.units, a.steps_ahead, a);
     } else if (p->mfma_unit_max_count > 32 && p->mfma_unit_max_count <= 64) {
-        hipLaunchKernelGGL((decode_step_finish_kernel<QT, PT, OT, 4, 2>), dim3(p->mfma_units, (G + 1) / 2), dim3(32, 2, 4), 0, s, a);
+        hipLaunchKernelGGL((decode_step_finish_kernel<QT, PT, OT, 4, 2>), dim3(p->mfma_units, (G + 1) / 2), dim3(32, 2, 4), 0, s, a.units, a.steps_ahead, a);
     } else {
         // 17..32 partials (batches of eight sequences or so): eight slices, so one batch of four per slice and a single
         // round of loads, and one head per workgroup -- four waves.  Measured on 32 layers at batch 8: 497 us per step
         // against 505 with two heads per workgroup (eight waves), 527 with four (sixteen), 507 with four slices of two
         // heads.  More than 64 partials (a few very long sequences): the same shape (4 x 32 768 tokens: 90.8 against
         // 91.8 us with two heads).
-        hipLaunchKernelGGL((decode_step_finish_kernel<QT, PT, OT, 8, 1>), dim3(p->mfma_units, G), dim3(32, 1, 8), 0, s, a);
+        hipLaunchKernelGGL((decode_step_finish_kernel<QT, PT, OT, 8, 1>), dim3(p->mfma_units, G), dim3(32, 1, 8), 0, s, a.units, a.steps_ahead, a);
     }
     BZ_LAUNCH_CHECK();
     return 0;

@@ -61,7 +61,7 @@ struct MfmaSlotHead {
 struct MfmaUnit {
     int32_t seq, unit, first_piece, count;
     int32_t ip0, seq_len; // indptr[seq] and the tokens of the sequence, from the host table the plan was made from
-    int32_t pad[2];
+    int32_t pad[2]; // zero (the finishing kernel reads pad[0] where the caller has no step counter)
 };
 
 // Growable array of plain records that does not clear what it hands out (the planner overwrites every
