@@ -37,9 +37,10 @@ HIPCC_FLAGS = [
 ]
 
 
-# bz_decode_mfma.hip: the first two pointers of a kernel's argument list arrive in registers with the wave
-# (kernel-argument preload of gfx950), which lets the finishing kernel of the decode step ask for its unit record at
-# once, while its other arguments are still being fetched.  A kernel whose first argument is a struct is unaffected.
+# bz_decode_mfma.hip: the leading pointers of a kernel's argument list arrive in registers with the wave
+# (kernel-argument preload of gfx950), which lets the decode kernel ask for its slot head, and the finishing kernel
+# of the decode step for its unit record, while the other arguments are still being fetched: one scalar round trip
+# less at the head of each.  A kernel whose first argument is a struct is unaffected.
 EXTRA_FLAGS = {
     "bz_decode_mfma.hip": ["-mllvm", "-amdgpu-kernarg-preload-count=4"],
 }

@@ -176,13 +176,13 @@ constexpr int kInfoChunk = 16; // tile descriptions fetched per round trip (one 
 // index of MFMA step ks, lane group j, element i is d = 64*(ks/2) + 16*j + 8*(ks%2) + i (q follows).
 // NT: K/V loads carry the non-temporal hint (see kNtK16 above); chosen by the planner.
 template <bool BF16, typename OT, bool ROPE_Q, bool KV8, bool NT>
-__global__ __launch_bounds__(64, 2) void decode_mfma_kernel(MfmaDecodeArgs a, const char* __restrict__ q_ptr,
+__global__ __launch_bounds__(64, 2) void decode_mfma_kernel(const MfmaSlotHead* __restrict__ heads, MfmaDecodeArgs a,
+                                                            const char* __restrict__ q_ptr,
                                                             const char* __restrict__ k_data,
                                                             const char* __restrict__ v_data,
                                                             const int32_t* __restrict__ indices,
                                                             const MfmaPiece* __restrict__ pieces,
                                                             const MfmaTile* __restrict__ tiles,
-                                                            const MfmaSlotHead* __restrict__ heads,
                                                             const float* __restrict__ k_scale,
                                                             const float* __restrict__ v_scale) {
     using M = Mma<BF16>;
@@ -215,7 +215,8 @@ __global__ __launch_bounds__(64, 2) void decode_mfma_kernel(MfmaDecodeArgs a, co
     // The slot's head holds its range of tile records and the description of the first tile: after one
     // round trip (head and counter together) only the two page ids stand between the wave and its first
     // K/V loads.
-    const int ahead_raw = a.steps_ahead ? *a.steps_ahead : 0;
+    // (`heads` is the kernel's first argument: with the kernel-argument preload the build asks for it arrives in
+    // registers with the wave, and the slot head is asked for together with the other arguments, not behind them)
     const MfmaSlotHead* __restrict__ head = heads + blockIdx.x;
     const int g_begin = head->begin, g_end = head->end;
     const MfmaSlotHead first = *head;
@@ -234,7 +235,7 @@ __global__ __launch_bounds__(64, 2) void decode_mfma_kernel(MfmaDecodeArgs a, co
     uint32_t early = (uint32_t)first.idx0 ^ (uint32_t)first.idx1 ^ (uint32_t)first.t ^ (uint32_t)first.seq ^ (uint32_t)first.kvh ^
                      (uint32_t)first.flags ^ (uint32_t)first.partial ^ (uint32_t)first.tile_end ^ (uint32_t)first.seq_len ^
                      (uint32_t)first.kv_head ^ (uint32_t)first.piece;
-    early ^= (uint32_t)(uintptr_t)tiles ^ (uint32_t)(uintptr_t)indices ^ (uint32_t)(uintptr_t)pieces ^ (uint32_t)(uintptr_t)k_data ^
+    early ^= (uint32_t)(uintptr_t)a.steps_ahead ^ (uint32_t)(uintptr_t)tiles ^ (uint32_t)(uintptr_t)indices ^ (uint32_t)(uintptr_t)pieces ^ (uint32_t)(uintptr_t)k_data ^
              (uint32_t)(uintptr_t)v_data ^ (uint32_t)(uintptr_t)q_ptr;
     early ^= (uint32_t)a.stride_page ^ (uint32_t)a.stride_n ^ (uint32_t)a.stride_h ^ a.page_size ^ a.num_qo_heads ^ a.group ^
              (uint32_t)a.step_mode;
@@ -242,6 +243,7 @@ __global__ __launch_bounds__(64, 2) void decode_mfma_kernel(MfmaDecodeArgs a, co
     // (g_begin is never negative: the second term only keeps the value above in use)
     if (g_begin >= g_end || (g_begin < 0 && early == 0x9e3779b9u)) return;
     int first_pid0 = indices[first.idx0], first_pid1 = indices[first.idx1];
+    const int ahead_raw = a.steps_ahead ? *a.steps_ahead : 0; // (beside the page ids: the same round trip)
     const int ahead = max(ahead_raw, 0);
 
     // ---- descriptions of kInfoChunk tiles at a time: lane l < kInfoChunk fetches the record of tile base+l, the two
@@ -1074,12 +1076,12 @@ struct DecodeArgs; // general-kernel argument block (bz_decode.hip); only its sc
 template <bool BF16, typename OT, bool ROPE_Q, bool KV8>
 static void launch_mfma_k(const DecodePlan* p, const MfmaDecodeArgs& a, hipStream_t s) {
     if (p->mfma_streaming)
-        hipLaunchKernelGGL((decode_mfma_kernel<BF16, OT, ROPE_Q, KV8, true>), dim3(p->mfma_slots), dim3(64), 0, s, a,
-                           (const char*)a.q, a.k_data, a.v_data, a.indices, a.pieces, a.tiles, a.heads, a.k_scale,
+        hipLaunchKernelGGL((decode_mfma_kernel<BF16, OT, ROPE_Q, KV8, true>), dim3(p->mfma_slots), dim3(64), 0, s, a.heads, a,
+                           (const char*)a.q, a.k_data, a.v_data, a.indices, a.pieces, a.tiles, a.k_scale,
                            a.v_scale);
     else
-        hipLaunchKernelGGL((decode_mfma_kernel<BF16, OT, ROPE_Q, KV8, false>), dim3(p->mfma_slots), dim3(64), 0, s, a,
-                           (const char*)a.q, a.k_data, a.v_data, a.indices, a.pieces, a.tiles, a.heads, a.k_scale,
+        hipLaunchKernelGGL((decode_mfma_kernel<BF16, OT, ROPE_Q, KV8, false>), dim3(p->mfma_slots), dim3(64), 0, s, a.heads, a,
+                           (const char*)a.q, a.k_data, a.v_data, a.indices, a.pieces, a.tiles, a.k_scale,
                            a.v_scale);
 }
 
