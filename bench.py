@@ -292,7 +292,11 @@ def bench_decode(args, name):
         for n in {GN if max(steps, warmup) >= GN else 0, steps % GN, warmup % GN} - {0}:
             graph_of(n)
         replays = steps // GN + (1 if steps % GN else 0)
-        regions = max(5, -(-25 // replays))  # >= 25 graph replays in all, >= 5 timed regions
+        # >= 25 graph replays in all, >= 5 timed regions, >= 2000 timed steps: the first hundred steps or so after the
+        # idle gap in front of the regions (graph construction) run 1-4 % slower while the memory clocks come up, and
+        # that start-up transient should weigh in proportion to a serving loop's steady state, not as a fifth of 25
+        # short regions
+        regions = max(5, -(-25 // replays), -(-2000 // steps))
         done = torch.cuda.Event()
         dev_ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(regions)]
         run_steps(warmup)
@@ -354,6 +358,8 @@ def bench_decode(args, name):
                         "one by one from Python are eager_us_per_step" if not args.no_graph else "eager launches",
         "step_us_per_region": pct(region_us) if region_us is not None else None,
         "step_us_per_region_on_device": pct(device_us) if device_us is not None else None,
+        # (the start-up transient after the idle gap in front of the regions, shown as it is)
+        "step_us_first_regions": [round(float(x) * 1e3, 2) for x in region_us[:6]] if region_us is not None else None,
         "eager_us_per_step": round(eager_ms * 1e3, 3),
         "decode_call_us": pct(dec_ms),
         "decode_kernel_us": pct(kern_ms),
